@@ -1,0 +1,429 @@
+// Expert histogram (continuous_count) and stable counting-sort index construction for the MoE layer.
+//
+// continuous_count: one launch. Every workgroup streams a contiguous chunk of ids with 16-byte loads and
+// counts into an LDS histogram that holds NREP lane-private copies of every bin (address = id*NREP + lane%NREP),
+// so lanes that carry the same id still hit different LDS banks and a skewed distribution costs the same as a
+// uniform one. The copies are folded, the per-workgroup histogram is written to a workspace row, and the
+// workgroup that draws the last ticket sums the rows into the output: no zeroing pass, no atomics on the
+// output, and the result does not depend on arrival order.
+//
+// index construction: three small launches (per-chunk histogram, scan, placement). Chunks are contiguous
+// ranges of slots, so "expert-major, chunk-minor, slot order inside the chunk" is exactly the stable order.
+#include "common.h"
+
+namespace fmahip {
+namespace {
+
+constexpr int kCountThreads = 1024;
+constexpr int kCountUnroll = 4;
+constexpr int kCountLdsWords = 16384;  // 64 KB of bins (all copies)
+constexpr int kTicketWords = 64;       // 256-byte ticket area in front of the partial rows
+
+__host__ __device__ inline uint32_t floor_pow2(uint32_t x) {
+    uint32_t p = 1;
+    while ((p << 1) != 0 && (p << 1) <= x) p <<= 1;
+    return p;
+}
+
+// number of lane-private copies of each bin
+__host__ __device__ inline uint32_t count_nrep(uint32_t E) {
+    uint32_t r = floor_pow2(kCountLdsWords / (E ? E : 1));
+    return r > 64 ? 64 : (r ? r : 1);
+}
+
+struct CountPlan {
+    uint32_t grid;
+    uint64_t chunk;  // ids per workgroup (multiple of the 16-byte vector width)
+};
+
+inline CountPlan plan_count(uint64_t n, int id_bytes, int cus) {
+    const uint64_t vec = 16 / id_bytes;
+    const uint64_t min_ids = (uint64_t)kCountThreads * vec * 2;  // at least two vectors per thread
+    uint64_t grid = (n + min_ids - 1) / min_ids;
+    const uint64_t max_grid = (uint64_t)(cus > 0 ? cus : 256) * 2;
+    if (grid > max_grid) grid = max_grid;
+    if (grid < 1) grid = 1;
+    uint64_t chunk = (n + grid - 1) / grid;
+    chunk = (chunk + vec - 1) / vec * vec;
+    if (chunk == 0) chunk = vec;
+    grid = (n + chunk - 1) / chunk;
+    if (grid < 1) grid = 1;
+    return CountPlan{(uint32_t)grid, chunk};
+}
+
+template <typename id_t>
+__device__ __forceinline__ void count_one(id_t id, uint32_t E, uint32_t nrep_log2, uint32_t rep, uint32_t* bins) {
+    // unsigned compare drops negative ids as well as ids >= E
+    if ((uint64_t)id < (uint64_t)E) {
+        __hip_atomic_fetch_add(&bins[((uint32_t)id << nrep_log2) + rep], 1u, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+}
+
+template <typename id_t>
+__global__ __launch_bounds__(kCountThreads) void continuous_count_kernel(const id_t* __restrict__ ids, uint64_t n,
+                                                                         uint32_t E, uint32_t nrep_log2,
+                                                                         uint64_t chunk, uint32_t* ws,
+                                                                         uint32_t* __restrict__ out) {
+    extern __shared__ uint32_t bins[];
+    __shared__ uint32_t s_is_last;
+
+    constexpr int VEC = 16 / sizeof(id_t);
+    struct alignas(16) IdVec {
+        id_t v[VEC];
+    };
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t nrep = 1u << nrep_log2;
+    const uint32_t rep = tid & (nrep - 1);
+    const uint32_t words = E << nrep_log2;
+    uint32_t* ticket = ws;
+    uint32_t* partials = ws + kTicketWords;
+
+    for (uint32_t i = tid; i < words; i += kCountThreads) bins[i] = 0;
+    __syncthreads();
+
+    const uint64_t lo = (uint64_t)blockIdx.x * chunk;
+    uint64_t hi = lo + chunk;
+    if (hi > n) hi = n;
+    if (lo < hi) {
+        const uint64_t len = hi - lo;
+        const uint64_t nvec = len / VEC;
+        const IdVec* vp = reinterpret_cast<const IdVec*>(ids + lo);
+        uint64_t v = tid;
+        // main loop: kCountUnroll independent 16-byte loads in flight per lane
+        for (; v + (uint64_t)(kCountUnroll - 1) * kCountThreads < nvec; v += (uint64_t)kCountUnroll * kCountThreads) {
+            IdVec r[kCountUnroll];
+#pragma unroll
+            for (int u = 0; u < kCountUnroll; ++u) r[u] = vp[v + (uint64_t)u * kCountThreads];
+#pragma unroll
+            for (int u = 0; u < kCountUnroll; ++u) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) count_one<id_t>(r[u].v[j], E, nrep_log2, rep, bins);
+            }
+        }
+        for (; v < nvec; v += kCountThreads) {
+            IdVec r = vp[v];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) count_one<id_t>(r.v[j], E, nrep_log2, rep, bins);
+        }
+        const uint64_t tail = lo + nvec * VEC + tid;
+        if (tail < hi) count_one<id_t>(ids[tail], E, nrep_log2, rep, bins);
+    }
+    __syncthreads();
+
+    // fold the copies: tpb lanes share one bin, each sums nrep/tpb copies, then a butterfly inside the group
+    uint32_t tpb = floor_pow2(kCountThreads / E ? kCountThreads / E : 1);
+    if (tpb > nrep) tpb = nrep;
+    if (tpb > (uint32_t)kWave) tpb = kWave;
+    const uint32_t bins_per_pass = kCountThreads / tpb;
+    const uint32_t sub = tid & (tpb - 1);
+    uint32_t* my_row = partials + (uint64_t)blockIdx.x * E;
+    for (uint32_t e0 = 0; e0 < E; e0 += bins_per_pass) {
+        const uint32_t e = e0 + tid / tpb;
+        uint32_t s = 0;
+        if (e < E) {
+            for (uint32_t r = sub; r < nrep; r += tpb) s += bins[(e << nrep_log2) + ((r + e) & (nrep - 1))];
+        }
+        for (uint32_t d = tpb >> 1; d > 0; d >>= 1) s += __shfl_xor(s, d, kWave);
+        if (e < E && sub == 0) my_row[e] = s;
+    }
+
+    // ticket: the last workgroup to arrive owns the final sum
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) {
+        const uint32_t t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        s_is_last = (t == gridDim.x - 1) ? 1u : 0u;
+    }
+    __syncthreads();
+    if (!s_is_last) return;
+    __threadfence();
+
+    uint32_t tpb2 = floor_pow2(kCountThreads / E ? kCountThreads / E : 1);
+    if (tpb2 > (uint32_t)kWave) tpb2 = kWave;
+    const uint32_t bpp2 = kCountThreads / tpb2;
+    const uint32_t sub2 = tid & (tpb2 - 1);
+    for (uint32_t e0 = 0; e0 < E; e0 += bpp2) {
+        const uint32_t e = e0 + tid / tpb2;
+        uint32_t s = 0;
+        if (e < E) {
+            for (uint32_t b = sub2; b < gridDim.x; b += tpb2)
+                s += __hip_atomic_load(&partials[(uint64_t)b * E + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        for (uint32_t d = tpb2 >> 1; d > 0; d >>= 1) s += __shfl_xor(s, d, kWave);
+        if (e < E && sub2 == 0) out[e] = s;
+    }
+    if (tid == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---- index construction ---------------------------------------------------------------------
+
+constexpr int kIdxSteps = 8;                  // 64-slot steps per chunk
+constexpr int kIdxChunk = kIdxSteps * kWave;  // 512 slots per wavefront
+constexpr int kIdxWaves = 4;                  // wavefronts (= chunks) per workgroup
+constexpr int kIdxThreads = kIdxWaves * kWave;
+constexpr int kScanThreads = 1024;
+
+template <typename id_t>
+__device__ __forceinline__ int32_t load_id(const id_t* ids, int64_t s, int64_t R, uint32_t E) {
+    if (s >= R) return -1;
+    const id_t v = ids[s];
+    return ((uint64_t)v < (uint64_t)E) ? (int32_t)v : -1;
+}
+
+// hist[c][e] = number of slots of chunk c routed to expert e
+template <typename id_t>
+__global__ __launch_bounds__(kIdxThreads) void index_hist_kernel(const id_t* __restrict__ ids, int64_t R, uint32_t E,
+                                                                 uint32_t nchunks, uint32_t* __restrict__ hist) {
+    extern __shared__ uint32_t lds[];
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x / kWave;
+    uint32_t* h = lds + wave * E;
+    const uint32_t c = blockIdx.x * kIdxWaves + wave;
+    for (uint32_t e = lane; e < E; e += kWave) h[e] = 0;
+    __syncthreads();
+    if (c < nchunks) {
+        const int64_t base = (int64_t)c * kIdxChunk;
+#pragma unroll
+        for (int s = 0; s < kIdxSteps; ++s) {
+            const int32_t id = load_id<id_t>(ids, base + s * kWave + lane, R, E);
+            if (id >= 0) __hip_atomic_fetch_add(&h[id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+    }
+    __syncthreads();
+    if (c < nchunks) {
+        for (uint32_t e = lane; e < E; e += kWave) hist[(uint64_t)c * E + e] = h[e];
+    }
+}
+
+// counts, inclusive offsets, and hist[c][e] <- first output position of chunk c's slots of expert e
+__global__ __launch_bounds__(kScanThreads) void index_scan_kernel(uint32_t E, uint32_t nchunks, uint32_t* hist,
+                                                                  uint32_t* __restrict__ counts,
+                                                                  uint32_t* __restrict__ offsets) {
+    __shared__ uint32_t s_seg[kScanThreads];  // [part][e]
+    __shared__ uint32_t s_start[FMA_MAX_GROUPS];
+    __shared__ uint32_t s_wave_tot[kScanThreads / kWave];
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t parts = kScanThreads / E;  // E <= 1024 so parts >= 1
+    const uint32_t e = tid % E;
+    const uint32_t part = tid / E;
+    const bool active = part < parts;
+    const uint32_t seg = (nchunks + parts - 1) / parts;
+    const uint32_t c_lo = part * seg;
+    uint32_t c_hi = c_lo + seg;
+    if (c_hi > nchunks) c_hi = nchunks;
+
+    uint32_t s = 0;
+    if (active) {
+        for (uint32_t c = c_lo; c < c_hi; ++c) s += hist[(uint64_t)c * E + e];
+        s_seg[part * E + e] = s;
+    }
+    __syncthreads();
+
+    // per-expert totals and exclusive prefix over the segments (thread e < E walks its column)
+    uint32_t total = 0;
+    if (tid < E) {
+        for (uint32_t p = 0; p < parts; ++p) {
+            const uint32_t v = s_seg[p * E + tid];
+            s_seg[p * E + tid] = total;
+            total += v;
+        }
+    }
+    // block-wide inclusive scan of the totals over experts
+    uint32_t incl = wave_inclusive_scan<uint32_t>(tid < E ? total : 0u);
+    if ((tid & (kWave - 1)) == kWave - 1) s_wave_tot[tid / kWave] = incl;
+    __syncthreads();
+    if (tid < kWave) {
+        const uint32_t nw = kScanThreads / kWave;
+        uint32_t w = tid < nw ? s_wave_tot[tid] : 0u;
+        w = wave_inclusive_scan<uint32_t>(w);
+        if (tid < nw) s_wave_tot[tid] = w;
+    }
+    __syncthreads();
+    if (tid >= kWave) incl += s_wave_tot[tid / kWave - 1];
+    if (tid < E) {
+        counts[tid] = total;
+        offsets[tid] = incl;
+        s_start[tid] = incl - total;
+    }
+    __syncthreads();
+
+    if (active) {
+        uint32_t running = s_start[e] + s_seg[part * E + e];
+        for (uint32_t c = c_lo; c < c_hi; ++c) {
+            const uint64_t i = (uint64_t)c * E + e;
+            const uint32_t v = hist[i];
+            hist[i] = running;
+            running += v;
+        }
+    }
+}
+
+// One wavefront per chunk walks its slots in order; lanes with the same expert id find each other with
+// ballots, the lowest of them advances the expert's cursor, each takes cursor + its rank in the group.
+template <typename id_t>
+__global__ __launch_bounds__(kIdxThreads) void index_place_kernel(const id_t* __restrict__ ids, int64_t R, uint32_t E,
+                                                                  uint32_t nbits, uint32_t nchunks,
+                                                                  const uint32_t* __restrict__ base,
+                                                                  int32_t* __restrict__ perm, int32_t* __restrict__ eid,
+                                                                  int32_t* __restrict__ inv) {
+    extern __shared__ uint32_t lds[];
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x / kWave;
+    uint32_t* cur = lds + wave * E;
+    const uint32_t c = blockIdx.x * kIdxWaves + wave;
+    const bool live = c < nchunks;
+    if (live) {
+        for (uint32_t e = lane; e < E; e += kWave) cur[e] = base[(uint64_t)c * E + e];
+    }
+    __syncthreads();
+    if (!live) return;
+
+    const int64_t first = (int64_t)c * kIdxChunk;
+    int32_t id[kIdxSteps];
+#pragma unroll
+    for (int s = 0; s < kIdxSteps; ++s) id[s] = load_id<id_t>(ids, first + s * kWave + lane, R, E);
+
+    const uint64_t below = (1ull << lane) - 1ull;
+#pragma unroll
+    for (int s = 0; s < kIdxSteps; ++s) {
+        const bool valid = id[s] >= 0;
+        uint64_t mask = __ballot(valid);
+        for (uint32_t b = 0; b < nbits; ++b) {
+            const bool bit = (id[s] >> b) & 1;
+            const uint64_t bal = __ballot(bit);
+            mask &= bit ? bal : ~bal;
+        }
+        if (valid) {
+            const uint32_t rank = __popcll(mask & below);
+            const uint32_t old = cur[id[s]];
+            if (rank == 0) cur[id[s]] = old + (uint32_t)__popcll(mask);
+            const int32_t pos = (int32_t)(old + rank);
+            const int64_t slot = first + s * kWave + lane;
+            perm[pos] = (int32_t)slot;
+            eid[pos] = id[s];
+            inv[slot] = pos;
+        }
+    }
+}
+
+inline uint32_t index_nchunks(int64_t R) { return (uint32_t)((R + kIdxChunk - 1) / kIdxChunk); }
+
+}  // namespace
+}  // namespace fmahip
+
+extern "C" {
+
+int64_t fma_continuous_count_workspace_bytes(int64_t n, int64_t E) {
+    if (n < 0 || E < 1) return 0;
+    // independent of id width and device: sized for the largest grid any call may use
+    const int cus = fmahip::num_compute_units();
+    const int64_t max_grid = (int64_t)(cus > 0 ? cus : 256) * 2;
+    return (int64_t)fmahip::kTicketWords * 4 + max_grid * E * 4;
+}
+
+int fma_continuous_count(const void* ids, int id_bytes, int64_t n, uint32_t* counts, int64_t E, void* workspace,
+                         int64_t workspace_bytes, void* stream) {
+    using namespace fmahip;
+    FMA_REQUIRE(id_bytes == 4 || id_bytes == 8, FMA_ERR_BAD_DTYPE,
+                "continuous_count: ids must be int32 or int64 (id_bytes=%d)", id_bytes);
+    FMA_REQUIRE(E >= 1, FMA_ERR_BAD_SIZE, "continuous_count: E must be >= 1 (got %lld)", (long long)E);
+    FMA_REQUIRE(E <= FMA_MAX_COUNT_BINS, FMA_ERR_TOO_MANY_EXPERTS, "continuous_count: E=%lld exceeds the limit %d",
+                (long long)E, FMA_MAX_COUNT_BINS);
+    FMA_REQUIRE(n >= 0, FMA_ERR_BAD_SIZE, "continuous_count: negative element count %lld", (long long)n);
+    FMA_REQUIRE((uint64_t)n <= 0xffffffffull, FMA_ERR_TOO_MANY_ELEMENTS,
+                "continuous_count: n=%lld exceeds 2^32-1", (long long)n);
+    FMA_REQUIRE(counts != nullptr, FMA_ERR_NULL_POINTER, "continuous_count: counts is NULL");
+    FMA_REQUIRE(ids != nullptr || n == 0, FMA_ERR_NULL_POINTER, "continuous_count: ids is NULL");
+    FMA_REQUIRE(workspace != nullptr, FMA_ERR_NULL_POINTER, "continuous_count: workspace is NULL");
+    FMA_REQUIRE(aligned16(ids), FMA_ERR_MISALIGNED, "continuous_count: ids must be 16-byte aligned");
+    FMA_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 3u) == 0, FMA_ERR_MISALIGNED,
+                "continuous_count: workspace must be 4-byte aligned");
+
+    const int cus = num_compute_units();
+    const CountPlan plan = plan_count((uint64_t)n, id_bytes, cus);
+    const int64_t need = (int64_t)kTicketWords * 4 + (int64_t)plan.grid * E * 4;
+    FMA_REQUIRE(workspace_bytes >= need, FMA_ERR_WORKSPACE_TOO_SMALL,
+                "continuous_count: workspace of %lld bytes is smaller than the %lld needed", (long long)workspace_bytes,
+                (long long)need);
+
+    const uint32_t nrep = count_nrep((uint32_t)E);
+    uint32_t nrep_log2 = 0;
+    while ((1u << nrep_log2) < nrep) ++nrep_log2;
+    const size_t lds_bytes = (size_t)E * nrep * 4;
+    hipStream_t st = (hipStream_t)stream;
+    if (id_bytes == 4) {
+        hipLaunchKernelGGL(continuous_count_kernel<int32_t>, dim3(plan.grid), dim3(kCountThreads), lds_bytes, st,
+                           (const int32_t*)ids, (uint64_t)n, (uint32_t)E, nrep_log2, plan.chunk, (uint32_t*)workspace,
+                           counts);
+    } else {
+        hipLaunchKernelGGL(continuous_count_kernel<int64_t>, dim3(plan.grid), dim3(kCountThreads), lds_bytes, st,
+                           (const int64_t*)ids, (uint64_t)n, (uint32_t)E, nrep_log2, plan.chunk, (uint32_t*)workspace,
+                           counts);
+    }
+    return launch_status("continuous_count");
+}
+
+int64_t fma_moe_build_index_workspace_bytes(int64_t R, int64_t E) {
+    if (R < 0 || E < 1) return 0;
+    const int64_t nchunks = fmahip::index_nchunks(R);
+    return (nchunks > 0 ? nchunks : 1) * E * 4;
+}
+
+int fma_moe_build_index(const void* ids, int id_bytes, int64_t R, int64_t E, uint32_t* counts, uint32_t* offsets,
+                        int32_t* perm, int32_t* eid, int32_t* inv, void* workspace, int64_t workspace_bytes,
+                        void* stream) {
+    using namespace fmahip;
+    FMA_REQUIRE(id_bytes == 4 || id_bytes == 8, FMA_ERR_BAD_DTYPE,
+                "moe_build_index: ids must be int32 or int64 (id_bytes=%d)", id_bytes);
+    FMA_REQUIRE(E >= 1, FMA_ERR_BAD_SIZE, "moe_build_index: E must be >= 1 (got %lld)", (long long)E);
+    FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "moe_build_index: E=%lld exceeds the limit %d",
+                (long long)E, FMA_MAX_GROUPS);
+    FMA_REQUIRE(R >= 0, FMA_ERR_BAD_SIZE, "moe_build_index: negative slot count %lld", (long long)R);
+    FMA_REQUIRE(R <= 0x7fffffffll, FMA_ERR_TOO_MANY_ELEMENTS, "moe_build_index: R=%lld exceeds 2^31-1", (long long)R);
+    FMA_REQUIRE(counts && offsets, FMA_ERR_NULL_POINTER, "moe_build_index: counts/offsets is NULL");
+    FMA_REQUIRE(R == 0 || (ids && perm && eid && inv), FMA_ERR_NULL_POINTER,
+                "moe_build_index: ids/perm/eid/inv is NULL");
+    FMA_REQUIRE(workspace != nullptr, FMA_ERR_NULL_POINTER, "moe_build_index: workspace is NULL");
+    const int64_t need = fma_moe_build_index_workspace_bytes(R, E);
+    FMA_REQUIRE(workspace_bytes >= need, FMA_ERR_WORKSPACE_TOO_SMALL,
+                "moe_build_index: workspace of %lld bytes is smaller than the %lld needed", (long long)workspace_bytes,
+                (long long)need);
+
+    hipStream_t st = (hipStream_t)stream;
+    const uint32_t nchunks = index_nchunks(R);
+    uint32_t* hist = (uint32_t*)workspace;
+    const uint32_t blocks = (nchunks + kIdxWaves - 1) / kIdxWaves;
+    const size_t lds_bytes = (size_t)kIdxWaves * E * 4;
+    uint32_t nbits = 0;
+    while ((1ll << nbits) < E) ++nbits;
+
+    if (nchunks > 0) {
+        if (id_bytes == 4)
+            hipLaunchKernelGGL(index_hist_kernel<int32_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
+                               (const int32_t*)ids, R, (uint32_t)E, nchunks, hist);
+        else
+            hipLaunchKernelGGL(index_hist_kernel<int64_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
+                               (const int64_t*)ids, R, (uint32_t)E, nchunks, hist);
+        int rc = launch_status("moe_build_index(hist)");
+        if (rc) return rc;
+    }
+    hipLaunchKernelGGL(index_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, (uint32_t)E, nchunks, hist, counts,
+                       offsets);
+    int rc = launch_status("moe_build_index(scan)");
+    if (rc) return rc;
+    if (nchunks > 0) {
+        if (id_bytes == 4)
+            hipLaunchKernelGGL(index_place_kernel<int32_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
+                               (const int32_t*)ids, R, (uint32_t)E, nbits, nchunks, hist, perm, eid, inv);
+        else
+            hipLaunchKernelGGL(index_place_kernel<int64_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
+                               (const int64_t*)ids, R, (uint32_t)E, nbits, nchunks, hist, perm, eid, inv);
+        rc = launch_status("moe_build_index(place)");
+    }
+    return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,207 @@
+// Row gather, router-weighted combine and the combine's backward: HBM-bound kernels that move whole rows of H
+// elements with 16-byte lanes. One wavefront reads/writes 1 KB of a row per instruction, so every access is a
+// full-line burst no matter how the row indices are scattered.
+#include "common.h"
+
+namespace fmahip {
+namespace {
+
+constexpr int kRowThreads = 256;
+constexpr int kGatherRows = 4;  // rows per workgroup in the gather
+
+// out[i] = x[idx[i] / divisor], rows of `vecs` 16-byte vectors
+__global__ __launch_bounds__(kRowThreads) void gather_rows_kernel(const uint4* __restrict__ x,
+                                                                  const int32_t* __restrict__ idx, int64_t R,
+                                                                  int64_t vecs, int32_t divisor,
+                                                                  uint4* __restrict__ out) {
+    const int64_t i0 = (int64_t)blockIdx.x * kGatherRows;
+    const uint4* src[kGatherRows];
+#pragma unroll
+    for (int r = 0; r < kGatherRows; ++r) {
+        const int64_t i = i0 + r < R ? i0 + r : R - 1;
+        src[r] = x + (int64_t)(idx[i] / divisor) * vecs;
+    }
+    for (int64_t v = threadIdx.x; v < vecs; v += kRowThreads) {
+        uint4 t[kGatherRows];
+#pragma unroll
+        for (int r = 0; r < kGatherRows; ++r) t[r] = src[r][v];
+#pragma unroll
+        for (int r = 0; r < kGatherRows; ++r) {
+            if (i0 + r < R) out[(i0 + r) * vecs + v] = t[r];
+        }
+    }
+}
+
+// y[t] = sum_j gates[t,j] * o[inv[t,j]]; one workgroup per token, fp32 accumulation in ascending j
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void combine_kernel(const Vec16<T>* __restrict__ o,
+                                                              const int32_t* __restrict__ inv,
+                                                              const T* __restrict__ gates, int64_t k, int64_t vecs,
+                                                              Vec16<T>* __restrict__ y) {
+    constexpr int N = Vec16<T>::N;
+    const int64_t t = blockIdx.x;
+    const int32_t* my_inv = inv + t * k;
+    const T* my_gates = gates ? gates + t * k : nullptr;
+    for (int64_t v = threadIdx.x; v < vecs; v += kRowThreads) {
+        float acc[N];
+#pragma unroll
+        for (int c = 0; c < N; ++c) acc[c] = 0.0f;
+        int64_t j = 0;
+        for (; j + 4 <= k; j += 4) {
+            Vec16<T> r[4];
+            float g[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                r[u] = o[(int64_t)my_inv[j + u] * vecs + v];
+                g[u] = my_gates ? Num<T>::up(my_gates[j + u]) : 1.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                for (int c = 0; c < N; ++c) acc[c] = fmaf(g[u], Num<T>::up(r[u].v[c]), acc[c]);
+            }
+        }
+        for (; j < k; ++j) {
+            const Vec16<T> r = o[(int64_t)my_inv[j] * vecs + v];
+            const float g = my_gates ? Num<T>::up(my_gates[j]) : 1.0f;
+#pragma unroll
+            for (int c = 0; c < N; ++c) acc[c] = fmaf(g, Num<T>::up(r.v[c]), acc[c]);
+        }
+        Vec16<T> w;
+#pragma unroll
+        for (int c = 0; c < N; ++c) w.v[c] = Num<T>::down(acc[c]);
+        y[t * vecs + v] = w;
+    }
+}
+
+// d_o[inv[t,j]] = gates[t,j] * dy[t];  d_gates[t,j] = <dy[t], o[inv[t,j]]>
+template <typename T>
+__global__ __launch_bounds__(kRowThreads) void combine_bwd_kernel(const Vec16<T>* __restrict__ dy,
+                                                                  const Vec16<T>* __restrict__ o,
+                                                                  const int32_t* __restrict__ inv,
+                                                                  const T* __restrict__ gates, int64_t k, int64_t vecs,
+                                                                  Vec16<T>* __restrict__ d_o, T* __restrict__ d_gates) {
+    constexpr int N = Vec16<T>::N;
+    constexpr int NW = kRowThreads / kWave;
+    __shared__ float s_part[NW];
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    for (int64_t j = 0; j < k; ++j) {
+        const int64_t row = inv[t * k + j];
+        const float g = gates ? Num<T>::up(gates[t * k + j]) : 1.0f;
+        float dot = 0.0f;
+        for (int64_t v = threadIdx.x; v < vecs; v += kRowThreads) {
+            const Vec16<T> d = dy[t * vecs + v];
+            Vec16<T> w;
+            if (d_gates) {
+                const Vec16<T> ov = o[row * vecs + v];
+#pragma unroll
+                for (int c = 0; c < N; ++c) dot = fmaf(Num<T>::up(d.v[c]), Num<T>::up(ov.v[c]), dot);
+            }
+#pragma unroll
+            for (int c = 0; c < N; ++c) w.v[c] = Num<T>::down(g * Num<T>::up(d.v[c]));
+            d_o[row * vecs + v] = w;
+        }
+        if (d_gates) {
+            dot = wave_sum(dot);
+            if (lane == 0) s_part[wave] = dot;
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                float s = 0.0f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) s += s_part[w];
+                d_gates[t * k + j] = Num<T>::down(s);
+            }
+            __syncthreads();
+        }
+    }
+}
+
+template <typename T>
+int launch_combine(const void* o, const int32_t* inv, const void* gates, int64_t T_, int64_t k, int64_t H, void* y,
+                   hipStream_t st) {
+    const int64_t vecs = H / Vec16<T>::N;
+    hipLaunchKernelGGL(combine_kernel<T>, dim3((uint32_t)T_), dim3(kRowThreads), 0, st, (const Vec16<T>*)o, inv,
+                       (const T*)gates, k, vecs, (Vec16<T>*)y);
+    return launch_status("combine");
+}
+
+template <typename T>
+int launch_combine_bwd(const void* dy, const void* o, const int32_t* inv, const void* gates, int64_t T_, int64_t k,
+                       int64_t H, void* d_o, void* d_gates, hipStream_t st) {
+    const int64_t vecs = H / Vec16<T>::N;
+    hipLaunchKernelGGL(combine_bwd_kernel<T>, dim3((uint32_t)T_), dim3(kRowThreads), 0, st, (const Vec16<T>*)dy,
+                       (const Vec16<T>*)o, inv, (const T*)gates, k, vecs, (Vec16<T>*)d_o, (T*)d_gates);
+    return launch_status("combine_bwd");
+}
+
+int check_rows(const char* who, int dtype, int64_t H) {
+    const int eb = dtype_bytes(dtype);
+    FMA_REQUIRE(eb != 0, FMA_ERR_BAD_DTYPE, "%s: unknown dtype code %d", who, dtype);
+    FMA_REQUIRE(H > 0 && (H * eb) % 16 == 0, FMA_ERR_BAD_SIZE, "%s: row of %lld elements is not a multiple of 16 bytes",
+                who, (long long)H);
+    return FMA_OK;
+}
+
+}  // namespace
+}  // namespace fmahip
+
+extern "C" {
+
+int fma_gather_rows(const void* x, const int32_t* idx, int64_t R, int64_t H, int32_t divisor, void* out, int dtype,
+                    void* stream) {
+    using namespace fmahip;
+    int rc = check_rows("gather_rows", dtype, H);
+    if (rc) return rc;
+    FMA_REQUIRE(R >= 0 && R <= 0x7fffffffll, FMA_ERR_BAD_SIZE, "gather_rows: bad row count %lld", (long long)R);
+    FMA_REQUIRE(divisor >= 1, FMA_ERR_BAD_SIZE, "gather_rows: divisor must be >= 1 (got %d)", divisor);
+    if (R == 0) return FMA_OK;
+    FMA_REQUIRE(x && idx && out, FMA_ERR_NULL_POINTER, "gather_rows: NULL pointer");
+    FMA_REQUIRE(aligned16(x) && aligned16(out), FMA_ERR_MISALIGNED, "gather_rows: x/out must be 16-byte aligned");
+    const int64_t vecs = H * dtype_bytes(dtype) / 16;
+    const uint32_t blocks = (uint32_t)((R + kGatherRows - 1) / kGatherRows);
+    hipLaunchKernelGGL(gather_rows_kernel, dim3(blocks), dim3(kRowThreads), 0, (hipStream_t)stream, (const uint4*)x,
+                       idx, R, vecs, divisor, (uint4*)out);
+    return launch_status("gather_rows");
+}
+
+int fma_combine(const void* o, const int32_t* inv, const void* gates, int64_t T, int64_t k, int64_t H, void* y,
+                int dtype, void* stream) {
+    using namespace fmahip;
+    int rc = check_rows("combine", dtype, H);
+    if (rc) return rc;
+    FMA_REQUIRE(T >= 0 && T <= 0x7fffffffll, FMA_ERR_BAD_SIZE, "combine: bad token count %lld", (long long)T);
+    FMA_REQUIRE(k >= 1 && T * k <= 0x7fffffffll, FMA_ERR_BAD_SIZE, "combine: bad top_k %lld", (long long)k);
+    if (T == 0) return FMA_OK;
+    FMA_REQUIRE(o && inv && y, FMA_ERR_NULL_POINTER, "combine: NULL pointer");
+    FMA_REQUIRE(aligned16(o) && aligned16(y), FMA_ERR_MISALIGNED, "combine: o/y must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case FMA_F32: return launch_combine<float>(o, inv, gates, T, k, H, y, st);
+        case FMA_F16: return launch_combine<f16_t>(o, inv, gates, T, k, H, y, st);
+        default: return launch_combine<bf16_t>(o, inv, gates, T, k, H, y, st);
+    }
+}
+
+int fma_combine_bwd(const void* dy, const void* o, const int32_t* inv, const void* gates, int64_t T, int64_t k,
+                    int64_t H, void* d_o, void* d_gates, int dtype, void* stream) {
+    using namespace fmahip;
+    int rc = check_rows("combine_bwd", dtype, H);
+    if (rc) return rc;
+    FMA_REQUIRE(T >= 0 && T <= 0x7fffffffll, FMA_ERR_BAD_SIZE, "combine_bwd: bad token count %lld", (long long)T);
+    FMA_REQUIRE(k >= 1 && T * k <= 0x7fffffffll, FMA_ERR_BAD_SIZE, "combine_bwd: bad top_k %lld", (long long)k);
+    if (T == 0) return FMA_OK;
+    FMA_REQUIRE(dy && inv && d_o, FMA_ERR_NULL_POINTER, "combine_bwd: NULL pointer");
+    FMA_REQUIRE(o || !d_gates, FMA_ERR_NULL_POINTER, "combine_bwd: d_gates requested but o is NULL");
+    FMA_REQUIRE(aligned16(dy) && aligned16(d_o) && aligned16(o), FMA_ERR_MISALIGNED,
+                "combine_bwd: dy/o/d_o must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case FMA_F32: return launch_combine_bwd<float>(dy, o, inv, gates, T, k, H, d_o, d_gates, st);
+        case FMA_F16: return launch_combine_bwd<f16_t>(dy, o, inv, gates, T, k, H, d_o, d_gates, st);
+        default: return launch_combine_bwd<bf16_t>(dy, o, inv, gates, T, k, H, d_o, d_gates, st);
+    }
+}
+
+}  // extern "C"

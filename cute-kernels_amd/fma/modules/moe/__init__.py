@@ -1,0 +1,187 @@
+"""Mixture-of-Experts layer: the reference's `Experts` and `MoE` modules (fma/modules/moe/__init__.py:17-298) with the
+expert computation done by the HIP kernels of libfma_hip.so.
+
+Parameter and buffer names and shapes are the reference's (`gate.weight [E, H]`, `c_fc.weight [E, 2I or I, H]`,
+`c_proj.weight [E, H, I]`, uint32 buffers `N_array` / `K_array`), so its state_dicts load unchanged.
+"""
+
+from typing import Callable
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from ...kernel_backend import KernelBackend, is_hip_kernel_backend
+from ...ops.swiglu import swiglu_packed
+from .cuda_implementation import (
+    build_routing_index,
+    combine,
+    gather_rows,
+    grouped_gemm_experts,
+    up_projection_swiglu_experts,
+)
+
+
+class Experts(nn.Module):
+    def __init__(
+        self, num_experts: int, in_features: int, out_features: int, add_bias: bool = True, std: float | None = None
+    ) -> None:
+        super().__init__()
+
+        self.weight = nn.Parameter(torch.empty(num_experts, out_features, in_features))
+
+        self.bias = None
+        if add_bias:
+            self.bias = nn.Parameter(torch.empty(num_experts, out_features))
+
+        self.std = std
+
+        self.num_experts = num_experts
+        self.in_features = in_features
+        self.out_features = out_features
+
+        self.register_buffer("N_array", torch.empty((num_experts,), dtype=torch.uint32))
+        self.register_buffer("K_array", torch.empty((num_experts,), dtype=torch.uint32))
+
+        self.reset_parameters()
+
+    def cuda_forward(self, input: torch.Tensor, expert_frequency: torch.Tensor) -> torch.Tensor:
+        # like the reference's cuda_forward (fma/modules/moe/__init__.py:89-92) the grouped GEMM has no bias term
+        assert self.bias is None, "the grouped-GEMM experts do not implement a bias"
+        return grouped_gemm_experts(
+            x=input, weight=self.weight, M_array=expert_frequency, N_array=self.N_array, K_array=self.K_array
+        )
+
+    def cuda_forward_swiglu(self, input: torch.Tensor, expert_frequency: torch.Tensor) -> torch.Tensor:
+        """up-projection with swiglu_packed fused into the GEMM epilogue: returns [sum(M), out_features / 2]"""
+        assert self.bias is None, "the grouped-GEMM experts do not implement a bias"
+        return up_projection_swiglu_experts(
+            x=input, weight=self.weight, M_array=expert_frequency, N_array=self.N_array, K_array=self.K_array
+        )
+
+    def extra_repr(self):
+        return "num_experts={}, in_features={}, out_features={}".format(
+            self.num_experts, self.in_features, self.out_features
+        )
+
+    @torch.no_grad()
+    def reset_parameters(self) -> None:
+        nn.init.normal_(self.weight, mean=0, std=self.std)
+        if hasattr(self, "bias") and self.bias is not None:
+            self.bias.zero_()
+
+        self.N_array.fill_(self.out_features)
+        self.K_array.fill_(self.in_features)
+
+
+def _is_swiglu_packed(activation_function: Callable) -> bool:
+    fn = getattr(activation_function, "func", activation_function)  # functools.partial(swiglu_packed, ...)
+    return fn is swiglu_packed
+
+
+class MoE(nn.Module):
+    def __init__(
+        self,
+        num_experts: int,
+        num_experts_per_tok: int,
+        hidden_size: int,
+        intermediate_size: int,
+        activation_function: Callable,
+        is_glu: bool,
+        add_bias: bool,
+        std: float,
+    ) -> None:
+        super().__init__()
+
+        self.num_experts = num_experts
+        self.top_k = num_experts_per_tok
+
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+
+        self.gate = nn.Linear(in_features=self.hidden_size, out_features=num_experts, bias=False)
+
+        self.c_fc = Experts(
+            num_experts=num_experts,
+            in_features=self.hidden_size,
+            out_features=2 * self.intermediate_size if is_glu else self.intermediate_size,
+            add_bias=add_bias,
+            std=std,
+        )
+
+        self.act = activation_function
+        # swiglu_packed as the activation of a GLU layer is computed inside the up-projection's epilogue
+        self.fuse_swiglu = is_glu and _is_swiglu_packed(activation_function)
+
+        self.c_proj = Experts(
+            num_experts=num_experts,
+            in_features=self.intermediate_size,
+            out_features=self.hidden_size,
+            add_bias=add_bias,
+            std=std,
+        )
+
+    def forward(
+        self, hidden_states: torch.Tensor, kernel_backend: KernelBackend = KernelBackend.triton
+    ) -> tuple[torch.Tensor, torch.Tensor]:
+        original_shape = hidden_states.shape
+
+        # hidden_states -> (total_q, hidden_size)
+        hidden_states = hidden_states.view(-1, self.hidden_size)
+        router_logits, router_weights, selected_experts = self._compute_routing_weights(hidden_states)
+
+        # router_logits -> (total_q, num_experts); router_weights, selected_experts -> (total_q, top_k)
+        hidden_states = self._compute_experts(
+            hidden_states, router_weights, selected_experts, kernel_backend=kernel_backend
+        )
+
+        hidden_states = hidden_states.view(original_shape)
+
+        return hidden_states, router_logits
+
+    def _compute_routing_weights(self, hidden_states: torch.Tensor) -> tuple[torch.Tensor]:
+        router_logits = self.gate(hidden_states)
+        router_weights, selected_experts = self._get_topk(router_logits)
+
+        # softmax over the k kept logits, in fp32
+        router_weights = F.softmax(router_weights.float(), dim=-1)
+        router_weights = router_weights.type_as(hidden_states)
+
+        return router_logits, router_weights, selected_experts
+
+    def _compute_experts(
+        self,
+        hidden_states: torch.Tensor,
+        router_weights: torch.Tensor,
+        selected_experts: torch.Tensor,
+        kernel_backend: KernelBackend,
+    ) -> torch.Tensor:
+        if not is_hip_kernel_backend(kernel_backend):
+            raise ValueError(f"unexpected kernel_backend ({kernel_backend})")
+
+        # counts, offsets and the stable expert-major order of the (token, choice) slots, with its inverse
+        expert_frequency, _, sorted_scattered_idxs, _, inverse = build_routing_index(selected_experts, self.num_experts)
+
+        # rows of every expert back to back: x[slot // top_k]
+        hidden_states = gather_rows(hidden_states, sorted_scattered_idxs, inverse, self.top_k)
+
+        if self.fuse_swiglu:
+            hidden_states = self.c_fc.cuda_forward_swiglu(input=hidden_states, expert_frequency=expert_frequency)
+        else:
+            hidden_states = self.c_fc.cuda_forward(input=hidden_states, expert_frequency=expert_frequency)
+            hidden_states = self.act(hidden_states)
+
+        hidden_states = self.c_proj.cuda_forward(input=hidden_states, expert_frequency=expert_frequency)
+
+        # y[t] = sum_j router_weights[t, j] * expert_output[row of slot (t, j)]
+        hidden_states = combine(hidden_states, router_weights, inverse)
+
+        return hidden_states
+
+    def _get_topk(self, x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+        if self.top_k == 1:
+            x, indices = x.max(dim=-1, keepdim=True)
+        else:
+            x, indices = x.topk(self.top_k, dim=-1)
+
+        return x, indices

@@ -1,0 +1,340 @@
+"""GPU side of the MoE layer: custom ops over libfma_hip.so and the autograd functions built from them.
+
+Stands in for the reference's fma/modules/moe/cuda_implementation/__init__.py (grouped-GEMM experts, group /
+ungroup row movement) and for the row kernels of fma/modules/moe/triton_implementation/. Differences by design:
+ * no padding: the HIP grouped GEMM masks ragged group edges, so rows are packed back to back (the reference pads
+   every group to a multiple of 8 rows for its TMA kernel, cuda_implementation/__init__.py:83-104);
+ * the routed order is built by a stable counting sort (counts -> offsets -> placement) that also yields the
+   inverse permutation, which makes the combine and every backward gather atomic-free and deterministic;
+ * index tensors are int32.
+"""
+
+import torch
+from torch.library import custom_op
+
+from ... import _lib
+from ...constants import LIBRARY_NAME
+from ...ops import grouped_gemm
+from ...utils import ensure_contiguous
+
+
+# ---- custom ops ---------------------------------------------------------------------------------
+
+
+@custom_op(
+    f"{LIBRARY_NAME}::moe_build_index_cuda", mutates_args={"counts", "offsets", "perm", "eid", "inv", "workspace"}
+)
+def moe_build_index_cuda(
+    ids: torch.Tensor,
+    counts: torch.Tensor,
+    offsets: torch.Tensor,
+    perm: torch.Tensor,
+    eid: torch.Tensor,
+    inv: torch.Tensor,
+    workspace: torch.Tensor,
+) -> None:
+    _lib.require_gpu(ids, counts, offsets, perm, eid, inv, workspace)
+    assert ids.dtype in (torch.int32, torch.int64) and ids.is_contiguous()
+    assert counts.dtype == torch.uint32 and offsets.dtype == torch.uint32
+    assert perm.dtype == eid.dtype == inv.dtype == torch.int32
+    R, E = ids.numel(), counts.numel()
+    assert perm.numel() == eid.numel() == inv.numel() == R and offsets.numel() == E
+    with torch.cuda.device(ids.device):
+        rc = _lib.load().fma_moe_build_index(
+            ids.data_ptr(), ids.element_size(), R, E, counts.data_ptr(), offsets.data_ptr(), perm.data_ptr(),
+            eid.data_ptr(), inv.data_ptr(), workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+            _lib.current_stream(ids.device),
+        )
+    _lib.check(rc, "moe_build_index_cuda")
+
+
+@custom_op(f"{LIBRARY_NAME}::gather_rows_cuda", mutates_args={"output"})
+def gather_rows_cuda(x: torch.Tensor, idx: torch.Tensor, divisor: int, output: torch.Tensor) -> None:
+    _lib.require_gpu(x, idx, output)
+    assert x.dim() == 2 and output.dim() == 2 and x.size(1) == output.size(1) and x.dtype == output.dtype
+    assert idx.dtype == torch.int32 and idx.numel() == output.size(0)
+    assert x.is_contiguous() and output.is_contiguous() and idx.is_contiguous()
+    with torch.cuda.device(x.device):
+        rc = _lib.load().fma_gather_rows(
+            x.data_ptr(), idx.data_ptr(), output.size(0), x.size(1), divisor, output.data_ptr(),
+            _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
+        )
+    _lib.check(rc, "gather_rows_cuda")
+
+
+@custom_op(f"{LIBRARY_NAME}::combine_cuda", mutates_args={"output"})
+def combine_cuda(
+    o: torch.Tensor, inv: torch.Tensor, gates: torch.Tensor | None, top_k: int, output: torch.Tensor
+) -> None:
+    _lib.require_gpu(o, inv, gates, output)
+    T, H = output.shape
+    assert o.dim() == 2 and o.size(1) == H and o.dtype == output.dtype
+    assert inv.dtype == torch.int32 and inv.numel() == T * top_k
+    assert gates is None or (gates.dtype == o.dtype and gates.numel() == T * top_k and gates.is_contiguous())
+    assert o.is_contiguous() and output.is_contiguous() and inv.is_contiguous()
+    with torch.cuda.device(o.device):
+        rc = _lib.load().fma_combine(
+            o.data_ptr(), inv.data_ptr(), _lib.ptr(gates), T, top_k, H, output.data_ptr(), _lib.dtype_code(o.dtype),
+            _lib.current_stream(o.device),
+        )
+    _lib.check(rc, "combine_cuda")
+
+
+@custom_op(f"{LIBRARY_NAME}::combine_backward_cuda", mutates_args={"o_grad", "gates_grad"})
+def combine_backward_cuda(
+    output_grad: torch.Tensor,
+    o: torch.Tensor,
+    inv: torch.Tensor,
+    gates: torch.Tensor | None,
+    top_k: int,
+    o_grad: torch.Tensor,
+    gates_grad: torch.Tensor | None,
+) -> None:
+    _lib.require_gpu(output_grad, o, inv, gates, o_grad, gates_grad)
+    T, H = output_grad.shape
+    assert o.shape == o_grad.shape and o.size(1) == H
+    assert output_grad.dtype == o.dtype == o_grad.dtype
+    assert inv.dtype == torch.int32 and inv.numel() == T * top_k
+    for t in (output_grad, o, o_grad, inv, gates, gates_grad):
+        assert t is None or t.is_contiguous()
+    assert gates is None or gates.dtype == o.dtype
+    assert gates_grad is None or (gates_grad.dtype == o.dtype and gates_grad.numel() == T * top_k)
+    with torch.cuda.device(o.device):
+        rc = _lib.load().fma_combine_bwd(
+            output_grad.data_ptr(), o.data_ptr(), inv.data_ptr(), _lib.ptr(gates), T, top_k, H, o_grad.data_ptr(),
+            _lib.ptr(gates_grad), _lib.dtype_code(o.dtype), _lib.current_stream(o.device),
+        )
+    _lib.check(rc, "combine_backward_cuda")
+
+
+@custom_op(f"{LIBRARY_NAME}::grouped_gemm_swiglu_cuda", mutates_args={"h", "act"})
+def grouped_gemm_swiglu_cuda(
+    x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, h: torch.Tensor | None, act: torch.Tensor
+) -> None:
+    _lib.require_gpu(x, weight, M_array, h, act)
+    E, N, K = weight.shape
+    assert N % 2 == 0
+    inter = N // 2
+    R = x.size(0)
+    assert x.shape == (R, K) and act.shape == (R, inter) and (h is None or h.shape == (R, N))
+    assert x.dtype == weight.dtype == act.dtype and (h is None or h.dtype == x.dtype)
+    assert M_array.dtype == torch.uint32 and M_array.numel() == E
+    for t in (x, weight, M_array, h, act):
+        assert t is None or t.is_contiguous()
+    with torch.cuda.device(x.device):
+        rc = _lib.load().fma_grouped_gemm_swiglu(
+            x.data_ptr(), weight.data_ptr(), _lib.ptr(h), act.data_ptr(), M_array.data_ptr(), E, inter, K,
+            _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
+        )
+    _lib.check(rc, "grouped_gemm_swiglu_cuda")
+
+
+# ---- index construction -----------------------------------------------------------------------------
+
+
+@torch.no_grad()
+def build_routing_index(
+    selected_experts: torch.Tensor, num_experts: int
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Stable counting sort of the flattened (token, choice) slots by expert.
+
+    Returns (expert_frequency uint32[E], expert_offsets uint32[E] (inclusive), sorted_scattered_idxs int32[R],
+    sorted_expert_idxs int32[R], inverse int32[R]); the first four are what the reference obtains from
+    `selected_experts.flatten().sort()`, continuous_count and cumsum (fma/modules/moe/__init__.py:214-217,249), with
+    the order inside one expert fixed to ascending slot.
+    """
+    ids = selected_experts.reshape(-1).contiguous()
+    device = ids.device
+    R = ids.numel()
+    counts = torch.empty(num_experts, dtype=torch.uint32, device=device)
+    offsets = torch.empty(num_experts, dtype=torch.uint32, device=device)
+    perm = torch.empty(R, dtype=torch.int32, device=device)
+    eid = torch.empty(R, dtype=torch.int32, device=device)
+    inv = torch.empty(R, dtype=torch.int32, device=device)
+    nbytes = _lib.load().fma_moe_build_index_workspace_bytes(R, num_experts)
+    workspace = torch.empty(max(nbytes, 4) // 4, dtype=torch.int32, device=device)
+    moe_build_index_cuda(ids, counts, offsets, perm, eid, inv, workspace)
+    return counts, offsets, perm, eid, inv
+
+
+# ---- autograd functions -----------------------------------------------------------------------------
+
+
+class _GatherRows(torch.autograd.Function):
+    """xg[i] = x[perm[i] // top_k]; backward sums the top_k grouped rows of every token through `inv`."""
+
+    @staticmethod
+    @ensure_contiguous
+    def forward(ctx, x: torch.Tensor, perm: torch.Tensor, inv: torch.Tensor, top_k: int) -> torch.Tensor:
+        assert x.dim() == 2
+        output = torch.empty(perm.numel(), x.size(1), device=x.device, dtype=x.dtype)
+        gather_rows_cuda(x, perm, top_k, output)
+        ctx.save_for_backward(inv)
+        ctx.top_k = top_k
+        ctx.T = x.size(0)
+        return output
+
+    @staticmethod
+    @ensure_contiguous
+    def backward(ctx, output_grad: torch.Tensor) -> tuple[torch.Tensor | None]:
+        (inv,) = ctx.saved_tensors
+        x_grad = torch.empty(ctx.T, output_grad.size(1), device=output_grad.device, dtype=output_grad.dtype)
+        combine_cuda(output_grad, inv, None, ctx.top_k, x_grad)
+        return x_grad, None, None, None
+
+
+class _Combine(torch.autograd.Function):
+    """y[t] = sum_j gates[t, j] * o[inv[t*k + j]]."""
+
+    @staticmethod
+    @ensure_contiguous
+    def forward(ctx, o: torch.Tensor, gates: torch.Tensor, inv: torch.Tensor) -> torch.Tensor:
+        T, top_k = gates.shape
+        output = torch.empty(T, o.size(1), device=o.device, dtype=o.dtype)
+        combine_cuda(o, inv, gates, top_k, output)
+        ctx.save_for_backward(o, gates, inv)
+        return output
+
+    @staticmethod
+    @ensure_contiguous
+    def backward(ctx, output_grad: torch.Tensor) -> tuple[torch.Tensor | None]:
+        o, gates, inv = ctx.saved_tensors
+        o_grad = torch.empty_like(o)
+        gates_grad = torch.empty_like(gates) if ctx.needs_input_grad[1] else None
+        combine_backward_cuda(output_grad, o, inv, gates, gates.size(1), o_grad, gates_grad)
+        return o_grad, gates_grad, None
+
+
+class _GroupedGemmExperts(torch.autograd.Function):
+    """y_e = x_e @ W_e^T per expert; the three GEMMs of the reference's _GroupedGemmExperts
+    (fma/modules/moe/cuda_implementation/__init__.py:15-80)."""
+
+    @staticmethod
+    @ensure_contiguous
+    def forward(
+        ctx, x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor
+    ) -> torch.Tensor:
+        # x -> sum(M) x K, weight -> E x N x K
+        _, N, K = weight.size()
+
+        assert N % 8 == 0
+        assert K % 8 == 0
+
+        output = grouped_gemm(
+            A=x,
+            B=weight,
+            C=None,
+            M_array=M_array,
+            N_array=N_array,
+            K_array=K_array,
+            output_shape=(x.size(0), N),
+            is_A_transposed=False,
+            is_B_transposed=True,
+        )
+
+        ctx.save_for_backward(x, weight, M_array, K_array, N_array)
+
+        return output
+
+    @staticmethod
+    @ensure_contiguous
+    def backward(ctx, output_grad: torch.Tensor) -> tuple[torch.Tensor | None]:
+        x, weight, M_array, K_array, N_array = ctx.saved_tensors
+        x_grad = weight_grad = None
+
+        if ctx.needs_input_grad[0]:
+            # dx_e = dy_e @ W_e : A = dy [sum(M), N], B = W_e stored [N, K] as a [K_gemm = N, N_gemm = K] matrix
+            x_grad = grouped_gemm(
+                A=output_grad,
+                B=weight,
+                C=None,
+                M_array=M_array,
+                N_array=K_array,
+                K_array=N_array,
+                output_shape=x.size(),
+                is_A_transposed=False,
+                is_B_transposed=False,
+            )
+
+        if ctx.needs_input_grad[1]:
+            # dW_e = dy_e^T @ x_e : both operands are stored with the reduction dim (the M_e rows) as row index
+            weight_grad = grouped_gemm(
+                A=output_grad,
+                B=x,
+                C=None,
+                M_array=N_array,
+                N_array=K_array,
+                K_array=M_array,
+                output_shape=weight.size(),
+                is_A_transposed=True,
+                is_B_transposed=False,
+            )
+
+        return x_grad, weight_grad, None, None, None
+
+
+class _UpProjectionSwiglu(torch.autograd.Function):
+    """a_e = swiglu_packed(x_e @ W_e^T) with the activation fused into the GEMM epilogue. The pre-activation h is
+    kept (bf16) for the backward, which is swiglu-backward followed by the two grouped GEMMs."""
+
+    @staticmethod
+    @ensure_contiguous
+    def forward(
+        ctx, x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor
+    ) -> torch.Tensor:
+        _, N, K = weight.size()
+        assert N % 16 == 0
+        assert K % 8 == 0
+        R = x.size(0)
+        needs_backward = any(ctx.needs_input_grad[:2])
+        h = torch.empty(R, N, device=x.device, dtype=x.dtype) if needs_backward else None
+        act = torch.empty(R, N // 2, device=x.device, dtype=x.dtype)
+        grouped_gemm_swiglu_cuda(x, weight, M_array, h, act)
+        if needs_backward:
+            ctx.save_for_backward(x, weight, h, M_array, K_array, N_array)
+        return act
+
+    @staticmethod
+    @ensure_contiguous
+    def backward(ctx, act_grad: torch.Tensor) -> tuple[torch.Tensor | None]:
+        from ...ops.swiglu.cuda_implementation import swiglu_backward_cuda
+
+        x, weight, h, M_array, K_array, N_array = ctx.saved_tensors
+        h_grad = torch.empty_like(h)
+        up, gate = h.chunk(2, dim=-1)
+        up_grad, gate_grad = h_grad.chunk(2, dim=-1)
+        swiglu_backward_cuda(
+            gate=gate, up=up, output_grad=act_grad, gate_grad=gate_grad, up_grad=up_grad, BLOCK_SIZE=1024
+        )
+        x_grad = weight_grad = None
+        if ctx.needs_input_grad[0]:
+            x_grad = grouped_gemm(
+                A=h_grad, B=weight, C=None, M_array=M_array, N_array=K_array, K_array=N_array,
+                output_shape=x.size(), is_A_transposed=False, is_B_transposed=False,
+            )
+        if ctx.needs_input_grad[1]:
+            weight_grad = grouped_gemm(
+                A=h_grad, B=x, C=None, M_array=N_array, N_array=K_array, K_array=M_array,
+                output_shape=weight.size(), is_A_transposed=True, is_B_transposed=False,
+            )
+        return x_grad, weight_grad, None, None, None
+
+
+def gather_rows(x: torch.Tensor, perm: torch.Tensor, inv: torch.Tensor, top_k: int) -> torch.Tensor:
+    return _GatherRows.apply(x, perm, inv, top_k)
+
+
+def combine(o: torch.Tensor, gates: torch.Tensor, inv: torch.Tensor) -> torch.Tensor:
+    return _Combine.apply(o, gates, inv)
+
+
+def grouped_gemm_experts(
+    x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor
+) -> torch.Tensor:
+    return _GroupedGemmExperts.apply(x, weight, M_array, N_array, K_array)
+
+
+def up_projection_swiglu_experts(
+    x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor
+) -> torch.Tensor:
+    return _UpProjectionSwiglu.apply(x, weight, M_array, N_array, K_array)

@@ -1,0 +1,168 @@
+/*
+ * fma_hip.h — C ABI of libfma_hip.so: the MoE-layer hot path of cute-kernels ("fma")
+ * as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer unless its comment says "host".
+ *  - The caller owns every buffer, including workspaces (sizes come from the *_workspace_bytes queries).
+ *    The library allocates nothing and keeps no state besides cached device properties.
+ *  - `stream` is a hipStream_t passed as void* (NULL = the null stream). Calls only enqueue work.
+ *  - Every entry point returns 0 on success, a negative FMA_ERR_* code for a rejected argument
+ *    (nothing is launched then) or a positive hipError_t if the launch itself failed.
+ *    fma_last_error_string() returns the message of the calling thread's last failure.
+ *  - dtype codes: FMA_F32 / FMA_F16 / FMA_BF16. Index tensors produced here are int32.
+ *
+ * Citations name the reference interface each entry point stands in for (paths relative to the
+ * cute-kernels source tree).
+ */
+#ifndef FMA_HIP_H
+#define FMA_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FMA_OK 0
+#define FMA_ERR_NULL_POINTER (-1)
+#define FMA_ERR_BAD_DTYPE (-2)
+#define FMA_ERR_BAD_SIZE (-3)
+#define FMA_ERR_TOO_MANY_EXPERTS (-4)
+#define FMA_ERR_TOO_MANY_ELEMENTS (-5)
+#define FMA_ERR_MISALIGNED (-6)
+#define FMA_ERR_WORKSPACE_TOO_SMALL (-7)
+#define FMA_ERR_UNSUPPORTED (-8)
+
+#define FMA_F32 0
+#define FMA_F16 1
+#define FMA_BF16 2
+
+/* limits (same values as the reference's: continuous_count forward.cu:12, grouped_gemm kernel.cu:38) */
+#define FMA_MAX_COUNT_BINS 16384
+#define FMA_MAX_GROUPS 1024
+
+/* ---- library ---------------------------------------------------------------------------- */
+
+/* Message of the calling thread's most recent failed call ("" if none). Host pointer, valid until the
+ * thread's next failing call. Replaces the TORCH_CHECK / c10::Error text of the reference's pybind
+ * functions (e.g. fma/ops/continuous_count/cuda_implementation/forward.cu:120-128). */
+const char* fma_last_error_string(void);
+
+/* ABI version of this header (bumped on any signature change). */
+int fma_abi_version(void);
+
+/* Number of compute units of the current device (0 if no device). The reference's get_num_SMs
+ * (fma/include/device.h:8-16). */
+int fma_num_compute_units(void);
+
+/* ---- continuous_count ------------------------------------------------------------------- */
+
+/* Bytes of workspace fma_continuous_count needs for n ids and E bins. The first 256 bytes must be zero
+ * before the FIRST call that uses the buffer; every call leaves them zero again, so one buffer zeroed
+ * once can be reused by stream-ordered calls (calls that overlap in time need separate buffers). */
+int64_t fma_continuous_count_workspace_bytes(int64_t n, int64_t E);
+
+/* counts[v] = #{ i < n : ids[i] == v } for v in [0, E); ids outside [0, E) are not counted.
+ * ids: n integers of id_bytes (4 = int32, 8 = int64) each, 16-byte aligned; counts: E uint32, fully
+ * overwritten (no need to zero). E <= FMA_MAX_COUNT_BINS, n <= 2^32-1.
+ * Replaces continuous_count_cuda(x, output, E, THREAD_BLOCK_CLUSTER_SIZE, BLOCK_SIZE)
+ * (fma/ops/continuous_count/cuda_implementation/ops.cpp:13-15, forward.cu:115-167); the two launch-shape
+ * arguments have no meaning on wave64 hardware and are dropped here. */
+int fma_continuous_count(const void* ids, int id_bytes, int64_t n, uint32_t* counts, int64_t E,
+                         void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ---- index construction ------------------------------------------------------------------ */
+
+/* Bytes of workspace fma_moe_build_index needs (no zeroing required). */
+int64_t fma_moe_build_index_workspace_bytes(int64_t R, int64_t E);
+
+/* Stable counting sort of the R routed slots by expert id. With slot s = t*top_k + j:
+ *   counts[e]  = #{ s : ids[s] == e }                       (uint32[E])
+ *   offsets[e] = counts[0] + ... + counts[e]   (inclusive)   (uint32[E])
+ *   perm[i]    = i-th slot in (expert, slot) order           (int32[R])  == sorted_scattered_idxs
+ *   eid[i]     = ids[perm[i]]                                (int32[R])  == sorted_expert_idxs
+ *   inv[s]     = i with perm[i] == s                         (int32[R])
+ * Every id must lie in [0, E); E <= FMA_MAX_GROUPS; R <= 2^31-1.
+ * Replaces `selected_experts.flatten().sort()` + continuous_count + `expert_frequency.cumsum(-1)`
+ * (fma/modules/moe/__init__.py:214-217,249); within one expert the order is ascending slot, i.e. the
+ * order torch.sort(stable=True) defines. */
+int fma_moe_build_index(const void* ids, int id_bytes, int64_t R, int64_t E, uint32_t* counts,
+                        uint32_t* offsets, int32_t* perm, int32_t* eid, int32_t* inv, void* workspace,
+                        int64_t workspace_bytes, void* stream);
+
+/* ---- row movement ------------------------------------------------------------------------- */
+
+/* out[i, :] = x[idx[i] / divisor, :] for i < R (rows of H elements, H*elem_bytes a multiple of 16).
+ * Replaces group_with_padding_triton(..., NEEDS_DUPLICATION=True) without padding
+ * (fma/modules/moe/cuda_implementation/group_kernel.py:26-74) and `hidden_states[fan_in_index]`
+ * (fma/modules/moe/__init__.py:269,275). divisor = top_k maps a slot to its token; divisor = 1 is a
+ * plain row gather. */
+int fma_gather_rows(const void* x, const int32_t* idx, int64_t R, int64_t H, int32_t divisor, void* out,
+                    int dtype, void* stream);
+
+/* y[t, :] = sum_{j<k} gates[t*k+j] * o[inv[t*k+j], :]  accumulated in fp32 in ascending j, rounded once.
+ * gates may be NULL (all ones; gives the k-way sum the backward of the gather needs). gates has dtype.
+ * Replaces ungroup_with_padding + torch.bmm(router_weights, y) (fma/modules/moe/__init__.py:235-246,
+ * ungroup_kernel.py:15-71) and `y * batch_gates` + index_add (fma/modules/moe/__init__.py:284-286). */
+int fma_combine(const void* o, const int32_t* inv, const void* gates, int64_t T, int64_t k, int64_t H,
+                void* y, int dtype, void* stream);
+
+/* Backward of fma_combine for one upstream gradient dy[T, H]:
+ *   d_o[inv[t*k+j], :] = gates[t*k+j] * dy[t, :]
+ *   d_gates[t*k+j]     = <dy[t, :], o[inv[t*k+j], :]>   (fp32 accumulate)
+ * d_gates may be NULL (skipped). Replaces the autograd of torch.bmm + _UngroupWithPadding.backward
+ * (fma/modules/moe/cuda_implementation/__init__.py:226-249) and group(grad_out, coeff=gates) +
+ * bmm(output_expanded, grad_out) of the triton branch (fma/modules/moe/triton_implementation/__init__.py:83-103). */
+int fma_combine_bwd(const void* dy, const void* o, const int32_t* inv, const void* gates, int64_t T,
+                    int64_t k, int64_t H, void* d_o, void* d_gates, int dtype, void* stream);
+
+/* ---- SwiGLU -------------------------------------------------------------------------------- */
+
+/* out[r, c] = up[r, c] * gate[r, c] * sigmoid(gate[r, c]) in fp32, rounded to dtype; rows x cols elements,
+ * each operand with its own row stride in elements (so the halves of a packed [rows, 2*cols] tensor can
+ * be passed without a copy). Replaces swiglu_forward_cuda(gate, up, output, BLOCK_SIZE)
+ * (fma/ops/swiglu/cuda_implementation/ops.cpp, forward.cu:59-94) and the strided Triton kernel
+ * (fma/ops/swiglu/triton_implementation/forward.py:16-46). */
+int fma_swiglu_forward(const void* gate, const void* up, void* out, int64_t rows, int64_t cols,
+                       int64_t gate_stride, int64_t up_stride, int64_t out_stride, int dtype, void* stream);
+
+/* gate_grad = dy * up * (s + gate*s*(1-s)), up_grad = dy * gate * s with s = sigmoid(gate).
+ * Replaces swiglu_backward_cuda(gate, up, output_grad, gate_grad, up_grad, BLOCK_SIZE)
+ * (fma/ops/swiglu/cuda_implementation/backward.cu:79-129) and triton_implementation/backward.py:16-55. */
+int fma_swiglu_backward(const void* gate, const void* up, const void* dy, void* gate_grad, void* up_grad,
+                        int64_t rows, int64_t cols, int64_t gate_stride, int64_t up_stride, int64_t dy_stride,
+                        int64_t gate_grad_stride, int64_t up_grad_stride, int dtype, void* stream);
+
+/* ---- grouped GEMM --------------------------------------------------------------------------- */
+
+/* For each group e < E:  D_e[M_e, N_e] = alpha * op(A_e) * op(B_e), fp32 accumulation, output rounded to dtype.
+ * Groups are packed back to back in the flat A / B / D buffers (element offsets sum M*K, sum K*N, sum M*N).
+ *   trans_a == 0: A_e stored [M_e, K_e] row-major;  trans_a != 0: stored [K_e, M_e].
+ *   trans_b != 0: B_e stored [N_e, K_e] row-major;  trans_b == 0: stored [K_e, N_e].
+ * M_arr / N_arr / K_arr: E uint32 each, DEVICE memory (never read on the host). A group with K_e == 0
+ * gets zeros; a group with M_e == 0 or N_e == 0 produces nothing. dtype: FMA_BF16 or FMA_F16.
+ * Each group's contiguous dimension should be a multiple of 8 elements (16 bytes); other groups are
+ * computed by a slow scalar path. E <= FMA_MAX_GROUPS.
+ * Replaces grouped_gemm_cuda(A, B, C, output, M_array, N_array, K_array, is_A_transposed,
+ * is_B_transposed, alpha, beta, benchmark) (fma/ops/grouped_gemm/cuda_implementation/ops.cpp,
+ * kernel.cu:354-388); beta must be 0 and C absent there, so neither exists here. */
+int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_arr, const uint32_t* N_arr,
+                     const uint32_t* K_arr, int64_t E, int trans_a, int trans_b, float alpha, int dtype,
+                     void* stream);
+
+/* Up-projection with SwiGLU fused into the epilogue. For each expert e with M_e rows (rows of all experts
+ * packed back to back, sum M_e = R):
+ *   h_e   = x_e[M_e, K] * W_e[2I, K]^T            (rounded to dtype; written to h if h != NULL)
+ *   act_e = h_e[:, :I] * silu(h_e[:, I:])         (first half "up", second half "gate")
+ * computed from the ROUNDED h so the result equals fma_grouped_gemm followed by fma_swiglu_forward bit for
+ * bit. W: [E, 2I, K] row-major; h: [R, 2I]; act: [R, I]; I % 8 == 0, K % 8 == 0.
+ * Fuses _GroupedGemmExperts.forward (fma/modules/moe/cuda_implementation/__init__.py:28-38) with
+ * swiglu_packed (fma/ops/swiglu/__init__.py:133-164, up/gate = chunk(2, -1) at :153). */
+int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, const uint32_t* M_arr,
+                            int64_t E, int64_t I, int64_t K, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FMA_HIP_H */
