@@ -1,0 +1,133 @@
+"""GPU parity of the grouped GEMM: exact on integer-valued operands (every layout, ragged / empty / one-row groups),
+within bf16 rounding on random operands, and the fused SwiGLU epilogue bit-identical to GEMM followed by swiglu."""
+
+import pytest
+import torch
+
+from fma import grouped_gemm, swiglu_packed
+from fma.modules.moe.cuda_implementation import grouped_gemm_swiglu_cuda
+from oracle import moe_oracle as O
+
+from gpu_util import DEV, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _u32(values):
+    return torch.tensor(values, dtype=torch.int64).to(torch.uint32).to(DEV)
+
+
+def _integer_operands(M_list, N_list, K_list, tA, tB, seed):
+    g = torch.Generator().manual_seed(seed)
+    As, Bs = [], []
+    for M, N, K in zip(M_list, N_list, K_list):
+        As.append(torch.randint(-8, 9, (K, M) if tA else (M, K), generator=g).to(torch.bfloat16))
+        Bs.append(torch.randint(-8, 9, (N, K) if tB else (K, N), generator=g).to(torch.bfloat16))
+    return torch.cat([a.reshape(-1) for a in As]), torch.cat([b.reshape(-1) for b in Bs])
+
+
+@pytest.mark.parametrize("tA", [False, True])
+@pytest.mark.parametrize("tB", [False, True])
+@pytest.mark.parametrize(
+    "M_list,N,K",
+    [
+        ([8], 8, 8),
+        ([256], 256, 64),
+        ([264, 0, 8, 520, 1000], 264, 200),  # empty group, tails in every dimension
+        ([1, 7, 13], 24, 40),  # M not a multiple of 8 (for tA that is the contiguous dimension: scalar path)
+        ([300, 300], 512, 72),
+        ([16, 16], 20, 36),  # N, K not multiples of 8: scalar path
+    ],
+)
+def test_integer_known_answer_small(tA, tB, M_list, N, K):
+    E = len(M_list)
+    A, B = _integer_operands(M_list, [N] * E, [K] * E, tA, tB, seed=7)
+    expect = O.grouped_gemm(A, B, M_list, [N] * E, [K] * E, tA, tB)
+    got = grouped_gemm(
+        A=A.to(DEV), B=B.to(DEV), C=None, M_array=_u32(M_list), N_array=_u32([N] * E), K_array=_u32([K] * E),
+        output_shape=(sum(M_list) * N,), is_A_transposed=tA, is_B_transposed=tB,
+    )
+    assert got.shape == expect.shape and got.dtype == torch.bfloat16
+    assert float((got.cpu().float() - expect.float()).abs().max()) == 0
+
+
+@pytest.mark.parametrize("tA", [False, True])
+@pytest.mark.parametrize("tB", [False, True])
+def test_integer_known_answer_reference_shape(tA, tB):
+    # the reference's test: E=16, sum(M)=65536, N=512, K=4096, operands integers in [-8, 8], max |diff| == 0
+    # (tests/ops/grouped_gemm_test.py:38-92). Expected values: fp32 matmul on the GPU, exact for these operands
+    # (|sum| <= 64*4096 < 2^24) in any summation order.
+    torch.manual_seed(42)
+    E, K, N = 16, 4096, 512
+    M_list = [512, 3176, 2048] * 5 + [36856]
+    As, Bs, Ds = [], [], []
+    for M in M_list:
+        a = torch.randint(-8, 9, (K, M) if tA else (M, K), device=DEV, dtype=torch.bfloat16)
+        b = torch.randint(-8, 9, (N, K) if tB else (K, N), device=DEV, dtype=torch.bfloat16)
+        As.append(a)
+        Bs.append(b)
+        Ds.append(((a.T if tA else a).float() @ (b.T if tB else b).float()).to(torch.bfloat16).reshape(-1))
+    A = torch.cat([a.reshape(-1) for a in As])
+    B = torch.cat([b.reshape(-1) for b in Bs])
+    out = grouped_gemm(
+        A=A, B=B, C=None, M_array=_u32(M_list), N_array=_u32([N] * E), K_array=_u32([K] * E),
+        output_shape=(sum(M_list) * N,), is_A_transposed=tA, is_B_transposed=tB,
+    )
+    assert float((out.float() - torch.cat(Ds).float()).abs().max()) == 0
+
+
+def test_varying_n_and_k_per_group_and_alpha():
+    M_list, N_list, K_list = [40, 264, 8], [16, 520, 256], [64, 8, 136]
+    A, B = _integer_operands(M_list, N_list, K_list, False, True, seed=9)
+    expect = O.grouped_gemm(A, B, M_list, N_list, K_list, False, True, alpha=0.5)
+    got = grouped_gemm(
+        A=A.to(DEV), B=B.to(DEV), C=None, M_array=_u32(M_list), N_array=_u32(N_list), K_array=_u32(K_list),
+        output_shape=(sum(m * n for m, n in zip(M_list, N_list)),), alpha=0.5, is_A_transposed=False,
+        is_B_transposed=True,
+    )
+    assert torch.equal(got.cpu(), expect)
+
+
+@pytest.mark.parametrize("tA,tB", [(False, True), (False, False), (True, False)])
+def test_random_operands_within_bf16_rounding(tA, tB):
+    # bf16 N(0,1) operands against fp32 math on the same bf16 values; the only difference is summation order in
+    # fp32 and the final rounding to bf16: relative error of one bf16 ulp (2^-8) of the largest output
+    torch.manual_seed(5)
+    M_list, N, K = [700, 3, 1029, 0, 256], 384, 1536
+    E = len(M_list)
+    As = [torch.randn((K, M) if tA else (M, K)).bfloat16() for M in M_list]
+    Bs = [torch.randn((N, K) if tB else (K, N)).bfloat16() for _ in M_list]
+    A = torch.cat([a.reshape(-1) for a in As])
+    B = torch.cat([b.reshape(-1) for b in Bs])
+    expect = O.grouped_gemm(A.float(), B.float(), M_list, [N] * E, [K] * E, tA, tB)
+    got = grouped_gemm(
+        A=A.to(DEV), B=B.to(DEV), C=None, M_array=_u32(M_list), N_array=_u32([N] * E), K_array=_u32([K] * E),
+        output_shape=(sum(M_list) * N,), is_A_transposed=tA, is_B_transposed=tB,
+    )
+    max_rel, frob_rel = rel_err(got, expect)
+    assert max_rel <= 2**-8 and frob_rel <= 2**-8
+
+
+@pytest.mark.parametrize("M_list,I,K", [([100, 0, 300, 1], 128, 64), ([512, 260], 1408, 256), ([40] * 16, 72, 520)])
+def test_fused_swiglu_equals_gemm_then_swiglu(M_list, I, K):
+    torch.manual_seed(I)
+    E, R = len(M_list), sum(M_list)
+    x = torch.randn(R, K).bfloat16().to(DEV)
+    w = (torch.randn(E, 2 * I, K) * 0.1).bfloat16().to(DEV)
+    M = _u32(M_list)
+    h = torch.empty(R, 2 * I, dtype=torch.bfloat16, device=DEV)
+    act = torch.empty(R, I, dtype=torch.bfloat16, device=DEV)
+    grouped_gemm_swiglu_cuda(x, w, M, h, act)
+    h_ref = grouped_gemm(
+        A=x, B=w, C=None, M_array=M, N_array=_u32([2 * I] * E), K_array=_u32([K] * E), output_shape=(R, 2 * I),
+        is_A_transposed=False, is_B_transposed=True,
+    )
+    assert torch.equal(h, h_ref)
+    assert torch.equal(act, swiglu_packed(h_ref))
+    # against the oracle: per-expert linear, then up * silu(gate) with up = first half
+    xs = x.cpu().float().split(M_list)
+    expect = torch.cat([O.swiglu_packed((xs[e] @ w[e].cpu().float().T).bfloat16()) for e in range(E)])
+    assert rel_err(act, expect)[0] <= 2**-7
+    act_only = torch.empty_like(act)
+    grouped_gemm_swiglu_cuda(x, w, M, None, act_only)
+    assert torch.equal(act_only, act)

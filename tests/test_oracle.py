@@ -1,0 +1,242 @@
+"""Pins the CPU oracle (oracle/) without the reference: library routines, closed forms, invariants, brute force and
+the reference's own known-answer constructions, chosen so that a dropped term, a wrong index or a transposed operand
+fails at least one of them."""
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import c_oracle, moe_oracle as O
+
+
+# ---- continuous_count --------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("impl", [O.continuous_count, c_oracle.continuous_count])
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_count_matches_bincount(impl, dtype):
+    # the reference's generator: randint(0, 72), seed 42 (tests/ops/continuous_count_test.py:36-41)
+    torch.manual_seed(42)
+    for n in [1, 2, 63, 64, 65, 1000, 4097, 100003]:
+        x = torch.randint(0, 72, (n,)).numpy().astype(dtype)
+        assert np.array_equal(impl(x, 72), np.bincount(x, minlength=72).astype(np.uint32))
+
+
+@pytest.mark.parametrize("impl", [O.continuous_count, c_oracle.continuous_count])
+def test_count_closed_forms(impl):
+    E, n = 64, 10_000
+    out = impl(np.full(n, 17, np.int32), E)
+    expect = np.zeros(E, np.uint32)
+    expect[17] = n
+    assert np.array_equal(out, expect)
+    out = impl((np.arange(n) % E).astype(np.int32), E)
+    assert np.array_equal(out, np.array([n // E + (1 if e < n % E else 0) for e in range(E)], np.uint32))
+    assert np.array_equal(impl(np.zeros(0, np.int32), E), np.zeros(E, np.uint32))
+
+
+@pytest.mark.parametrize("impl", [O.continuous_count, c_oracle.continuous_count])
+def test_count_brute_force_and_out_of_range(impl):
+    rng = np.random.default_rng(0)
+    x = rng.integers(-3, 12, size=777).astype(np.int64)
+    expect = np.zeros(8, np.uint32)
+    for v in x.tolist():
+        if 0 <= v < 8:
+            expect[v] += 1
+    assert np.array_equal(impl(x, 8), expect)
+    assert int(impl(x, 8).sum()) == int(((x >= 0) & (x < 8)).sum())
+
+
+def test_count_size_one_shortcut():
+    # size == 1 returns the element count whatever the values are (fma/ops/continuous_count/__init__.py:29-30)
+    assert np.array_equal(O.continuous_count(np.array([5, 7, 9], np.int32), 1), np.array([3], np.uint32))
+
+
+# ---- routing index -------------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("impl", [O.routing_index, c_oracle.routing_index])
+@pytest.mark.parametrize("T,E,k,kind", [(7, 8, 2, "uniform"), (512, 8, 2, "uniform"), (300, 64, 8, "zipf"), (129, 128, 8, "uniform")])
+def test_index_matches_stable_sort(impl, T, E, k, kind):
+    selected, _ = O.make_routing(T, E, k, kind, seed=3, empty_tail=4 if kind == "zipf" else 0)
+    idx = impl(selected.numpy(), E)
+    flat = selected.flatten()
+    sorted_ids, sorted_slots = flat.sort(stable=True)
+    assert np.array_equal(idx["perm"], sorted_slots.numpy().astype(np.int32))
+    assert np.array_equal(idx["eid"], sorted_ids.numpy().astype(np.int32))
+    assert np.array_equal(idx["counts"], np.bincount(flat.numpy(), minlength=E).astype(np.uint32))
+    assert np.array_equal(idx["offsets"], np.cumsum(idx["counts"]).astype(np.uint32))
+    R = T * k
+    assert np.array_equal(np.sort(idx["perm"]), np.arange(R, dtype=np.int32))  # a permutation
+    assert np.array_equal(idx["inv"][idx["perm"]], np.arange(R, dtype=np.int32))  # its inverse
+    assert (np.diff(idx["eid"]) >= 0).all()
+    if kind == "zipf":
+        assert (idx["counts"][-4:] == 0).all()  # the forced-empty experts really are empty
+
+
+def test_index_brute_force_tiny():
+    ids = np.array([[2, 0], [1, 2], [0, 1], [2, 1]])
+    idx = O.routing_index(ids, 3)
+    # slots: 0:2 1:0 2:1 3:2 4:0 5:1 6:2 7:1 -> expert 0: [1,4], expert 1: [2,5,7], expert 2: [0,3,6]
+    assert idx["perm"].tolist() == [1, 4, 2, 5, 7, 0, 3, 6]
+    assert idx["eid"].tolist() == [0, 0, 1, 1, 1, 2, 2, 2]
+    assert idx["counts"].tolist() == [2, 3, 3] and idx["offsets"].tolist() == [2, 5, 8]
+    assert idx["inv"].tolist() == [5, 0, 2, 6, 1, 3, 7, 4]
+
+
+# ---- grouped GEMM ---------------------------------------------------------------------------------------------
+
+
+def _integer_kat(M_list, N, K, tA, tB, seed=42):
+    """the reference's known-answer construction (tests/ops/grouped_gemm_test.py:38-92): bf16 operands that are
+    integers in [-8, 8], so fp32 accumulation is exact; expected values come from an int64 matmul here."""
+    g = torch.Generator().manual_seed(seed)
+    As, Bs, Ds = [], [], []
+    for M in M_list:
+        a = torch.randint(-8, 9, (K, M) if tA else (M, K), generator=g)
+        b = torch.randint(-8, 9, (N, K) if tB else (K, N), generator=g)
+        As.append(a)
+        Bs.append(b)
+        Ds.append(((a.T if tA else a) @ (b.T if tB else b)).reshape(-1))
+    A = torch.cat([a.reshape(-1) for a in As]).to(torch.bfloat16)
+    B = torch.cat([b.reshape(-1) for b in Bs]).to(torch.bfloat16)
+    D = torch.cat(Ds)
+    return A, B, D
+
+
+@pytest.mark.parametrize("tA", [False, True])
+@pytest.mark.parametrize("tB", [False, True])
+def test_grouped_gemm_integer_kat(tA, tB):
+    M_list, N, K = [5, 0, 33, 1, 17], 24, 40
+    A, B, D = _integer_kat(M_list, N, K, tA, tB)
+    out = O.grouped_gemm(A, B, M_list, [N] * 5, [K] * 5, tA, tB)
+    expect = D.to(torch.float32).to(torch.bfloat16)  # |D| <= 64*40 fits fp32 exactly, then one RNE to bf16
+    assert torch.equal(out, expect)
+
+
+def test_grouped_gemm_reduces_to_mm_and_bmm():
+    torch.manual_seed(0)
+    a, b = torch.randn(9, 16), torch.randn(16, 12)
+    assert torch.allclose(O.grouped_gemm(a, b, [9], [12], [16]).reshape(9, 12), a @ b, atol=1e-5)
+    assert torch.allclose(O.grouped_gemm(a, b.T.contiguous(), [9], [12], [16], False, True).reshape(9, 12), a @ b, atol=1e-5)
+    assert torch.allclose(O.grouped_gemm(a.T.contiguous(), b, [9], [12], [16], True, False).reshape(9, 12), a @ b, atol=1e-5)
+    a3, b3 = torch.randn(4, 9, 16), torch.randn(4, 16, 12)
+    out = O.grouped_gemm(a3, b3, [9] * 4, [12] * 4, [16] * 4, alpha=0.5)
+    assert torch.allclose(out.reshape(4, 9, 12), 0.5 * torch.bmm(a3, b3), atol=1e-5)
+
+
+# ---- SwiGLU ---------------------------------------------------------------------------------------------------
+
+
+def test_swiglu_closed_forms():
+    g = torch.tensor([0.0, 100.0, -100.0, 1.0])
+    u = torch.tensor([3.0, 2.0, 2.0, -1.5])
+    y = O.swiglu(g, u)
+    assert y[0] == 0 and y[1] == 200.0 and abs(float(y[2])) < 1e-30
+    assert torch.allclose(y[3], torch.tensor(-1.5 / (1 + np.exp(-1.0)), dtype=torch.float32), atol=1e-7)
+    assert torch.equal(O.swiglu(g, u), u * F.silu(g))
+    dg, du = O.swiglu_backward(torch.zeros(3), u[:3], torch.ones(3))
+    assert torch.allclose(dg, u[:3] / 2) and torch.equal(du, torch.zeros(3))  # gate = 0: dgate = dy*up/2, dup = 0
+
+
+def test_swiglu_packed_halves_and_derivative():
+    torch.manual_seed(1)
+    x = torch.randn(5, 8, dtype=torch.float64, requires_grad=True)
+    y = O.swiglu_packed(x)
+    assert torch.allclose(y, x[:, :4] * F.silu(x[:, 4:]))  # first half up, second half gate
+    dy = torch.randn(5, 4, dtype=torch.float64)
+    (gx,) = torch.autograd.grad(y, x, dy)
+    dg, du = O.swiglu_backward(x[:, 4:].detach().float(), x[:, :4].detach().float(), dy.float())
+    assert torch.allclose(gx[:, 4:].float(), dg, atol=1e-5) and torch.allclose(gx[:, :4].float(), du, atol=1e-5)
+
+
+# ---- routing weights and the layer -----------------------------------------------------------------------------
+
+
+def test_routing_weights_properties():
+    torch.manual_seed(2)
+    x, w = torch.randn(33, 16), torch.randn(8, 16)
+    logits, weights, selected = O.routing_weights(x, w, 3)
+    assert torch.allclose(logits, x @ w.T, atol=1e-6)
+    assert torch.allclose(weights.sum(-1), torch.ones(33), atol=1e-6)
+    assert torch.equal(selected, logits.topk(3).indices)
+    assert torch.allclose(weights, F.softmax(logits.gather(1, selected), -1))
+    _, w_all, sel_all = O.routing_weights(x, w, 8)  # k == E: a full softmax, reordered
+    assert torch.allclose(torch.zeros(33, 8).scatter(1, sel_all, w_all), F.softmax(logits, -1), atol=1e-6)
+    _, w1, s1 = O.routing_weights(x, w, 1)
+    assert torch.equal(s1[:, 0], logits.argmax(-1)) and torch.equal(w1, torch.ones(33, 1))
+
+
+def test_layer_collapses_to_dense_mlp():
+    # E = 1, k = 1: softmax of one logit is 1, so the layer is linear -> swiglu -> linear
+    torch.manual_seed(3)
+    T, H, I = 19, 16, 24
+    x, wg = torch.randn(T, H), torch.randn(1, H)
+    w1, w2 = torch.randn(1, 2 * I, H) * 0.1, torch.randn(1, H, I) * 0.1
+    y, _ = O.moe_layer(x, wg, w1, w2, 1)
+    h = x @ w1[0].T
+    dense = (h[:, :I] * F.silu(h[:, I:])) @ w2[0].T
+    assert torch.allclose(y, dense, atol=1e-5)
+
+
+def test_layer_against_per_token_loop():
+    # brute force: every token visits its k experts one by one
+    torch.manual_seed(4)
+    T, H, I, E, k = 23, 8, 12, 5, 2
+    x = torch.randn(T, H, dtype=torch.float64)
+    w1 = torch.randn(E, 2 * I, H, dtype=torch.float64) * 0.3
+    w2 = torch.randn(E, H, I, dtype=torch.float64) * 0.3
+    selected, weights = O.make_routing(T, E, k, "uniform", seed=5)
+    weights = weights.double()
+    y = O.moe_experts(x, weights, selected, w1, w2)
+    expect = torch.zeros(T, H, dtype=torch.float64)
+    for t in range(T):
+        for j in range(k):
+            e = int(selected[t, j])
+            h = w1[e] @ x[t]
+            expect[t] += weights[t, j] * (w2[e] @ (h[:I] * F.silu(h[I:])))
+    assert torch.allclose(y, expect, atol=1e-10)
+
+
+def test_layer_token_permutation_equivariance_and_empty_expert_grads():
+    torch.manual_seed(6)
+    T, H, I, E, k = 40, 8, 8, 6, 2
+    x = torch.randn(T, H, dtype=torch.float64)
+    w1 = (torch.randn(E, 2 * I, H, dtype=torch.float64) * 0.3).requires_grad_()
+    w2 = (torch.randn(E, H, I, dtype=torch.float64) * 0.3).requires_grad_()
+    selected, weights = O.make_routing(T, E, k, "zipf", seed=7, empty_tail=2)
+    weights = weights.double()
+    y = O.moe_experts(x, weights, selected, w1, w2)
+    p = torch.randperm(T)
+    assert torch.allclose(O.moe_experts(x[p], weights[p], selected[p], w1, w2), y[p], atol=1e-12)
+    y.sum().backward()
+    assert torch.equal(w1.grad[-2:], torch.zeros_like(w1.grad[-2:]))  # experts without tokens: exact zeros
+    assert torch.equal(w2.grad[-2:], torch.zeros_like(w2.grad[-2:]))
+    assert w1.grad[:4].abs().sum() > 0
+
+
+def test_layer_gradcheck_fp64():
+    torch.manual_seed(8)
+    T, H, I, E, k = 6, 4, 4, 3, 2
+    selected, weights = O.make_routing(T, E, k, "uniform", seed=9)
+    x = torch.randn(T, H, dtype=torch.float64, requires_grad=True)
+    g = weights.double().requires_grad_()
+    w1 = (torch.randn(E, 2 * I, H, dtype=torch.float64) * 0.5).requires_grad_()
+    w2 = (torch.randn(E, H, I, dtype=torch.float64) * 0.5).requires_grad_()
+    assert torch.autograd.gradcheck(lambda a, b, c, d: O.moe_experts(a, b, selected, c, d), (x, g, w1, w2))
+
+
+def test_golden_fixture_is_what_the_oracle_computes():
+    import os
+
+    from tests.golden.make_golden import c1_inputs
+
+    fx = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "c1_moe_fp32.npz"))
+    x, wg, w1, w2 = c1_inputs()
+    assert abs(float(x.double().sum()) - float(fx["x_sum"])) < 1e-6
+    _, weights, selected = O.routing_weights(x, wg, 2)
+    assert np.array_equal(selected.numpy(), fx["selected"])
+    y = O.moe_experts(x, weights, selected, w1, w2)
+    assert np.allclose(y.numpy(), fx["y"], atol=1e-6)
+    idx = O.routing_index(selected.numpy(), 8)
+    assert np.array_equal(idx["perm"], fx["perm"]) and np.array_equal(idx["counts"], fx["counts"])
