@@ -42,20 +42,26 @@ def parse_args():
     return p.parse_args()
 
 
-def time_gpu(fn, iters, warmup=2):
-    """average milliseconds per call of fn(i), events recorded on the current stream (the launch stream)"""
+def time_gpu(fn, iters, warmup=3, blocker=None):
+    """Median and mean milliseconds of one launch of fn(i). Every launch is bracketed by its own pair of events on the
+    current stream (the stream the kernels are launched on). `blocker` first queues a few milliseconds of other GPU
+    work, so that all launches are already in the queue when the GPU reaches them and no host latency is measured."""
     import torch
 
     for i in range(warmup):
         fn(i)
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
     torch.cuda.synchronize()
-    start.record()
+    if blocker is not None:
+        blocker()
     for i in range(iters):
+        starts[i].record()
         fn(i)
-    stop.record()
-    stop.synchronize()
-    return start.elapsed_time(stop) / iters
+        stops[i].record()
+    torch.cuda.synchronize()
+    times = sorted(starts[i].elapsed_time(stops[i]) for i in range(iters))
+    return times[len(times) // 2], sum(times) / len(times)
 
 
 def main():
@@ -138,72 +144,104 @@ def main():
         "layer_gemm_frac_of_peak": gemm_flops_step / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
     }
 
-    # ---- per-kernel measurements -------------------------------------------------------------------------
+    # ---- per-kernel measurements: direct C-ABI calls, one event pair per launch ----------------------------
     if not args.no_kernels:
+        lib = fma._lib.load()
+        stream = torch.cuda.current_stream().cuda_stream
+        BF16 = fma._lib.FMA_BF16
         kernels = {}
         counts, offsets, perm, eid, inv = ci.build_routing_index(selected_d, E)
         N_fc, K_fc = moe.c_fc.N_array, moe.c_fc.K_array
         N_pj, K_pj = moe.c_proj.N_array, moe.c_proj.K_array
         w1, w2 = moe.c_fc.weight.detach(), moe.c_proj.weight.detach()
-        xg = torch.empty(R, H, dtype=torch.bfloat16, device=dev)
-        h = torch.empty(R, 2 * I, dtype=torch.bfloat16, device=dev)
-        a = torch.empty(R, I, dtype=torch.bfloat16, device=dev)
+        bf = dict(dtype=torch.bfloat16, device=dev)
+        xg = torch.empty(R, H, **bf)
+        h = torch.empty(R, 2 * I, **bf)
+        a = torch.empty(R, I, **bf)
         o = torch.randn(R, H, device=dev).bfloat16()
         dh = torch.randn(R, 2 * I, device=dev).bfloat16()
-        y = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
-        d_o = torch.empty(R, H, dtype=torch.bfloat16, device=dev)
-        dgates = torch.empty(T, k, dtype=torch.bfloat16, device=dev)
-        ci.gather_rows_cuda(x, perm, k, xg)
-        iters = max(3, args.steps)
+        y = torch.empty(T, H, **bf)
+        d_o = torch.randn(R, H, device=dev).bfloat16()
+        da = torch.empty(R, I, **bf)
+        dxg = torch.empty(R, H, **bf)
+        dw1 = torch.empty(E, 2 * I, H, **bf)
+        dw2 = torch.empty(E, H, I, **bf)
+        dgates = torch.empty(T, k, **bf)
+        blk = torch.randn(8192, 8192, device=dev).bfloat16()
 
-        def mfma(name, flops, ms):
-            tf = flops / (ms * 1e-3) / 1e12
-            kernels[name] = {"ms": ms, "bound": "mfma", "achieved": tf, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                             "frac": tf / PEAK_BF16_TFLOPS}
+        def blocker():  # ~10 ms of queued GPU work, so the host runs ahead of the GPU
+            for _ in range(6):
+                torch.mm(blk, blk)
 
-        def hbm(name, nbytes, ms):
-            gbs = nbytes / (ms * 1e-3) / 1e9
-            kernels[name] = {"ms": ms, "bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                             "frac": gbs / PEAK_HBM_GBS, "bytes": nbytes}
+        def ok(rc):
+            if rc != 0:
+                raise RuntimeError(lib.fma_last_error_string().decode())
 
-        ms = time_gpu(lambda i: ci.grouped_gemm_swiglu_cuda(xg, w1, counts, h, a), iters)
-        mfma("up_projection_swiglu_fwd(NT)", 2.0 * R * 2 * I * H, ms)
-        ms = time_gpu(lambda i: grouped_gemm(A=a, B=w2, C=None, M_array=counts, N_array=N_pj, K_array=K_pj,
-                                             output_shape=(R, H), is_A_transposed=False, is_B_transposed=True), iters)
-        mfma("down_projection_fwd(NT)", 2.0 * R * I * H, ms)
-        ms = time_gpu(lambda i: grouped_gemm(A=d_o, B=w2, C=None, M_array=counts, N_array=K_pj, K_array=N_pj,
-                                             output_shape=(R, I), is_A_transposed=False, is_B_transposed=False), iters)
-        mfma("down_projection_dgrad(NN)", 2.0 * R * I * H, ms)
-        ms = time_gpu(lambda i: grouped_gemm(A=d_o, B=a, C=None, M_array=N_pj, N_array=K_pj, K_array=counts,
-                                             output_shape=(E, H, I), is_A_transposed=True, is_B_transposed=False), iters)
-        mfma("down_projection_wgrad(TN)", 2.0 * R * I * H, ms)
-        ms = time_gpu(lambda i: grouped_gemm(A=dh, B=w1, C=None, M_array=counts, N_array=K_fc, K_array=N_fc,
-                                             output_shape=(R, H), is_A_transposed=False, is_B_transposed=False), iters)
-        mfma("up_projection_dgrad(NN)", 2.0 * R * 2 * I * H, ms)
-        ms = time_gpu(lambda i: grouped_gemm(A=dh, B=xg, C=None, M_array=N_fc, N_array=K_fc, K_array=counts,
-                                             output_shape=(E, 2 * I, H), is_A_transposed=True, is_B_transposed=False), iters)
-        mfma("up_projection_wgrad(TN)", 2.0 * R * 2 * I * H, ms)
+        def gemm(A, B, D, M, N, K, ta, tb):
+            ok(lib.fma_grouped_gemm(A.data_ptr(), B.data_ptr(), D.data_ptr(), M.data_ptr(), N.data_ptr(), K.data_ptr(),
+                                    E, ta, tb, 1.0, BF16, stream))
 
-        # row kernels: algorithmic bytes = each distinct input row once + each output row once + index/gate words
-        ms = time_gpu(lambda i: ci.gather_rows_cuda(x, perm, k, xg), 20)
-        hbm("gather_rows", T * H * s + R * H * s + R * 4, ms)
-        ms = time_gpu(lambda i: ci.combine_cuda(o, inv, weights_d, k, y), 20)
-        hbm("combine", R * H * s + R * (4 + s) + T * H * s, ms)
-        ms = time_gpu(lambda i: ci.combine_backward_cuda(dy, o, inv, weights_d, k, d_o, dgates), 20)
-        hbm("combine_backward", T * H * s + 2 * R * H * s + R * (4 + 2 * s), ms)
-        up, gate = h.chunk(2, dim=-1)
-        dup, dgate = dh.chunk(2, dim=-1)
-        ms = time_gpu(lambda i: swiglu_backward_cuda(gate, up, a, dgate, dup, 1024), 10)
-        hbm("swiglu_backward", 5 * R * I * s, ms)
-        ms = time_gpu(lambda i: ci.build_routing_index(selected_d, E), 20)
-        kernels["build_routing_index(3 launches)"] = {"ms": ms}
+        ok(lib.fma_gather_rows(x.data_ptr(), perm.data_ptr(), R, H, k, xg.data_ptr(), BF16, stream))
+        iters = max(5, args.steps)
+
+        def mfma(name, flops, t):
+            tf = flops / (t[0] * 1e-3) / 1e12
+            kernels[name] = {"ms": t[0], "ms_mean": t[1], "bound": "mfma", "achieved": tf, "peak": PEAK_BF16_TFLOPS,
+                             "unit": "TFLOP/s", "frac": tf / PEAK_BF16_TFLOPS, "flop": flops}
+
+        def hbm(name, nbytes, t):
+            gbs = nbytes / (t[0] * 1e-3) / 1e9
+            kernels[name] = {"ms": t[0], "ms_mean": t[1], "bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS,
+                             "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "bytes": nbytes}
+
+        t = time_gpu(lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), h.data_ptr(), a.data_ptr(),
+                                                              counts.data_ptr(), E, I, H, BF16, stream)), iters, blocker=blocker)
+        mfma("up_projection_swiglu_fwd(NT)", 2.0 * R * 2 * I * H, t)
+        mfma("down_projection_fwd(NT)", 2.0 * R * I * H,
+             time_gpu(lambda i: gemm(a, w2, o, counts, N_pj, K_pj, 0, 1), iters, blocker=blocker))
+        mfma("down_projection_dgrad(NN)", 2.0 * R * I * H,
+             time_gpu(lambda i: gemm(d_o, w2, da, counts, K_pj, N_pj, 0, 0), iters, blocker=blocker))
+        mfma("down_projection_wgrad(TN)", 2.0 * R * I * H,
+             time_gpu(lambda i: gemm(d_o, a, dw2, N_pj, K_pj, counts, 1, 0), iters, blocker=blocker))
+        mfma("up_projection_dgrad(NN)", 2.0 * R * 2 * I * H,
+             time_gpu(lambda i: gemm(dh, w1, dxg, counts, K_fc, N_fc, 0, 0), iters, blocker=blocker))
+        mfma("up_projection_wgrad(TN)", 2.0 * R * 2 * I * H,
+             time_gpu(lambda i: gemm(dh, xg, dw1, N_fc, K_fc, counts, 1, 0), iters, blocker=blocker))
+
+        # row kernels: algorithmic bytes = each distinct input row once + each output row once + index / gate words
+        hbm("gather_rows", T * H * s + R * H * s + R * 4,
+            time_gpu(lambda i: ok(lib.fma_gather_rows(x.data_ptr(), perm.data_ptr(), R, H, k, xg.data_ptr(), BF16, stream)),
+                     20, blocker=blocker))
+        hbm("combine", R * H * s + R * (4 + s) + T * H * s,
+            time_gpu(lambda i: ok(lib.fma_combine(o.data_ptr(), inv.data_ptr(), weights_d.data_ptr(), T, k, H, y.data_ptr(),
+                                                  BF16, stream)), 20, blocker=blocker))
+        hbm("combine_backward", T * H * s + 2 * R * H * s + R * (4 + 2 * s),
+            time_gpu(lambda i: ok(lib.fma_combine_bwd(dy.data_ptr(), o.data_ptr(), inv.data_ptr(), weights_d.data_ptr(), T, k,
+                                                      H, d_o.data_ptr(), dgates.data_ptr(), BF16, stream)), 20, blocker=blocker))
+        es = 2 * I  # row stride of the packed pre-activation and of its gradient
+        hbm("swiglu_backward", 5 * R * I * s,
+            time_gpu(lambda i: ok(lib.fma_swiglu_backward(h.data_ptr() + I * s, h.data_ptr(), da.data_ptr(),
+                                                          dh.data_ptr() + I * s, dh.data_ptr(), R, I, es, es, I, es, es,
+                                                          BF16, stream)), 10, blocker=blocker))
+        ws_idx = torch.empty(max(lib.fma_moe_build_index_workspace_bytes(R, E), 4) // 4, dtype=torch.int32, device=dev)
+        t = time_gpu(lambda i: ok(lib.fma_moe_build_index(selected_d.data_ptr(), 8, R, E, counts.data_ptr(), offsets.data_ptr(),
+                                                          perm.data_ptr(), eid.data_ptr(), inv.data_ptr(), ws_idx.data_ptr(),
+                                                          ws_idx.numel() * 4, stream)), 20, blocker=blocker)
+        kernels["build_routing_index(3 launches)"] = {"ms": t[0], "ms_mean": t[1]}
 
         # continuous_count on 16 Mi int32 ids in [0, 64): five distinct 64 MiB buffers (320 MiB > the 256 MiB
         # last-level cache) so that every launch reads from HBM
+        n_ids, bins = 16 << 20, 64
+        ws_cnt = torch.empty(lib.fma_continuous_count_workspace_bytes(n_ids, bins), dtype=torch.uint8, device=dev)
+        out_cnt = torch.empty(bins, dtype=torch.uint32, device=dev)
         for kind in ("uniform", "zipf"):
-            ids = [torch.from_numpy(O.make_ids(16 << 20, 64, kind, seed=100 + j)).to(dev) for j in range(5)]
-            ms = time_gpu(lambda i: continuous_count(ids[i % 5], 64), 50, warmup=5)
-            hbm(f"continuous_count_16Mi_{kind}", (16 << 20) * 4 + 64 * 4, ms)
+            ids = [torch.from_numpy(O.make_ids(n_ids, bins, kind, seed=100 + j)).to(dev) for j in range(5)]
+            t = time_gpu(lambda i: ok(lib.fma_continuous_count(ids[i % 5].data_ptr(), 4, n_ids, out_cnt.data_ptr(), bins,
+                                                               ws_cnt.data_ptr(), ws_cnt.numel(), stream)), 50, warmup=5,
+                         blocker=blocker)
+            hbm(f"continuous_count_16Mi_{kind}", n_ids * 4 + bins * 4, t)
+            expect = np.bincount(O.make_ids(n_ids, bins, kind, seed=100 + 49 % 5), minlength=bins)
+            assert np.array_equal(out_cnt.cpu().view(torch.int32).numpy().astype(np.int64), expect), "count mismatch"
             del ids
         result["kernels"] = kernels
         dominant = kernels["up_projection_swiglu_fwd(NT)"]
@@ -216,7 +254,7 @@ def main():
             "frac": dominant["frac"],
             "traffic": None,
         }
-        del xg, h, a, o, dh, y, d_o
+        del xg, h, a, o, dh, y, d_o, da, dxg, dw1, dw2, blk
 
     # ---- CPU baseline: the oracle (a port of the reference's torch backend) on a bounded sample -------------
     if not args.no_cpu:

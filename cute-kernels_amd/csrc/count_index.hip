@@ -3,9 +3,10 @@
 // continuous_count: one launch. Every workgroup streams a contiguous chunk of ids with 16-byte loads and
 // counts into an LDS histogram that holds NREP lane-private copies of every bin (address = id*NREP + lane%NREP),
 // so lanes that carry the same id still hit different LDS banks and a skewed distribution costs the same as a
-// uniform one. The copies are folded, the per-workgroup histogram is written to a workspace row, and the
-// workgroup that draws the last ticket sums the rows into the output: no zeroing pass, no atomics on the
-// output, and the result does not depend on arrival order.
+// uniform one. The copies are folded and the per-workgroup histogram is written to a workspace row; a second, tiny
+// launch sums the rows into the output. No zeroing pass, no atomics on global memory and no fences: a last-arriver
+// ticket inside one launch needs agent-scope release/acquire fences, which on this multi-XCD part write back and
+// invalidate the L2 once per workgroup and cost twenty times the streaming itself.
 //
 // index construction: three small launches (per-chunk histogram, scan, placement). Chunks are contiguous
 // ranges of slots, so "expert-major, chunk-minor, slot order inside the chunk" is exactly the stable order.
@@ -17,7 +18,6 @@ namespace {
 constexpr int kCountThreads = 1024;
 constexpr int kCountUnroll = 4;
 constexpr int kCountLdsWords = 16384;  // 64 KB of bins (all copies)
-constexpr int kTicketWords = 64;       // 256-byte ticket area in front of the partial rows
 
 __host__ __device__ inline uint32_t floor_pow2(uint32_t x) {
     uint32_t p = 1;
@@ -63,10 +63,9 @@ __device__ __forceinline__ void count_one(id_t id, uint32_t E, uint32_t nrep_log
 template <typename id_t>
 __global__ __launch_bounds__(kCountThreads) void continuous_count_kernel(const id_t* __restrict__ ids, uint64_t n,
                                                                          uint32_t E, uint32_t nrep_log2,
-                                                                         uint64_t chunk, uint32_t* ws,
-                                                                         uint32_t* __restrict__ out) {
+                                                                         uint64_t chunk,
+                                                                         uint32_t* __restrict__ partials) {
     extern __shared__ uint32_t bins[];
-    __shared__ uint32_t s_is_last;
 
     constexpr int VEC = 16 / sizeof(id_t);
     struct alignas(16) IdVec {
@@ -77,8 +76,6 @@ __global__ __launch_bounds__(kCountThreads) void continuous_count_kernel(const i
     const uint32_t nrep = 1u << nrep_log2;
     const uint32_t rep = tid & (nrep - 1);
     const uint32_t words = E << nrep_log2;
-    uint32_t* ticket = ws;
-    uint32_t* partials = ws + kTicketWords;
 
     for (uint32_t i = tid; i < words; i += kCountThreads) bins[i] = 0;
     __syncthreads();
@@ -129,32 +126,32 @@ __global__ __launch_bounds__(kCountThreads) void continuous_count_kernel(const i
         if (e < E && sub == 0) my_row[e] = s;
     }
 
-    // ticket: the last workgroup to arrive owns the final sum
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        const uint32_t t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        s_is_last = (t == gridDim.x - 1) ? 1u : 0u;
-    }
-    __syncthreads();
-    if (!s_is_last) return;
-    __threadfence();
+}
 
-    uint32_t tpb2 = floor_pow2(kCountThreads / E ? kCountThreads / E : 1);
-    if (tpb2 > (uint32_t)kWave) tpb2 = kWave;
-    const uint32_t bpp2 = kCountThreads / tpb2;
-    const uint32_t sub2 = tid & (tpb2 - 1);
-    for (uint32_t e0 = 0; e0 < E; e0 += bpp2) {
-        const uint32_t e = e0 + tid / tpb2;
-        uint32_t s = 0;
-        if (e < E) {
-            for (uint32_t b = sub2; b < gridDim.x; b += tpb2)
-                s += __hip_atomic_load(&partials[(uint64_t)b * E + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        for (uint32_t d = tpb2 >> 1; d > 0; d >>= 1) s += __shfl_xor(s, d, kWave);
-        if (e < E && sub2 == 0) out[e] = s;
+// out[e] = sum over the `rows` workgroup histograms; one workgroup per 64 bins, 16 lanes-groups share the rows
+constexpr int kReduceThreads = 1024;
+constexpr int kReduceBins = 64;
+
+__global__ __launch_bounds__(kReduceThreads) void count_reduce_kernel(const uint32_t* __restrict__ partials,
+                                                                      uint32_t rows, uint32_t E,
+                                                                      uint32_t* __restrict__ out) {
+    __shared__ uint32_t s_sum[kReduceThreads];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t e = blockIdx.x * kReduceBins + (tid % kReduceBins);
+    const uint32_t part = tid / kReduceBins;
+    constexpr uint32_t parts = kReduceThreads / kReduceBins;
+    uint32_t s = 0;
+    if (e < E) {
+        for (uint32_t b = part; b < rows; b += parts) s += partials[(uint64_t)b * E + e];
     }
-    if (tid == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_sum[tid] = s;
+    __syncthreads();
+    if (tid < kReduceBins && e < E) {
+        uint32_t total = 0;
+#pragma unroll
+        for (uint32_t p = 0; p < parts; ++p) total += s_sum[p * kReduceBins + tid];
+        out[e] = total;
+    }
 }
 
 // ---- index construction ---------------------------------------------------------------------
@@ -321,7 +318,7 @@ int64_t fma_continuous_count_workspace_bytes(int64_t n, int64_t E) {
     // independent of id width and device: sized for the largest grid any call may use
     const int cus = fmahip::num_compute_units();
     const int64_t max_grid = (int64_t)(cus > 0 ? cus : 256) * 2;
-    return (int64_t)fmahip::kTicketWords * 4 + max_grid * E * 4;
+    return max_grid * E * 4;
 }
 
 int fma_continuous_count(const void* ids, int id_bytes, int64_t n, uint32_t* counts, int64_t E, void* workspace,
@@ -344,7 +341,7 @@ int fma_continuous_count(const void* ids, int id_bytes, int64_t n, uint32_t* cou
 
     const int cus = num_compute_units();
     const CountPlan plan = plan_count((uint64_t)n, id_bytes, cus);
-    const int64_t need = (int64_t)kTicketWords * 4 + (int64_t)plan.grid * E * 4;
+    const int64_t need = (int64_t)plan.grid * E * 4;
     FMA_REQUIRE(workspace_bytes >= need, FMA_ERR_WORKSPACE_TOO_SMALL,
                 "continuous_count: workspace of %lld bytes is smaller than the %lld needed", (long long)workspace_bytes,
                 (long long)need);
@@ -356,14 +353,16 @@ int fma_continuous_count(const void* ids, int id_bytes, int64_t n, uint32_t* cou
     hipStream_t st = (hipStream_t)stream;
     if (id_bytes == 4) {
         hipLaunchKernelGGL(continuous_count_kernel<int32_t>, dim3(plan.grid), dim3(kCountThreads), lds_bytes, st,
-                           (const int32_t*)ids, (uint64_t)n, (uint32_t)E, nrep_log2, plan.chunk, (uint32_t*)workspace,
-                           counts);
+                           (const int32_t*)ids, (uint64_t)n, (uint32_t)E, nrep_log2, plan.chunk, (uint32_t*)workspace);
     } else {
         hipLaunchKernelGGL(continuous_count_kernel<int64_t>, dim3(plan.grid), dim3(kCountThreads), lds_bytes, st,
-                           (const int64_t*)ids, (uint64_t)n, (uint32_t)E, nrep_log2, plan.chunk, (uint32_t*)workspace,
-                           counts);
+                           (const int64_t*)ids, (uint64_t)n, (uint32_t)E, nrep_log2, plan.chunk, (uint32_t*)workspace);
     }
-    return launch_status("continuous_count");
+    int rc = launch_status("continuous_count");
+    if (rc) return rc;
+    hipLaunchKernelGGL(count_reduce_kernel, dim3((uint32_t)((E + kReduceBins - 1) / kReduceBins)), dim3(kReduceThreads),
+                       0, st, (const uint32_t*)workspace, plan.grid, (uint32_t)E, counts);
+    return launch_status("continuous_count(reduce)");
 }
 
 int64_t fma_moe_build_index_workspace_bytes(int64_t R, int64_t E) {

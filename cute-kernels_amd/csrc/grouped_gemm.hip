@@ -6,16 +6,19 @@
 //    prefix and packed element offsets of every group) in LDS from the device-side M/N/K arrays, then walks
 //    256x256 output tiles. Tile ids are handed out so that the 32 workgroups of one XCD (workgroup id mod 8)
 //    always hold a compact 8x4 block of tiles of the same group: they share A and B panels in that XCD's L2.
-//  * K is consumed in steps of 64 through two LDS stages of 2 x 32 KB. Both operand tiles live in LDS as
-//    [row][64 k] (k contiguous, 128-byte rows) whatever their layout in memory:
-//      - an operand whose reduction dimension is contiguous in memory goes global -> LDS directly
-//        (global_load_lds_dwordx4, 1 KB per wavefront instruction, no staging registers);
-//      - an operand stored with the reduction dimension as the row index is loaded as 8x8 blocks (eight
-//        16-byte loads per lane), transposed in registers with byte permutes and written as 16-byte rows.
-//    Row r / 16-byte chunk c of a tile sits at  phys_row(r)*128 + ((c ^ (r & 7)) << 4)  where phys_row rotates
-//    the low four row bits left by one. With it the MFMA operand reads (32 consecutive rows, one chunk), the
-//    direct loads (whole 128-byte rows) and the transposed stores (rows 8 apart, 8 chunks) each touch every
-//    LDS bank group once.
+//  * K is consumed in steps of 64 through two LDS stages of 2 x 32 KB. Every operand tile goes global -> LDS directly
+//    (global_load_lds_dwordx4, 1 KB per wavefront instruction, no staging registers), in one of two layouts:
+//      - an operand whose reduction dimension is contiguous in memory is kept as [row][64 k] (128-byte rows); row r,
+//        16-byte chunk c sits at phys_row(r)*128 + ((c ^ (r & 7)) << 4), phys_row rotating the low four row bits
+//        left by one, and an MFMA fragment (32 rows x 16 k) is one ds_read_b128 per lane;
+//      - an operand stored with the reduction dimension as the row index is kept as it is in memory, [64 k][256 out]
+//        (512-byte rows), chunk c of row k at k*512 + ((c ^ (4*(k & 3))) << 4), and a fragment is two
+//        ds_read_b64_tr_b16 per lane: the transposing LDS read hands lane i of a 16-lane group the four k values of
+//        out column i when lane j of the group addresses row j/4, columns 4*(j%4)..+3.
+//    Both swizzles are applied on the source side of the direct load (which lane fetches which chunk) and make the
+//    fragment reads touch every LDS bank once per pass.
+//  * Fragments are double buffered in registers and the workgroup barrier of a K step sits before the MFMAs of its
+//    last k slice, so the LDS and barrier latencies are covered by matrix work.
 //  * The MFMA is issued with B as the first operand, so a lane ends up holding four consecutive output
 //    columns of one output row and stores them as one 8-byte word.
 #include "common.h"
@@ -27,13 +30,17 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
 constexpr int BM = 256;
 constexpr int BN = 256;
 constexpr int BK = 64;
-constexpr int kRowBytes = BK * 2;           // 128
-constexpr int kTileBytes = BM * kRowBytes;  // 32 KB per operand per stage
+constexpr int kRowBytes = BK * 2;           // 128: row of a [row][64 k] tile
+constexpr int kTRowBytes = BM * 2;          // 512: row of a [64 k][256 out] tile
+constexpr int kTileBytes = BM * kRowBytes;  // 32 KB per operand per stage, either layout
 constexpr int kGroupM = 8;                  // m-tiles that share one column sweep of the tile order
 constexpr int kXcds = 8;
 
@@ -51,7 +58,6 @@ struct GemmArgs {
     uint32_t E;
     uint32_t const_n;
     uint32_t const_k;
-    uint32_t inter;  // swiglu only: I (N = 2*I)
     float alpha;
 };
 
@@ -59,8 +65,17 @@ __device__ __forceinline__ uint32_t phys_row(uint32_t r) { return (r & ~15u) | (
 __device__ __forceinline__ uint32_t logical_row(uint32_t pr) {
     return (pr & ~15u) | ((pr & 15u) >> 1) | ((pr & 1u) << 3);
 }
-__device__ __forceinline__ uint32_t lds_off(uint32_t r, uint32_t chunk) {
+// [row][64 k] tile: byte offset of 16-byte chunk `chunk` of row r
+__device__ __forceinline__ uint32_t kc_off(uint32_t r, uint32_t chunk) {
     return phys_row(r) * kRowBytes + ((chunk ^ (r & 7u)) << 4);
+}
+// [64 k][256 out] tile: byte offset, for k slice 0, of the first transposing read of the fragment that starts at out
+// row r0 (a multiple of 32). Slice ks adds 16 rows, the second read of a fragment (k + 4) adds 4 rows.
+__device__ __forceinline__ uint32_t mc_frag_off(uint32_t r0, uint32_t lane) {
+    const uint32_t g = lane >> 4, j = lane & 15u;
+    const uint32_t q = j & 3u, kr = j >> 2;
+    const uint32_t chunk = (r0 >> 3) + 2u * (g & 1u) + (q >> 1);
+    return (8u * (g >> 1) + kr) * kTRowBytes + ((chunk ^ (4u * kr)) << 4) + (q & 1u) * 8u;
 }
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
@@ -74,13 +89,13 @@ __device__ __forceinline__ float round_bf16(float x) {
     return (float)b;
 }
 
-// ---- loader for an operand whose reduction dimension is contiguous in memory ---------------------
-// The tile has 256 rows; a wavefront instruction moves 8 physical rows (1 KB). NI instructions per wavefront.
+// ---- direct global -> LDS loader, operand with the reduction dimension contiguous: tile [256 rows][64 k] ------
+// A wavefront instruction moves 8 physical rows (1 KB); NI instructions per wavefront and K step.
 template <int NW>
-struct DirectLoader {
+struct LoaderK {
     static constexpr int NI = 32 / NW;
     const uint16_t* gp[NI];  // this lane's source of each instruction at k0 = 0
-    uint32_t chunk;          // this lane's logical 16-byte chunk (same for every instruction)
+    uint32_t chunk;          // this lane's logical 16-byte chunk (the same for every instruction: NW is even)
     uint32_t kdim;
     uint32_t wave;
 
@@ -88,6 +103,7 @@ struct DirectLoader {
     template <typename RowFn>
     __device__ __forceinline__ void setup(const uint16_t* base, uint64_t ld, uint32_t kdim_, uint32_t wave_,
                                           uint32_t lane, RowFn row_of) {
+        static_assert(NW % 2 == 0, "chunk is per lane only for an even number of wavefronts");
         kdim = kdim_;
         wave = wave_;
 #pragma unroll
@@ -121,60 +137,78 @@ struct DirectLoader {
     }
 };
 
-// ---- loader for an operand stored [reduction][out] (out contiguous): 8x8 blocks, register transpose ----
-struct TransposeLoader {
-    const uint16_t* gp;  // base + (kb*8)*ld + out chunk of this lane
+// ---- direct global -> LDS loader, operand stored [reduction][out] (out contiguous): tile [64 k][256 out] -------
+// A wavefront instruction moves two k rows (2 x 512 B).
+template <int NW>
+struct LoaderT {
+    static constexpr int NI = 32 / NW;
+    const uint16_t* gp[NI];  // this lane's source of each instruction at k0 = 0
     uint64_t ld;
-    uint32_t kb, ob;  // 8-row block of the reduction dim (0..7), 8-column block of the out dim (0..31)
     uint32_t kdim;
-    uint4 st[8];
+    uint32_t wave;
+    uint32_t khalf;  // which of the two rows of an instruction this lane loads
 
     __device__ __forceinline__ void setup(const uint16_t* base, uint64_t ld_, uint32_t kdim_, uint32_t out0,
-                                          uint32_t out_total, uint32_t tl) {
-        const uint32_t lane = tl & 63u;
-        kb = lane & 7u;
-        ob = (tl >> 6) * 8u + (lane >> 3);
+                                          uint32_t out_total, uint32_t wave_, uint32_t lane) {
         ld = ld_;
         kdim = kdim_;
-        uint32_t oc = out0 + ob * 8u;
-        if (oc + 8u > out_total) oc = out_total - 8u;  // columns past the edge: results are never stored
-        gp = base + (uint64_t)(kb * 8u) * ld_ + oc;
-    }
-
-    __device__ __forceinline__ void load(uint32_t k0) {
-        const uint16_t* p = gp + (uint64_t)k0 * ld;
-        if (k0 + BK <= kdim) {
+        wave = wave_;
+        khalf = lane >> 5;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) st[j] = *reinterpret_cast<const uint4*>(p + (uint64_t)j * ld);
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                if (k0 + kb * 8u + j < kdim)
-                    st[j] = *reinterpret_cast<const uint4*>(p + (uint64_t)j * ld);
-                else
-                    st[j] = make_uint4(0, 0, 0, 0);
-            }
+        for (int i = 0; i < NI; ++i) {
+            const uint32_t krow = (uint32_t)(i * NW + wave_) * 2u + khalf;
+            const uint32_t chunk = (lane & 31u) ^ (4u * (krow & 3u));
+            uint32_t col = out0 + chunk * 8u;
+            if (col + 8u > out_total) col = out_total - 8u;  // columns past the edge: results are never stored
+            gp[i] = base + (uint64_t)krow * ld_ + col;
         }
     }
 
-    __device__ __forceinline__ void store(uint8_t* tile) const {
-        // st[j] holds out columns 0..7 of reduction row j; column c must become 8 reduction values
-        const uint32_t* w = reinterpret_cast<const uint32_t*>(st);  // w[j*4 + d]: columns 2d, 2d+1 of row j
+    __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0, uint32_t lane) const {
+        const uint64_t adv = (uint64_t)k0 * ld;
+        if (k0 + BK <= kdim) {
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            uint32_t lo[4], hi[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const uint32_t even = w[(2 * q) * 4 + d];
-                const uint32_t odd = w[(2 * q + 1) * 4 + d];
-                lo[q] = __builtin_amdgcn_perm(odd, even, 0x05040100u);  // column 2d  : rows 2q, 2q+1
-                hi[q] = __builtin_amdgcn_perm(odd, even, 0x07060302u);  // column 2d+1: rows 2q, 2q+1
+            for (int i = 0; i < NI; ++i) {
+                __builtin_amdgcn_global_load_lds(gp[i] + adv, (lds_void*)(tile + (i * NW + wave) * 1024), 16, 0, 0);
             }
-            *reinterpret_cast<uint4*>(tile + lds_off(ob * 8u + 2 * d, kb)) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-            *reinterpret_cast<uint4*>(tile + lds_off(ob * 8u + 2 * d + 1, kb)) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        } else {
+            // last, partial K step: rows past the end of the reduction are zero-filled instead of loaded
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                uint8_t* dst = tile + (i * NW + wave) * 1024;
+                if (k0 + (uint32_t)(i * NW + wave) * 2u + khalf < kdim) {
+                    __builtin_amdgcn_global_load_lds(gp[i] + adv, (lds_void*)dst, 16, 0, 0);
+                } else {
+                    *reinterpret_cast<uint4*>(dst + lane * 16u) = make_uint4(0, 0, 0, 0);
+                }
+            }
         }
     }
 };
+
+__device__ __forceinline__ bf16x8 read_kc_frag(const uint8_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+
+__device__ __forceinline__ bf16x8 read_tr_frag(const uint8_t* p) {
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p + 4 * kTRowBytes));
+    const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, v);
+}
+
+// Scheduling hint for one k slice: MFMAS matrix instructions with READS LDS reads spread evenly between them.
+template <int R, int MFMAS, int READS>
+__device__ __forceinline__ void interleave_mfma_lds() {
+    constexpr int kPairs = READS < MFMAS ? READS : MFMAS;
+    constexpr int kPer = READS / kPairs;           // LDS reads after each of the first kPairs MFMAs
+    constexpr int kExtra = READS - kPairs * kPer;  // the first kExtra of them get one more
+    if constexpr (R < kPairs) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, kPer + (R < kExtra ? 1 : 0), 0);
+        interleave_mfma_lds<R + 1, MFMAS, READS>();
+    } else if constexpr (MFMAS - kPairs > 0) {
+        __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - kPairs, 0);
+    }
+}
 
 // Slow, layout-agnostic path for a group whose contiguous dimensions are not multiples of 8 elements.
 template <bool A_KC, bool B_KC>
@@ -203,7 +237,6 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     constexpr int FM = WM / 32;
     constexpr int FN = WN / 32;
     static_assert(EPI == EPI_PLAIN || (A_KC && B_KC), "the SwiGLU epilogue exists for the NT layout only");
-    static_assert(NT == 256 || NT == 512, "the transpose loader is written for 256-thread groups");
 
     // one array per stage and operand: distinct LDS objects let the compiler see that a direct-to-LDS load
     // into one stage cannot alias the fragment reads of the other, so it does not wait for the load first
@@ -272,12 +305,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     __syncthreads();
     const uint32_t total_tiles = s_tile_start[E];
 
-    // per-lane LDS read offsets of an MFMA operand fragment whose first row is a multiple of 32
-    uint32_t frag_off[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) frag_off[ks] = lds_off(lane & 31u, (uint32_t)ks * 2u + (lane >> 5));
-    const uint32_t a_wave_off = wm * WM * kRowBytes;
-    // first LDS row of B fragment j of this wavefront
+    // first tile row of B fragment j of this wavefront
     auto b_frag_row = [&](int j) -> uint32_t {
         if constexpr (EPI == EPI_SWIGLU) {
             return j < FN / 2 ? wn * (WN / 2) + j * 32 : BN / 2 + wn * (WN / 2) + (j - FN / 2) * 32;
@@ -285,6 +313,22 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             return wn * WN + j * 32;
         }
     };
+    // per-lane LDS byte offsets of this wavefront's fragments for k slice 0 (slice ks adds a constant)
+    uint32_t a_off[FM], b_off[FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        const uint32_t r0 = wm * WM + i * 32;
+        a_off[i] = A_KC ? r0 * kRowBytes : mc_frag_off(r0, lane);
+    }
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+        const uint32_t r0 = b_frag_row(j);
+        b_off[j] = B_KC ? r0 * kRowBytes : mc_frag_off(r0, lane);
+    }
+    // [row][64 k] tiles: offset of this lane's row and chunk inside a 32-row fragment, per k slice
+    uint32_t kc_slice[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) kc_slice[ks] = kc_off(lane & 31u, (uint32_t)ks * 2u + (lane >> 5));
 
     // workgroup id -> position in the round of gridDim.x tiles: workgroups of one XCD take 32 neighbours
     const uint32_t grid = gridDim.x;
@@ -318,8 +362,11 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         const uint16_t* Be = args.B + s_off_b[e];
         const uint64_t off_d = s_off_d[e];
 
-        bool fast = (Ke % 8u == 0) && (Ne % 8u == 0) && (s_off_a[e] % 8u == 0) && (s_off_b[e] % 8u == 0) &&
-                    (off_d % 8u == 0);
+        // 16-byte accesses need: every contiguous dimension a multiple of 8 elements (K for an operand whose
+        // reduction dim is contiguous, M / N for one stored reduction-major, N for the output rows) and packed
+        // group bases that stayed multiples of 8. A ragged reduction length is fine for reduction-major operands.
+        bool fast = (Ne % 8u == 0) && (s_off_a[e] % 8u == 0) && (s_off_b[e] % 8u == 0) && (off_d % 8u == 0);
+        if (A_KC || B_KC) fast = fast && (Ke % 8u == 0);
         if (!A_KC) fast = fast && (Me % 8u == 0);
         if (EPI == EPI_SWIGLU) fast = fast && (n_span % 8u == 0);
 
@@ -333,20 +380,18 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         }
 
         // ---- loaders ----
-        DirectLoader<NW> dl_a, dl_b;
-        TransposeLoader tl_a, tl_b;
-        const bool mc_a_on = !A_KC && (NT == 256 || wave < 4);
-        const bool mc_b_on = !B_KC && (NT == 256 || (A_KC ? wave < 4 : wave >= 4));
+        LoaderK<NW> lk_a, lk_b;
+        LoaderT<NW> lt_a, lt_b;
         if constexpr (A_KC) {
-            dl_a.setup(Ae, Ke, Ke, wave, lane, [&](uint32_t r) {
+            lk_a.setup(Ae, Ke, Ke, wave, lane, [&](uint32_t r) {
                 const uint32_t m = m0 + r;
                 return m < Me ? m : Me - 1;
             });
         } else {
-            if (mc_a_on) tl_a.setup(Ae, Me, Ke, m0, Me, tid & 255u);
+            lt_a.setup(Ae, Me, Ke, m0, Me, wave, lane);
         }
         if constexpr (B_KC) {
-            dl_b.setup(Be, Ke, Ke, wave, lane, [&](uint32_t r) {
+            lk_b.setup(Be, Ke, Ke, wave, lane, [&](uint32_t r) {
                 uint32_t n;
                 if constexpr (EPI == EPI_SWIGLU) {
                     // rows 0..127: "up" rows n0 + r; rows 128..255: "gate" rows I + n0 + (r - 128)
@@ -359,22 +404,13 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                 return n;
             });
         } else {
-            if (mc_b_on) tl_b.setup(Be, Ne, Ke, n0, Ne, tid & 255u);
+            lt_b.setup(Be, Ne, Ke, n0, Ne, wave, lane);
         }
-
         auto issue = [&](int stage, uint32_t k0) {
-            if constexpr (A_KC) dl_a.issue(stage ? s_a1 : s_a0, k0, lane);
-            else if (mc_a_on) tl_a.load(k0);
-            if constexpr (B_KC) dl_b.issue(stage ? s_b1 : s_b0, k0, lane);
-            else if (mc_b_on) tl_b.load(k0);
-        };
-        auto finish = [&](int stage) {
-            if constexpr (!A_KC) {
-                if (mc_a_on) tl_a.store(stage ? s_a1 : s_a0);
-            }
-            if constexpr (!B_KC) {
-                if (mc_b_on) tl_b.store(stage ? s_b1 : s_b0);
-            }
+            if constexpr (A_KC) lk_a.issue(stage ? s_a1 : s_a0, k0, lane);
+            else lt_a.issue(stage ? s_a1 : s_a0, k0, lane);
+            if constexpr (B_KC) lk_b.issue(stage ? s_b1 : s_b0, k0, lane);
+            else lt_b.issue(stage ? s_b1 : s_b0, k0, lane);
         };
 
         f32x16 acc[FM][FN];
@@ -385,44 +421,64 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
 #pragma unroll
                 for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.0f;
 
-        auto compute = [&](int stage) {
-            const uint8_t* ta = (stage ? s_a1 : s_a0) + a_wave_off;
+        // MFMA operand fragments of one 16-wide k slice, double buffered in registers
+        bf16x8 fa[2][FM], fb[2][FN];
+        auto load_frags = [&](int stage, int ks, int buf) {
+            const uint8_t* ta = stage ? s_a1 : s_a0;
             const uint8_t* tb = stage ? s_b1 : s_b0;
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                bf16x8 a[FM], b[FN];
+            for (int i = 0; i < FM; ++i) {
+                if constexpr (A_KC) fa[buf][i] = read_kc_frag(ta + a_off[i] + kc_slice[ks]);
+                else fa[buf][i] = read_tr_frag(ta + a_off[i] + ks * 16 * kTRowBytes);
+            }
 #pragma unroll
-                for (int i = 0; i < FM; ++i)
-                    a[i] = *reinterpret_cast<const bf16x8*>(ta + i * 32 * kRowBytes + frag_off[ks]);
-#pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    b[j] = *reinterpret_cast<const bf16x8*>(tb + b_frag_row(j) * kRowBytes + frag_off[ks]);
-#pragma unroll
-                for (int i = 0; i < FM; ++i)
-#pragma unroll
-                    for (int j = 0; j < FN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < FN; ++j) {
+                if constexpr (B_KC) fb[buf][j] = read_kc_frag(tb + b_off[j] + kc_slice[ks]);
+                else fb[buf][j] = read_tr_frag(tb + b_off[j] + ks * 16 * kTRowBytes);
             }
         };
+        auto mma = [&](int buf) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+        };
+        // ask the scheduler to alternate the MFMAs of one slice with the LDS reads of the next
+        constexpr int kReads = (A_KC ? FM : 2 * FM) + (B_KC ? FN : 2 * FN);
+        auto interleave_reads = [&]() { interleave_mfma_lds<0, FM * FN, kReads>(); };
 
-        // ---- main loop over K: stage s is computed while stage s^1 is being filled ----
+        // ---- main loop over K ----
+        // Step kt computes from stage kt&1. The workgroup barrier of a step sits between the LDS reads of its last
+        // k slice and the MFMAs of that slice: once it is passed, the stage just read is free (the loads of step kt+2
+        // are issued into it) and the other stage is complete (its first fragments are fetched), and both overlap
+        // with the MFMAs still to be issued, so the matrix pipe has work while the barrier's latencies play out.
         const uint32_t KT = (Ke + BK - 1) / BK;
+        auto step = [&](int stage, uint32_t kt) {
+            load_frags(stage, 1, 1);
+            mma(0);
+            interleave_reads();
+            load_frags(stage, 2, 0);
+            mma(1);
+            interleave_reads();
+            load_frags(stage, 3, 1);
+            mma(0);
+            interleave_reads();
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (kt + 1 < KT) load_frags(stage ^ 1, 0, 0);
+            mma(1);
+            if (kt + 2 < KT) issue(stage, (kt + 2) * BK);
+        };
         if (KT > 0) {
             issue(0, 0);
-            finish(0);
-        }
-        for (uint32_t kt = 0; kt < KT; kt += 2) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (KT > 1) issue(1, BK);
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __syncthreads();
-            if (kt + 1 < KT) issue(1, (kt + 1) * BK);
-            compute(0);
-            if (kt + 1 < KT) {
-                finish(1);
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                __syncthreads();
-                if (kt + 2 < KT) issue(0, (kt + 2) * BK);
-                compute(1);
-                if (kt + 2 < KT) finish(0);
+            load_frags(0, 0, 0);
+            for (uint32_t kt = 0; kt < KT; kt += 2) {
+                step(0, kt);
+                if (kt + 1 < KT) step(1, kt + 1);
             }
         }
 
@@ -572,7 +628,6 @@ int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, co
     args.E = (uint32_t)E;
     args.const_n = (uint32_t)(2 * I);
     args.const_k = (uint32_t)K;
-    args.inter = (uint32_t)I;
     args.alpha = 1.0f;
     return launch<2, 4, true, true, EPI_SWIGLU>(args, (hipStream_t)stream);
 }

@@ -8,20 +8,6 @@ from ... import _lib
 from ...constants import LIBRARY_NAME
 
 
-# One workspace per device, zeroed once: the kernel keeps its 256-byte ticket area zero between launches. Launches
-# that share it must be ordered on one stream; concurrent streams would need a workspace each.
-_WORKSPACES: dict[int, torch.Tensor] = {}
-
-
-def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    index = device.index if device.index is not None else torch.cuda.current_device()
-    ws = _WORKSPACES.get(index)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _WORKSPACES[index] = ws
-    return ws
-
-
 @custom_op(f"{LIBRARY_NAME}::continuous_count_cuda", mutates_args={"output"})
 def continuous_count_cuda(
     x: torch.Tensor, output: torch.Tensor, E: int, THREAD_BLOCK_CLUSTER_SIZE: int, BLOCK_SIZE: int
@@ -35,7 +21,8 @@ def continuous_count_cuda(
     lib = _lib.load()
     n = x.numel()
     with torch.cuda.device(x.device):
-        ws = _workspace(x.device, lib.fma_continuous_count_workspace_bytes(n, E))
+        # per-workgroup partial histograms; uninitialised memory from the caching allocator, owned by this call
+        ws = torch.empty(max(lib.fma_continuous_count_workspace_bytes(n, E), 4), dtype=torch.uint8, device=x.device)
         rc = lib.fma_continuous_count(
             x.data_ptr(), x.element_size(), n, output.data_ptr(), E, ws.data_ptr(), ws.numel(),
             _lib.current_stream(x.device),

@@ -58,9 +58,8 @@ int fma_num_compute_units(void);
 
 /* ---- continuous_count ------------------------------------------------------------------- */
 
-/* Bytes of workspace fma_continuous_count needs for n ids and E bins. The first 256 bytes must be zero
- * before the FIRST call that uses the buffer; every call leaves them zero again, so one buffer zeroed
- * once can be reused by stream-ordered calls (calls that overlap in time need separate buffers). */
+/* Bytes of workspace fma_continuous_count needs for n ids and E bins (one partial histogram per workgroup). The
+ * buffer needs no initialisation; calls that overlap in time need separate buffers. */
 int64_t fma_continuous_count_workspace_bytes(int64_t n, int64_t E);
 
 /* counts[v] = #{ i < n : ids[i] == v } for v in [0, E); ids outside [0, E) are not counted.
