@@ -39,6 +39,8 @@ def parse_args():
     p.add_argument("--workload", default="mixtral", choices=list(WORKLOADS))
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     p.add_argument("--no-kernels", action="store_true", help="skip the per-kernel measurements")
+    p.add_argument("--no-layer", action="store_true", help="skip the whole-layer timing (for short profiler runs)")
+    p.add_argument("--only", default="", help="comma-separated substrings: measure only the kernels whose name matches")
     return p.parse_args()
 
 
@@ -110,6 +112,8 @@ def main():
         y.backward(dy)
         return y
 
+    if args.no_layer:
+        args.steps = args.warmup = 0
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -117,8 +121,8 @@ def main():
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
+    elapsed = max(time.perf_counter() - t0, 1e-9) if args.steps else float("inf")
+    ms_per_step = elapsed * 1e3 / max(args.steps, 1)
     tokens_per_s = T * args.steps / elapsed
     gemm_flops_step = 3 * 2.0 * R * (2 * I * H + I * H)  # fwd + dgrad + wgrad of both projections
 
@@ -184,67 +188,75 @@ def main():
         ok(lib.fma_gather_rows(x.data_ptr(), perm.data_ptr(), R, H, k, xg.data_ptr(), BF16, stream))
         iters = max(5, args.steps)
 
-        def mfma(name, flops, t):
+        only = [w for w in args.only.split(",") if w]
+
+        def want(name):
+            return not only or any(w in name for w in only)
+
+        def mfma(name, flops, fn, n=iters):
+            if not want(name):
+                return
+            t = time_gpu(fn, n, blocker=blocker)
             tf = flops / (t[0] * 1e-3) / 1e12
             kernels[name] = {"ms": t[0], "ms_mean": t[1], "bound": "mfma", "achieved": tf, "peak": PEAK_BF16_TFLOPS,
                              "unit": "TFLOP/s", "frac": tf / PEAK_BF16_TFLOPS, "flop": flops}
 
-        def hbm(name, nbytes, t):
+        def hbm(name, nbytes, fn, n=20, warmup=3):
+            if not want(name):
+                return
+            t = time_gpu(fn, n, warmup=warmup, blocker=blocker)
             gbs = nbytes / (t[0] * 1e-3) / 1e9
             kernels[name] = {"ms": t[0], "ms_mean": t[1], "bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS,
                              "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "bytes": nbytes}
 
-        t = time_gpu(lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), h.data_ptr(), a.data_ptr(),
-                                                              counts.data_ptr(), E, I, H, BF16, stream)), iters, blocker=blocker)
-        mfma("up_projection_swiglu_fwd(NT)", 2.0 * R * 2 * I * H, t)
-        mfma("down_projection_fwd(NT)", 2.0 * R * I * H,
-             time_gpu(lambda i: gemm(a, w2, o, counts, N_pj, K_pj, 0, 1), iters, blocker=blocker))
-        mfma("down_projection_dgrad(NN)", 2.0 * R * I * H,
-             time_gpu(lambda i: gemm(d_o, w2, da, counts, K_pj, N_pj, 0, 0), iters, blocker=blocker))
-        mfma("down_projection_wgrad(TN)", 2.0 * R * I * H,
-             time_gpu(lambda i: gemm(d_o, a, dw2, N_pj, K_pj, counts, 1, 0), iters, blocker=blocker))
-        mfma("up_projection_dgrad(NN)", 2.0 * R * 2 * I * H,
-             time_gpu(lambda i: gemm(dh, w1, dxg, counts, K_fc, N_fc, 0, 0), iters, blocker=blocker))
-        mfma("up_projection_wgrad(TN)", 2.0 * R * 2 * I * H,
-             time_gpu(lambda i: gemm(dh, xg, dw1, N_fc, K_fc, counts, 1, 0), iters, blocker=blocker))
+        mfma("up_projection_swiglu_fwd(NT)", 2.0 * R * 2 * I * H,
+             lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), h.data_ptr(), a.data_ptr(),
+                                                      counts.data_ptr(), E, I, H, BF16, stream)))
+        mfma("down_projection_fwd(NT)", 2.0 * R * I * H, lambda i: gemm(a, w2, o, counts, N_pj, K_pj, 0, 1))
+        mfma("down_projection_dgrad(NN)", 2.0 * R * I * H, lambda i: gemm(d_o, w2, da, counts, K_pj, N_pj, 0, 0))
+        mfma("down_projection_wgrad(TN)", 2.0 * R * I * H, lambda i: gemm(d_o, a, dw2, N_pj, K_pj, counts, 1, 0))
+        mfma("up_projection_dgrad(NN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, w1, dxg, counts, K_fc, N_fc, 0, 0))
+        mfma("up_projection_wgrad(TN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, xg, dw1, N_fc, K_fc, counts, 1, 0))
 
         # row kernels: algorithmic bytes = each distinct input row once + each output row once + index / gate words
         hbm("gather_rows", T * H * s + R * H * s + R * 4,
-            time_gpu(lambda i: ok(lib.fma_gather_rows(x.data_ptr(), perm.data_ptr(), R, H, k, xg.data_ptr(), BF16, stream)),
-                     20, blocker=blocker))
+            lambda i: ok(lib.fma_gather_rows(x.data_ptr(), perm.data_ptr(), R, H, k, xg.data_ptr(), BF16, stream)))
         hbm("combine", R * H * s + R * (4 + s) + T * H * s,
-            time_gpu(lambda i: ok(lib.fma_combine(o.data_ptr(), inv.data_ptr(), weights_d.data_ptr(), T, k, H, y.data_ptr(),
-                                                  BF16, stream)), 20, blocker=blocker))
+            lambda i: ok(lib.fma_combine(o.data_ptr(), inv.data_ptr(), weights_d.data_ptr(), T, k, H, y.data_ptr(), BF16,
+                                         stream)))
         hbm("combine_backward", T * H * s + 2 * R * H * s + R * (4 + 2 * s),
-            time_gpu(lambda i: ok(lib.fma_combine_bwd(dy.data_ptr(), o.data_ptr(), inv.data_ptr(), weights_d.data_ptr(), T, k,
-                                                      H, d_o.data_ptr(), dgates.data_ptr(), BF16, stream)), 20, blocker=blocker))
+            lambda i: ok(lib.fma_combine_bwd(dy.data_ptr(), o.data_ptr(), inv.data_ptr(), weights_d.data_ptr(), T, k, H,
+                                             d_o.data_ptr(), dgates.data_ptr(), BF16, stream)))
         es = 2 * I  # row stride of the packed pre-activation and of its gradient
         hbm("swiglu_backward", 5 * R * I * s,
-            time_gpu(lambda i: ok(lib.fma_swiglu_backward(h.data_ptr() + I * s, h.data_ptr(), da.data_ptr(),
-                                                          dh.data_ptr() + I * s, dh.data_ptr(), R, I, es, es, I, es, es,
-                                                          BF16, stream)), 10, blocker=blocker))
-        ws_idx = torch.empty(max(lib.fma_moe_build_index_workspace_bytes(R, E), 4) // 4, dtype=torch.int32, device=dev)
-        t = time_gpu(lambda i: ok(lib.fma_moe_build_index(selected_d.data_ptr(), 8, R, E, counts.data_ptr(), offsets.data_ptr(),
-                                                          perm.data_ptr(), eid.data_ptr(), inv.data_ptr(), ws_idx.data_ptr(),
-                                                          ws_idx.numel() * 4, stream)), 20, blocker=blocker)
-        kernels["build_routing_index(3 launches)"] = {"ms": t[0], "ms_mean": t[1]}
+            lambda i: ok(lib.fma_swiglu_backward(h.data_ptr() + I * s, h.data_ptr(), da.data_ptr(), dh.data_ptr() + I * s,
+                                                 dh.data_ptr(), R, I, es, es, I, es, es, BF16, stream)), n=10)
+        if want("build_routing_index"):
+            ws_idx = torch.empty(max(lib.fma_moe_build_index_workspace_bytes(R, E), 4) // 4, dtype=torch.int32, device=dev)
+            t = time_gpu(lambda i: ok(lib.fma_moe_build_index(selected_d.data_ptr(), 8, R, E, counts.data_ptr(),
+                                                              offsets.data_ptr(), perm.data_ptr(), eid.data_ptr(),
+                                                              inv.data_ptr(), ws_idx.data_ptr(), ws_idx.numel() * 4, stream)),
+                         20, blocker=blocker)
+            kernels["build_routing_index(3 launches)"] = {"ms": t[0], "ms_mean": t[1]}
 
         # continuous_count on 16 Mi int32 ids in [0, 64): five distinct 64 MiB buffers (320 MiB > the 256 MiB
-        # last-level cache) so that every launch reads from HBM
+        # last-level cache) so that every launch reads from HBM. The figure covers both launches of one call
+        # (count + reduce).
         n_ids, bins = 16 << 20, 64
         ws_cnt = torch.empty(lib.fma_continuous_count_workspace_bytes(n_ids, bins), dtype=torch.uint8, device=dev)
         out_cnt = torch.empty(bins, dtype=torch.uint32, device=dev)
         for kind in ("uniform", "zipf"):
+            if not want(f"continuous_count_16Mi_{kind}"):
+                continue
             ids = [torch.from_numpy(O.make_ids(n_ids, bins, kind, seed=100 + j)).to(dev) for j in range(5)]
-            t = time_gpu(lambda i: ok(lib.fma_continuous_count(ids[i % 5].data_ptr(), 4, n_ids, out_cnt.data_ptr(), bins,
-                                                               ws_cnt.data_ptr(), ws_cnt.numel(), stream)), 50, warmup=5,
-                         blocker=blocker)
-            hbm(f"continuous_count_16Mi_{kind}", n_ids * 4 + bins * 4, t)
+            hbm(f"continuous_count_16Mi_{kind}", n_ids * 4 + bins * 4,
+                lambda i: ok(lib.fma_continuous_count(ids[i % 5].data_ptr(), 4, n_ids, out_cnt.data_ptr(), bins,
+                                                      ws_cnt.data_ptr(), ws_cnt.numel(), stream)), n=50, warmup=5)
             expect = np.bincount(O.make_ids(n_ids, bins, kind, seed=100 + 49 % 5), minlength=bins)
             assert np.array_equal(out_cnt.cpu().view(torch.int32).numpy().astype(np.int64), expect), "count mismatch"
             del ids
         result["kernels"] = kernels
-        dominant = kernels["up_projection_swiglu_fwd(NT)"]
+        dominant = kernels.get("up_projection_swiglu_fwd(NT)") or next(iter(kernels.values()))
         result["roofline"] = {
             "kernel": "grouped_gemm_kernel<NT, SwiGLU epilogue> (up-projection forward)",
             "bound": "mfma",

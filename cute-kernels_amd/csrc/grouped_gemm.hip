@@ -355,8 +355,14 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         const uint32_t band_m = tiles_m - first_m < (uint32_t)kGroupM ? tiles_m - first_m : (uint32_t)kGroupM;
         const uint32_t mt = first_m + (local % band) % band_m;
         const uint32_t nt = (local % band) / band_m;
+#if defined(FMA_EXPERIMENT_SAME_TILE)
+        const uint32_t m0 = 0, n0 = 0;  // diagnostic build: every workgroup reads the same, cache-resident tile
+        (void)mt;
+        (void)nt;
+#else
         const uint32_t m0 = mt * BM;
         const uint32_t n0 = nt * TN;
+#endif
 
         const uint16_t* Ae = args.A + s_off_a[e];
         const uint16_t* Be = args.B + s_off_b[e];
@@ -407,6 +413,9 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             lt_b.setup(Be, Ne, Ke, n0, Ne, wave, lane);
         }
         auto issue = [&](int stage, uint32_t k0) {
+#if defined(FMA_EXPERIMENT_SKIP_LOADS)
+            if (k0 >= 2 * BK) return;  // diagnostic build: steady-state loads removed (results are wrong)
+#endif
             if constexpr (A_KC) lk_a.issue(stage ? s_a1 : s_a0, k0, lane);
             else lt_a.issue(stage ? s_a1 : s_a0, k0, lane);
             if constexpr (B_KC) lk_b.issue(stage ? s_b1 : s_b0, k0, lane);
@@ -464,8 +473,10 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             load_frags(stage, 3, 1);
             mma(0);
             interleave_reads();
+            // every load of step kt+1 has landed and every LDS read of this stage has returned
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-            __syncthreads();
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
             if (kt + 1 < KT) load_frags(stage ^ 1, 0, 0);
             mma(1);
             if (kt + 2 < KT) issue(stage, (kt + 2) * BK);
@@ -474,7 +485,8 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             issue(0, 0);
             if (KT > 1) issue(1, BK);
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-            __syncthreads();
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
             load_frags(0, 0, 0);
             for (uint32_t kt = 0; kt < KT; kt += 2) {
                 step(0, kt);
@@ -546,12 +558,19 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     }
 }
 
+// wavefronts per workgroup: kWavesM x kWavesN (2 x 4 = eight 128x64 wave tiles, 2 x 2 = four 128x128 wave tiles)
+#ifndef FMA_GEMM_WAVES_N
+#define FMA_GEMM_WAVES_N 4
+#endif
+constexpr int kWavesM = 2;
+constexpr int kWavesN = FMA_GEMM_WAVES_N;
+
 // every instantiation the entry points launch (explicit, so that host stub and device code are both emitted)
-template __global__ void grouped_gemm_kernel<2, 4, true, true, EPI_PLAIN>(const GemmArgs);
-template __global__ void grouped_gemm_kernel<2, 4, true, false, EPI_PLAIN>(const GemmArgs);
-template __global__ void grouped_gemm_kernel<2, 4, false, true, EPI_PLAIN>(const GemmArgs);
-template __global__ void grouped_gemm_kernel<2, 4, false, false, EPI_PLAIN>(const GemmArgs);
-template __global__ void grouped_gemm_kernel<2, 4, true, true, EPI_SWIGLU>(const GemmArgs);
+template __global__ void grouped_gemm_kernel<kWavesM, kWavesN, true, true, EPI_PLAIN>(const GemmArgs);
+template __global__ void grouped_gemm_kernel<kWavesM, kWavesN, true, false, EPI_PLAIN>(const GemmArgs);
+template __global__ void grouped_gemm_kernel<kWavesM, kWavesN, false, true, EPI_PLAIN>(const GemmArgs);
+template __global__ void grouped_gemm_kernel<kWavesM, kWavesN, false, false, EPI_PLAIN>(const GemmArgs);
+template __global__ void grouped_gemm_kernel<kWavesM, kWavesN, true, true, EPI_SWIGLU>(const GemmArgs);
 
 template <int NWM, int NWN, bool A_KC, bool B_KC, int EPI>
 int launch(const GemmArgs& args, hipStream_t st) {
@@ -594,10 +613,10 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
     hipStream_t st = (hipStream_t)stream;
     const bool a_kc = trans_a == 0;  // A stored [M, K]: reduction dim contiguous
     const bool b_kc = trans_b != 0;  // B stored [N, K]: reduction dim contiguous
-    if (a_kc && b_kc) return launch<2, 4, true, true, EPI_PLAIN>(args, st);
-    if (a_kc && !b_kc) return launch<2, 4, true, false, EPI_PLAIN>(args, st);
-    if (!a_kc && b_kc) return launch<2, 4, false, true, EPI_PLAIN>(args, st);
-    return launch<2, 4, false, false, EPI_PLAIN>(args, st);
+    if (a_kc && b_kc) return launch<kWavesM, kWavesN, true, true, EPI_PLAIN>(args, st);
+    if (a_kc && !b_kc) return launch<kWavesM, kWavesN, true, false, EPI_PLAIN>(args, st);
+    if (!a_kc && b_kc) return launch<kWavesM, kWavesN, false, true, EPI_PLAIN>(args, st);
+    return launch<kWavesM, kWavesN, false, false, EPI_PLAIN>(args, st);
 }
 
 int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, const uint32_t* M_arr, int64_t E,
@@ -629,7 +648,7 @@ int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, co
     args.const_n = (uint32_t)(2 * I);
     args.const_k = (uint32_t)K;
     args.alpha = 1.0f;
-    return launch<2, 4, true, true, EPI_SWIGLU>(args, (hipStream_t)stream);
+    return launch<kWavesM, kWavesN, true, true, EPI_SWIGLU>(args, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -14,7 +14,8 @@ import torch
 
 
 _LIB_NAME = "libfma_hip.so"
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
+# FMA_HIP_LIBRARY names another build of the same library (e.g. one compiled with different tuning macros)
+_LIB_PATH = os.environ.get("FMA_HIP_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
 _ABI_VERSION = 1
 
 FMA_F32, FMA_F16, FMA_BF16 = 0, 1, 2
