@@ -218,9 +218,19 @@ def main():
         mfma("up_projection_dgrad(NN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, w1, dxg, counts, K_fc, N_fc, 0, 0))
         mfma("up_projection_wgrad(TN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, xg, dw1, N_fc, K_fc, counts, 1, 0))
 
+        # calibration for the profiler's FETCH_SIZE / WRITE_SIZE counters: a plain device copy of known size (ATen's
+        # elementwise copy kernel): reads 1 GiB, writes 1 GiB
+        if want("hbm_copy_1GiB"):
+            src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()
+            dst = torch.empty_like(src)
+            hbm("hbm_copy_1GiB", 2 * src.numel() * s, lambda i: dst.copy_(src), n=10)
+            del src, dst
+
         # row kernels: algorithmic bytes = each distinct input row once + each output row once + index / gate words
         hbm("gather_rows", T * H * s + R * H * s + R * 4,
             lambda i: ok(lib.fma_gather_rows(x.data_ptr(), perm.data_ptr(), R, H, k, xg.data_ptr(), BF16, stream)))
+        hbm("dispatch_rows", T * H * s + R * H * s + R * 4,
+            lambda i: ok(lib.fma_dispatch_rows(x.data_ptr(), inv.data_ptr(), T, k, H, xg.data_ptr(), BF16, stream)))
         hbm("combine", R * H * s + R * (4 + s) + T * H * s,
             lambda i: ok(lib.fma_combine(o.data_ptr(), inv.data_ptr(), weights_d.data_ptr(), T, k, H, y.data_ptr(), BF16,
                                          stream)))

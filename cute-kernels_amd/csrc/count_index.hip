@@ -142,7 +142,16 @@ __global__ __launch_bounds__(kReduceThreads) void count_reduce_kernel(const uint
     constexpr uint32_t parts = kReduceThreads / kReduceBins;
     uint32_t s = 0;
     if (e < E) {
-        for (uint32_t b = part; b < rows; b += parts) s += partials[(uint64_t)b * E + e];
+        // eight independent loads in flight per thread: the rows are few, the latency of each load is what costs
+        uint32_t b = part;
+        for (; b + 7 * parts < rows; b += 8 * parts) {
+            uint32_t r[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) r[u] = partials[(uint64_t)(b + u * parts) * E + e];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += r[u];
+        }
+        for (; b < rows; b += parts) s += partials[(uint64_t)b * E + e];
     }
     s_sum[tid] = s;
     __syncthreads();

@@ -32,6 +32,27 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_kernel(const uint4* _
     }
 }
 
+// out[inv[t*k + j]] = x[t] for j < k: the same gather written from the token's side, so that every input row is
+// fetched once however many experts it is routed to
+constexpr int kDispatchTokens = 2;  // tokens per workgroup
+__global__ __launch_bounds__(kRowThreads) void dispatch_rows_kernel(const uint4* __restrict__ x,
+                                                                    const int32_t* __restrict__ inv, int64_t T,
+                                                                    int64_t k, int64_t vecs, uint4* __restrict__ out) {
+    const int64_t t0 = (int64_t)blockIdx.x * kDispatchTokens;
+    for (int64_t v = threadIdx.x; v < vecs; v += kRowThreads) {
+        uint4 row[kDispatchTokens];
+#pragma unroll
+        for (int u = 0; u < kDispatchTokens; ++u) row[u] = x[(t0 + u < T ? t0 + u : T - 1) * vecs + v];
+#pragma unroll
+        for (int u = 0; u < kDispatchTokens; ++u) {
+            if (t0 + u < T) {
+                const int32_t* dst = inv + (t0 + u) * k;
+                for (int64_t j = 0; j < k; ++j) out[(int64_t)dst[j] * vecs + v] = row[u];
+            }
+        }
+    }
+}
+
 // y[t] = sum_j gates[t,j] * o[inv[t,j]]; one workgroup per token, fp32 accumulation in ascending j
 template <typename T>
 __global__ __launch_bounds__(kRowThreads) void combine_kernel(const Vec16<T>* __restrict__ o,
@@ -75,7 +96,10 @@ __global__ __launch_bounds__(kRowThreads) void combine_kernel(const Vec16<T>* __
 }
 
 // d_o[inv[t,j]] = gates[t,j] * dy[t];  d_gates[t,j] = <dy[t], o[inv[t,j]]>
-template <typename T>
+// One workgroup per token. dy[t] is read once and kept in registers (up to kBwdVecs 16-byte vectors per thread,
+// i.e. rows of up to 4096 bf16); longer rows fall back to re-reading it per expert choice.
+constexpr int kBwdVecs = 2;
+template <typename T, bool CACHED>
 __global__ __launch_bounds__(kRowThreads) void combine_bwd_kernel(const Vec16<T>* __restrict__ dy,
                                                                   const Vec16<T>* __restrict__ o,
                                                                   const int32_t* __restrict__ inv,
@@ -87,12 +111,19 @@ __global__ __launch_bounds__(kRowThreads) void combine_bwd_kernel(const Vec16<T>
     const int64_t t = blockIdx.x;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
+    Vec16<T> d_reg[kBwdVecs];
+    if constexpr (CACHED) {
+#pragma unroll
+        for (int u = 0; u < kBwdVecs; ++u) {
+            const int64_t v = threadIdx.x + (int64_t)u * kRowThreads;
+            if (v < vecs) d_reg[u] = dy[t * vecs + v];
+        }
+    }
     for (int64_t j = 0; j < k; ++j) {
         const int64_t row = inv[t * k + j];
         const float g = gates ? Num<T>::up(gates[t * k + j]) : 1.0f;
         float dot = 0.0f;
-        for (int64_t v = threadIdx.x; v < vecs; v += kRowThreads) {
-            const Vec16<T> d = dy[t * vecs + v];
+        auto one = [&](int64_t v, const Vec16<T>& d) {
             Vec16<T> w;
             if (d_gates) {
                 const Vec16<T> ov = o[row * vecs + v];
@@ -102,16 +133,25 @@ __global__ __launch_bounds__(kRowThreads) void combine_bwd_kernel(const Vec16<T>
 #pragma unroll
             for (int c = 0; c < N; ++c) w.v[c] = Num<T>::down(g * Num<T>::up(d.v[c]));
             d_o[row * vecs + v] = w;
+        };
+        if constexpr (CACHED) {
+#pragma unroll
+            for (int u = 0; u < kBwdVecs; ++u) {
+                const int64_t v = threadIdx.x + (int64_t)u * kRowThreads;
+                if (v < vecs) one(v, d_reg[u]);
+            }
+        } else {
+            for (int64_t v = threadIdx.x; v < vecs; v += kRowThreads) one(v, dy[t * vecs + v]);
         }
         if (d_gates) {
             dot = wave_sum(dot);
             if (lane == 0) s_part[wave] = dot;
             __syncthreads();
             if (threadIdx.x == 0) {
-                float s = 0.0f;
+                float sum = 0.0f;
 #pragma unroll
-                for (int w = 0; w < NW; ++w) s += s_part[w];
-                d_gates[t * k + j] = Num<T>::down(s);
+                for (int w = 0; w < NW; ++w) sum += s_part[w];
+                d_gates[t * k + j] = Num<T>::down(sum);
             }
             __syncthreads();
         }
@@ -131,8 +171,14 @@ template <typename T>
 int launch_combine_bwd(const void* dy, const void* o, const int32_t* inv, const void* gates, int64_t T_, int64_t k,
                        int64_t H, void* d_o, void* d_gates, hipStream_t st) {
     const int64_t vecs = H / Vec16<T>::N;
-    hipLaunchKernelGGL(combine_bwd_kernel<T>, dim3((uint32_t)T_), dim3(kRowThreads), 0, st, (const Vec16<T>*)dy,
-                       (const Vec16<T>*)o, inv, (const T*)gates, k, vecs, (Vec16<T>*)d_o, (T*)d_gates);
+    if (vecs <= (int64_t)kBwdVecs * kRowThreads)
+        hipLaunchKernelGGL((combine_bwd_kernel<T, true>), dim3((uint32_t)T_), dim3(kRowThreads), 0, st,
+                           (const Vec16<T>*)dy, (const Vec16<T>*)o, inv, (const T*)gates, k, vecs, (Vec16<T>*)d_o,
+                           (T*)d_gates);
+    else
+        hipLaunchKernelGGL((combine_bwd_kernel<T, false>), dim3((uint32_t)T_), dim3(kRowThreads), 0, st,
+                           (const Vec16<T>*)dy, (const Vec16<T>*)o, inv, (const T*)gates, k, vecs, (Vec16<T>*)d_o,
+                           (T*)d_gates);
     return launch_status("combine_bwd");
 }
 
@@ -164,6 +210,23 @@ int fma_gather_rows(const void* x, const int32_t* idx, int64_t R, int64_t H, int
     hipLaunchKernelGGL(gather_rows_kernel, dim3(blocks), dim3(kRowThreads), 0, (hipStream_t)stream, (const uint4*)x,
                        idx, R, vecs, divisor, (uint4*)out);
     return launch_status("gather_rows");
+}
+
+int fma_dispatch_rows(const void* x, const int32_t* inv, int64_t T, int64_t k, int64_t H, void* out, int dtype,
+                      void* stream) {
+    using namespace fmahip;
+    int rc = check_rows("dispatch_rows", dtype, H);
+    if (rc) return rc;
+    FMA_REQUIRE(T >= 0 && T <= 0x7fffffffll, FMA_ERR_BAD_SIZE, "dispatch_rows: bad token count %lld", (long long)T);
+    FMA_REQUIRE(k >= 1 && T * k <= 0x7fffffffll, FMA_ERR_BAD_SIZE, "dispatch_rows: bad top_k %lld", (long long)k);
+    if (T == 0) return FMA_OK;
+    FMA_REQUIRE(x && inv && out, FMA_ERR_NULL_POINTER, "dispatch_rows: NULL pointer");
+    FMA_REQUIRE(aligned16(x) && aligned16(out), FMA_ERR_MISALIGNED, "dispatch_rows: x/out must be 16-byte aligned");
+    const int64_t vecs = H * dtype_bytes(dtype) / 16;
+    const uint32_t blocks = (uint32_t)((T + kDispatchTokens - 1) / kDispatchTokens);
+    hipLaunchKernelGGL(dispatch_rows_kernel, dim3(blocks), dim3(kRowThreads), 0, (hipStream_t)stream, (const uint4*)x,
+                       inv, T, k, vecs, (uint4*)out);
+    return launch_status("dispatch_rows");
 }
 
 int fma_combine(const void* o, const int32_t* inv, const void* gates, int64_t T, int64_t k, int64_t H, void* y,

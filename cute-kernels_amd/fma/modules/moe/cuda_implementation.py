@@ -62,6 +62,21 @@ def gather_rows_cuda(x: torch.Tensor, idx: torch.Tensor, divisor: int, output: t
     _lib.check(rc, "gather_rows_cuda")
 
 
+@custom_op(f"{LIBRARY_NAME}::dispatch_rows_cuda", mutates_args={"output"})
+def dispatch_rows_cuda(x: torch.Tensor, inv: torch.Tensor, top_k: int, output: torch.Tensor) -> None:
+    _lib.require_gpu(x, inv, output)
+    T, H = x.shape
+    assert output.shape == (T * top_k, H) and x.dtype == output.dtype
+    assert inv.dtype == torch.int32 and inv.numel() == T * top_k
+    assert x.is_contiguous() and output.is_contiguous() and inv.is_contiguous()
+    with torch.cuda.device(x.device):
+        rc = _lib.load().fma_dispatch_rows(
+            x.data_ptr(), inv.data_ptr(), T, top_k, H, output.data_ptr(), _lib.dtype_code(x.dtype),
+            _lib.current_stream(x.device),
+        )
+    _lib.check(rc, "dispatch_rows_cuda")
+
+
 @custom_op(f"{LIBRARY_NAME}::combine_cuda", mutates_args={"output"})
 def combine_cuda(
     o: torch.Tensor, inv: torch.Tensor, gates: torch.Tensor | None, top_k: int, output: torch.Tensor
@@ -168,7 +183,8 @@ class _GatherRows(torch.autograd.Function):
     def forward(ctx, x: torch.Tensor, perm: torch.Tensor, inv: torch.Tensor, top_k: int) -> torch.Tensor:
         assert x.dim() == 2
         output = torch.empty(perm.numel(), x.size(1), device=x.device, dtype=x.dtype)
-        gather_rows_cuda(x, perm, top_k, output)
+        # token-side form of output[i] = x[perm[i] // top_k]: every row of x is read once
+        dispatch_rows_cuda(x, inv, top_k, output)
         ctx.save_for_backward(inv)
         ctx.top_k = top_k
         ctx.T = x.size(0)

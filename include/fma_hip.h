@@ -100,6 +100,12 @@ int fma_moe_build_index(const void* ids, int id_bytes, int64_t R, int64_t E, uin
 int fma_gather_rows(const void* x, const int32_t* idx, int64_t R, int64_t H, int32_t divisor, void* out,
                     int dtype, void* stream);
 
+/* out[inv[t*k+j], :] = x[t, :] for t < T, j < k: the gather above for idx = the stable routing order and divisor =
+ * top_k, written from the token's side (inv is the inverse permutation fma_moe_build_index returns), so each input
+ * row is read once however many experts it goes to. Same references as fma_gather_rows. */
+int fma_dispatch_rows(const void* x, const int32_t* inv, int64_t T, int64_t k, int64_t H, void* out, int dtype,
+                      void* stream);
+
 /* y[t, :] = sum_{j<k} gates[t*k+j] * o[inv[t*k+j], :]  accumulated in fp32 in ascending j, rounded once.
  * gates may be NULL (all ones; gives the k-way sum the backward of the gather needs). gates has dtype.
  * Replaces ungroup_with_padding + torch.bmm(router_weights, y) (fma/modules/moe/__init__.py:235-246,

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from fma import KernelBackend, swiglu, swiglu_packed
-from fma.modules.moe.cuda_implementation import build_routing_index, combine, gather_rows
+from fma.modules.moe.cuda_implementation import build_routing_index, combine, gather_rows, gather_rows_cuda
 from oracle import moe_oracle as O
 
 from gpu_util import DEV, rel_err
@@ -25,9 +25,12 @@ def test_gather_is_bit_exact(dtype, T, H, E, k):
     selected, _ = O.make_routing(T, E, k, "uniform", seed=1)
     idx = O.routing_index(selected.numpy(), E)
     _, _, perm, _, inv = build_routing_index(selected.to(DEV), E)
-    got = gather_rows(x.to(DEV), perm, inv, k).cpu()
+    got = gather_rows(x.to(DEV), perm, inv, k).cpu()  # token-side form (fma_dispatch_rows)
     expect = x[torch.from_numpy(idx["perm"].astype(np.int64)) // k]  # fma/modules/moe/__init__.py:269,275
     assert torch.equal(got, expect)
+    out = torch.empty(T * k, H, dtype=dtype, device=DEV)  # row-side form (fma_gather_rows)
+    gather_rows_cuda(x.to(DEV), perm, k, out)
+    assert torch.equal(out.cpu(), expect)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
