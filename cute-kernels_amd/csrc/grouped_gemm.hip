@@ -195,6 +195,62 @@ __device__ __forceinline__ bf16x8 read_tr_frag(const uint8_t* p) {
     return __builtin_bit_cast(bf16x8, v);
 }
 
+// ---- epilogue staging: a wavefront transposes its accumulator sub-tile through a private 16 KB slice of LDS ----
+// The MFMA leaves a lane with 4 consecutive columns of one row per 32x32 block, so storing straight from registers
+// writes 8-byte pieces of 32 different rows per instruction. Staged through LDS as rows of ROWB bytes, every store
+// instruction writes 16 bytes per lane and whole 64- or 128-byte row segments.
+// Row m, 16-byte chunk c of the image sits at m*ROWB + ((c ^ key(m)) << 4), key(m) = (m / rows-per-256-B) mod chunks:
+// the 8-byte writes of 32 consecutive rows conflict at most two ways, the 16-byte reads not at all.
+template <int ROWB>
+__device__ __forceinline__ uint32_t stage_off(uint32_t m, uint32_t chunk16) {
+    constexpr uint32_t kChunks = ROWB / 16;
+    constexpr uint32_t kRowsPer256 = 256 / ROWB;
+    return m * ROWB + ((chunk16 ^ ((m / kRowsPer256) & (kChunks - 1))) << 4);
+}
+// lane's 4 columns [col, col+4) of image row m
+template <int ROWB>
+__device__ __forceinline__ void stage_put(uint8_t* img, uint32_t m, uint32_t col, uint2 v) {
+    *reinterpret_cast<uint2*>(img + stage_off<ROWB>(m, col >> 3) + ((col >> 2) & 1u) * 8u) = v;
+}
+// Stores the image (rows x ROWB/2 columns) to out[(row0 + r) * ld + col0 + c], rows >= row_end and columns >= col_end
+// masked. col0, ld and col_end are multiples of 8 elements, so every 16-byte piece is wholly inside or outside.
+template <int ROWB, int ROWS>
+__device__ __forceinline__ void stage_flush(const uint8_t* img, uint16_t* out, uint64_t ld, uint32_t row0,
+                                            uint32_t row_end, uint32_t col0, uint32_t col_end, uint32_t lane) {
+    constexpr uint32_t kChunks = ROWB / 16;      // 16-byte pieces per image row
+    constexpr uint32_t kRowsPerInst = 64 / kChunks;
+    const uint32_t c16 = lane % kChunks;
+    const uint32_t col = col0 + c16 * 8u;
+#pragma unroll
+    for (uint32_t it = 0; it < ROWS / kRowsPerInst; ++it) {
+        const uint32_t r = it * kRowsPerInst + lane / kChunks;
+        const uint4 v = *reinterpret_cast<const uint4*>(img + stage_off<ROWB>(r, c16));
+        if (row0 + r < row_end && col < col_end)
+            *reinterpret_cast<uint4*>(out + (uint64_t)(row0 + r) * ld + col) = v;
+    }
+}
+
+// Like stage_flush for an image whose row holds two windows of HALF columns each: window 0 goes to columns
+// col0.., window 1 to columns second0 + col0.. of the same output row (the "up" and "gate" halves of h).
+template <int ROWB, int ROWS, int HALF>
+__device__ __forceinline__ void stage_flush_split(const uint8_t* img, uint16_t* out, uint64_t ld, uint32_t row0,
+                                                  uint32_t row_end, uint32_t col0, uint32_t col_end, uint32_t second0,
+                                                  uint32_t lane) {
+    constexpr uint32_t kChunks = ROWB / 16;
+    constexpr uint32_t kRowsPerInst = 64 / kChunks;
+    const uint32_t c16 = lane % kChunks;
+    const uint32_t in_window = (c16 * 8u) % HALF;
+    const uint32_t window = (c16 * 8u) / HALF;
+    const uint32_t col = col0 + in_window;
+#pragma unroll
+    for (uint32_t it = 0; it < ROWS / kRowsPerInst; ++it) {
+        const uint32_t r = it * kRowsPerInst + lane / kChunks;
+        const uint4 v = *reinterpret_cast<const uint4*>(img + stage_off<ROWB>(r, c16));
+        if (row0 + r < row_end && col < col_end)
+            *reinterpret_cast<uint4*>(out + (uint64_t)(row0 + r) * ld + window * second0 + col) = v;
+    }
+}
+
 // Scheduling hint for one k slice: MFMAS matrix instructions with READS LDS reads spread evenly between them.
 template <int R, int MFMAS, int READS>
 __device__ __forceinline__ void interleave_mfma_lds() {
@@ -477,7 +533,9 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            if (kt + 1 < KT) load_frags(stage ^ 1, 0, 0);
+            // unconditional (after the last step the fragments are simply not used): straight-line code lets the
+            // compiler count outstanding LDS reads exactly, so the MFMAs below do not wait for these reads
+            load_frags(stage ^ 1, 0, 0);
             mma(1);
             if (kt + 2 < KT) issue(stage, (kt + 2) * BK);
         };
@@ -494,66 +552,82 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             }
         }
 
-        // ---- epilogue: lane holds row m = (lane & 31), columns q*8 + (lane >> 5)*4 + 0..3 of each 32x32 block ----
+        // ---- epilogue ----
+        // Past the last barrier of the K loop nobody reads the LDS stages any more; each wavefront takes its own 16 KB
+        // slice of them as staging space (the barrier at the top of the next tile keeps the next loads away from it).
+        // A lane holds row (lane & 31), columns q*8 + (lane >> 5)*4 + 0..3 of each 32x32 accumulator block.
+        static_assert(WM * WN * 2 == 16384 && NW == 8, "staging slices are sized for eight 128x64 wave tiles");
+        // the lane id is made opaque here so that the epilogue's per-lane address arithmetic is redone per tile instead
+        // of being hoisted out of the tile loop, where it would occupy registers throughout the K loop
+        uint32_t el = lane;
+        asm volatile("" : "+v"(el));
+        uint8_t* const img = (wave < 2 ? s_a0 : wave < 4 ? s_b0 : wave < 6 ? s_a1 : s_b1) + (wave & 1u) * 16384u;
         const float alpha = args.alpha;
+        const uint32_t row0 = m0 + wm * WM;  // first output row of this wavefront
         if constexpr (EPI == EPI_PLAIN) {
-            uint16_t* De = args.D + off_d;
 #pragma unroll
-            for (int i = 0; i < FM; ++i) {
-                const uint32_t m = m0 + wm * WM + i * 32 + (lane & 31u);
-                if (m >= Me) continue;
-                uint16_t* drow = De + (uint64_t)m * Ne;
+            for (int i = 0; i < FM; ++i)
 #pragma unroll
-                for (int j = 0; j < FN; ++j) {
+                for (int j = 0; j < FN; ++j)
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        const uint32_t n = n0 + wn * WN + j * 32 + q * 8 + (lane >> 5) * 4;
-                        if (n < Ne) {
-                            uint2 w;
-                            w.x = pack_bf16x2(alpha * acc[i][j][q * 4 + 0], alpha * acc[i][j][q * 4 + 1]);
-                            w.y = pack_bf16x2(alpha * acc[i][j][q * 4 + 2], alpha * acc[i][j][q * 4 + 3]);
-                            *reinterpret_cast<uint2*>(drow + n) = w;
-                        }
+                        uint2 w;
+                        w.x = pack_bf16x2(alpha * acc[i][j][q * 4 + 0], alpha * acc[i][j][q * 4 + 1]);
+                        w.y = pack_bf16x2(alpha * acc[i][j][q * 4 + 2], alpha * acc[i][j][q * 4 + 3]);
+                        stage_put<WN * 2>(img, i * 32 + (el & 31u), j * 32 + q * 8 + (el >> 5) * 4, w);
                     }
-                }
-            }
+            stage_flush<WN * 2, WM>(img, args.D + off_d, Ne, row0, Me, n0 + wn * WN, Ne, el);
         } else {
+            // first the rounded pre-activation (32 "up" columns | 32 "gate" columns per row), then the activation
+            constexpr int HB = WN * 2;  // bytes per staged row of h: 32 "up" columns | 32 "gate" columns
+            constexpr int YB = WN;      // bytes per staged row of the activation
             uint16_t* He = args.D ? args.D + off_d : nullptr;
             uint16_t* Ce = args.ACT + off_d / 2;
+            const uint32_t ncol0 = n0 + wn * (WN / 2);
 #pragma unroll
-            for (int i = 0; i < FM; ++i) {
-                const uint32_t m = m0 + wm * WM + i * 32 + (lane & 31u);
-                if (m >= Me) continue;
+            for (int i = 0; i < FM; ++i)
 #pragma unroll
-                for (int j = 0; j < FN / 2; ++j) {
+                for (int j = 0; j < FN / 2; ++j)
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        const uint32_t n = n0 + wn * (WN / 2) + j * 32 + q * 8 + (lane >> 5) * 4;
-                        if (n < n_span) {
-                            float u[4], g[4], y[4];
+                        float u[4], g[4], y[4];
 #pragma unroll
-                            for (int x = 0; x < 4; ++x) {
-                                u[x] = round_bf16(alpha * acc[i][j][q * 4 + x]);
-                                g[x] = round_bf16(alpha * acc[i][j + FN / 2][q * 4 + x]);
-                                y[x] = u[x] * g[x] * sigmoid_clamped(g[x]);
-                            }
-                            if (He) {
-                                uint2 wu, wg;
-                                wu.x = pack_bf16x2(u[0], u[1]);
-                                wu.y = pack_bf16x2(u[2], u[3]);
-                                wg.x = pack_bf16x2(g[0], g[1]);
-                                wg.y = pack_bf16x2(g[2], g[3]);
-                                *reinterpret_cast<uint2*>(He + (uint64_t)m * Ne + n) = wu;
-                                *reinterpret_cast<uint2*>(He + (uint64_t)m * Ne + n_span + n) = wg;
-                            }
-                            uint2 wy;
-                            wy.x = pack_bf16x2(y[0], y[1]);
-                            wy.y = pack_bf16x2(y[2], y[3]);
-                            *reinterpret_cast<uint2*>(Ce + (uint64_t)m * n_span + n) = wy;
+                        for (int x = 0; x < 4; ++x) {
+                            u[x] = round_bf16(alpha * acc[i][j][q * 4 + x]);
+                            g[x] = round_bf16(alpha * acc[i][j + FN / 2][q * 4 + x]);
+                            y[x] = u[x] * g[x] * sigmoid_for<bf16_t>(g[x]);
+                        }
+                        const uint32_t m = i * 32 + (el & 31u);
+                        const uint32_t c = j * 32 + q * 8 + (el >> 5) * 4;
+                        uint2 wy;
+                        wy.x = pack_bf16x2(y[0], y[1]);
+                        wy.y = pack_bf16x2(y[2], y[3]);
+                        // the packed activation waits in two accumulator registers until h has left the staging slice
+                        acc[i][j][q * 4 + 0] = __uint_as_float(wy.x);
+                        acc[i][j][q * 4 + 1] = __uint_as_float(wy.y);
+                        if (He) {
+                            uint2 wu, wg;
+                            wu.x = pack_bf16x2(u[0], u[1]);
+                            wu.y = pack_bf16x2(u[2], u[3]);
+                            wg.x = pack_bf16x2(g[0], g[1]);
+                            wg.y = pack_bf16x2(g[2], g[3]);
+                            stage_put<HB>(img, m, c, wu);
+                            stage_put<HB>(img, m, WN / 2 + c, wg);
                         }
                     }
-                }
-            }
+            if (He) stage_flush_split<HB, WM, WN / 2>(img, He, Ne, row0, Me, ncol0, n_span, n_span, el);
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN / 2; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        uint2 wy;
+                        wy.x = __float_as_uint(acc[i][j][q * 4 + 0]);
+                        wy.y = __float_as_uint(acc[i][j][q * 4 + 1]);
+                        stage_put<YB>(img, i * 32 + (el & 31u), j * 32 + q * 8 + (el >> 5) * 4, wy);
+                    }
+            stage_flush<YB, WM>(img, Ce, n_span, row0, Me, ncol0, n_span, el);
         }
     }
 }

@@ -9,10 +9,14 @@ namespace {
 
 constexpr int kSwThreads = 256;
 
-__device__ __forceinline__ float swiglu_f(float g, float u) { return u * g * sigmoid_clamped(g); }
+template <typename T>
+__device__ __forceinline__ float swiglu_f(float g, float u) {
+    return u * g * sigmoid_for<T>(g);
+}
 
+template <typename T>
 __device__ __forceinline__ void swiglu_b(float g, float u, float dy, float& dg, float& du) {
-    const float s = sigmoid_clamped(g);
+    const float s = sigmoid_for<T>(g);
     dg = dy * u * (s + g * s * (1.0f - s));
     du = dy * g * s;
 }
@@ -39,10 +43,10 @@ __global__ __launch_bounds__(kSwThreads) void swiglu_fwd_kernel(const T* __restr
             const Vec16<T> u = *reinterpret_cast<const Vec16<T>*>(up + r * s.up + c);
             Vec16<T> y;
 #pragma unroll
-            for (int e = 0; e < N; ++e) y.v[e] = Num<T>::down(swiglu_f(Num<T>::up(g.v[e]), Num<T>::up(u.v[e])));
+            for (int e = 0; e < N; ++e) y.v[e] = Num<T>::down(swiglu_f<T>(Num<T>::up(g.v[e]), Num<T>::up(u.v[e])));
             *reinterpret_cast<Vec16<T>*>(out + r * s.out + c) = y;
         } else {
-            out[r * s.out + c] = Num<T>::down(swiglu_f(Num<T>::up(gate[r * s.gate + c]), Num<T>::up(up[r * s.up + c])));
+            out[r * s.out + c] = Num<T>::down(swiglu_f<T>(Num<T>::up(gate[r * s.gate + c]), Num<T>::up(up[r * s.up + c])));
         }
     }
 }
@@ -66,7 +70,7 @@ __global__ __launch_bounds__(kSwThreads) void swiglu_bwd_kernel(const T* __restr
 #pragma unroll
             for (int e = 0; e < N; ++e) {
                 float a, b;
-                swiglu_b(Num<T>::up(g.v[e]), Num<T>::up(u.v[e]), Num<T>::up(d.v[e]), a, b);
+                swiglu_b<T>(Num<T>::up(g.v[e]), Num<T>::up(u.v[e]), Num<T>::up(d.v[e]), a, b);
                 og.v[e] = Num<T>::down(a);
                 ou.v[e] = Num<T>::down(b);
             }
@@ -74,7 +78,7 @@ __global__ __launch_bounds__(kSwThreads) void swiglu_bwd_kernel(const T* __restr
             *reinterpret_cast<Vec16<T>*>(dup + r * s.dup + c) = ou;
         } else {
             float a, b;
-            swiglu_b(Num<T>::up(gate[r * s.gate + c]), Num<T>::up(up[r * s.up + c]), Num<T>::up(dy[r * s.dy + c]), a, b);
+            swiglu_b<T>(Num<T>::up(gate[r * s.gate + c]), Num<T>::up(up[r * s.up + c]), Num<T>::up(dy[r * s.dy + c]), a, b);
             dgate[r * s.dgate + c] = Num<T>::down(a);
             dup[r * s.dup + c] = Num<T>::down(b);
         }
