@@ -21,9 +21,7 @@ from ...utils import ensure_contiguous
 # ---- custom ops ---------------------------------------------------------------------------------
 
 
-@custom_op(
-    f"{LIBRARY_NAME}::moe_build_index_cuda", mutates_args={"counts", "offsets", "perm", "eid", "inv", "workspace"}
-)
+@custom_op(f"{LIBRARY_NAME}::moe_build_index_cuda", mutates_args={"counts", "offsets", "perm", "eid", "inv"})
 def moe_build_index_cuda(
     ids: torch.Tensor,
     counts: torch.Tensor,
@@ -31,19 +29,22 @@ def moe_build_index_cuda(
     perm: torch.Tensor,
     eid: torch.Tensor,
     inv: torch.Tensor,
-    workspace: torch.Tensor,
 ) -> None:
-    _lib.require_gpu(ids, counts, offsets, perm, eid, inv, workspace)
+    _lib.require_gpu(ids, counts, offsets, perm, eid, inv)
     assert ids.dtype in (torch.int32, torch.int64) and ids.is_contiguous()
     assert counts.dtype == torch.uint32 and offsets.dtype == torch.uint32
     assert perm.dtype == eid.dtype == inv.dtype == torch.int32
     R, E = ids.numel(), counts.numel()
     assert perm.numel() == eid.numel() == inv.numel() == R and offsets.numel() == E
+    lib = _lib.load()
     with torch.cuda.device(ids.device):
-        rc = _lib.load().fma_moe_build_index(
+        # per-chunk histograms; scratch owned by this call (the op body is opaque to tracing, so the size query
+        # and the allocation may live here)
+        nbytes = max(lib.fma_moe_build_index_workspace_bytes(R, E), 4)
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=ids.device)
+        rc = lib.fma_moe_build_index(
             ids.data_ptr(), ids.element_size(), R, E, counts.data_ptr(), offsets.data_ptr(), perm.data_ptr(),
-            eid.data_ptr(), inv.data_ptr(), workspace.data_ptr(), workspace.numel() * workspace.element_size(),
-            _lib.current_stream(ids.device),
+            eid.data_ptr(), inv.data_ptr(), workspace.data_ptr(), nbytes, _lib.current_stream(ids.device),
         )
     _lib.check(rc, "moe_build_index_cuda")
 
@@ -166,9 +167,7 @@ def build_routing_index(
     perm = torch.empty(R, dtype=torch.int32, device=device)
     eid = torch.empty(R, dtype=torch.int32, device=device)
     inv = torch.empty(R, dtype=torch.int32, device=device)
-    nbytes = _lib.load().fma_moe_build_index_workspace_bytes(R, num_experts)
-    workspace = torch.empty(max(nbytes, 4) // 4, dtype=torch.int32, device=device)
-    moe_build_index_cuda(ids, counts, offsets, perm, eid, inv, workspace)
+    moe_build_index_cuda(ids, counts, offsets, perm, eid, inv)
     return counts, offsets, perm, eid, inv
 
 
