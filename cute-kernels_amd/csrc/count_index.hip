@@ -15,8 +15,18 @@
 namespace fmahip {
 namespace {
 
-constexpr int kCountThreads = 1024;
-constexpr int kCountUnroll = 4;
+#ifndef FMA_COUNT_THREADS
+#define FMA_COUNT_THREADS 1024
+#endif
+#ifndef FMA_COUNT_UNROLL
+#define FMA_COUNT_UNROLL 4
+#endif
+#ifndef FMA_COUNT_BLOCKS_PER_CU
+#define FMA_COUNT_BLOCKS_PER_CU 2
+#endif
+constexpr int kCountThreads = FMA_COUNT_THREADS;
+constexpr int kCountUnroll = FMA_COUNT_UNROLL;
+constexpr int kCountBlocksPerCu = FMA_COUNT_BLOCKS_PER_CU;
 constexpr int kCountLdsWords = 16384;  // 64 KB of bins (all copies)
 
 __host__ __device__ inline uint32_t floor_pow2(uint32_t x) {
@@ -40,7 +50,7 @@ inline CountPlan plan_count(uint64_t n, int id_bytes, int cus) {
     const uint64_t vec = 16 / id_bytes;
     const uint64_t min_ids = (uint64_t)kCountThreads * vec * 2;  // at least two vectors per thread
     uint64_t grid = (n + min_ids - 1) / min_ids;
-    const uint64_t max_grid = (uint64_t)(cus > 0 ? cus : 256) * 2;
+    const uint64_t max_grid = (uint64_t)(cus > 0 ? cus : 256) * kCountBlocksPerCu;
     if (grid > max_grid) grid = max_grid;
     if (grid < 1) grid = 1;
     uint64_t chunk = (n + grid - 1) / grid;
@@ -92,7 +102,14 @@ __global__ __launch_bounds__(kCountThreads) void continuous_count_kernel(const i
         for (; v + (uint64_t)(kCountUnroll - 1) * kCountThreads < nvec; v += (uint64_t)kCountUnroll * kCountThreads) {
             IdVec r[kCountUnroll];
 #pragma unroll
-            for (int u = 0; u < kCountUnroll; ++u) r[u] = vp[v + (uint64_t)u * kCountThreads];
+            for (int u = 0; u < kCountUnroll; ++u) {
+                // streamed once: non-temporal loads keep the ids from displacing useful lines in L2 (measured
+                // 14.3 us instead of 15.5 us per 64 MiB)
+                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                const u32x4 raw =
+                    __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(&vp[v + (uint64_t)u * kCountThreads]));
+                r[u] = __builtin_bit_cast(IdVec, raw);
+            }
 #pragma unroll
             for (int u = 0; u < kCountUnroll; ++u) {
 #pragma unroll
@@ -326,7 +343,7 @@ int64_t fma_continuous_count_workspace_bytes(int64_t n, int64_t E) {
     if (n < 0 || E < 1) return 0;
     // independent of id width and device: sized for the largest grid any call may use
     const int cus = fmahip::num_compute_units();
-    const int64_t max_grid = (int64_t)(cus > 0 ? cus : 256) * 2;
+    const int64_t max_grid = (int64_t)(cus > 0 ? cus : 256) * fmahip::kCountBlocksPerCu;
     return max_grid * E * 4;
 }
 
