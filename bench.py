@@ -212,6 +212,8 @@ def main():
         mfma("up_projection_swiglu_fwd(NT)", 2.0 * R * 2 * I * H,
              lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), h.data_ptr(), a.data_ptr(),
                                                       counts.data_ptr(), E, I, H, BF16, stream)))
+        # the unfused pair the fused kernel above replaces (same bits): plain up-projection, then swiglu_forward below
+        mfma("up_projection_plain_fwd(NT)", 2.0 * R * 2 * I * H, lambda i: gemm(xg, w1, h, counts, N_fc, K_fc, 0, 1))
         mfma("down_projection_fwd(NT)", 2.0 * R * I * H, lambda i: gemm(a, w2, o, counts, N_pj, K_pj, 0, 1))
         mfma("down_projection_dgrad(NN)", 2.0 * R * I * H, lambda i: gemm(d_o, w2, da, counts, K_pj, N_pj, 0, 0))
         mfma("down_projection_wgrad(TN)", 2.0 * R * I * H, lambda i: gemm(d_o, a, dw2, N_pj, K_pj, counts, 1, 0))
@@ -238,6 +240,9 @@ def main():
             lambda i: ok(lib.fma_combine_bwd(dy.data_ptr(), o.data_ptr(), inv.data_ptr(), weights_d.data_ptr(), T, k, H,
                                              d_o.data_ptr(), dgates.data_ptr(), BF16, stream)))
         es = 2 * I  # row stride of the packed pre-activation and of its gradient
+        hbm("swiglu_forward", 3 * R * I * s,
+            lambda i: ok(lib.fma_swiglu_forward(h.data_ptr() + I * s, h.data_ptr(), a.data_ptr(), R, I, es, es, I, BF16,
+                                                stream)), n=10)
         hbm("swiglu_backward", 5 * R * I * s,
             lambda i: ok(lib.fma_swiglu_backward(h.data_ptr() + I * s, h.data_ptr(), da.data_ptr(), dh.data_ptr() + I * s,
                                                  dh.data_ptr(), R, I, es, es, I, es, es, BF16, stream)), n=10)

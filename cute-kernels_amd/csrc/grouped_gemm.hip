@@ -7,7 +7,8 @@
 //    256x256 output tiles. Tile ids are handed out so that the 32 workgroups of one XCD (workgroup id mod 8)
 //    always hold a compact 8x4 block of tiles of the same group: they share A and B panels in that XCD's L2.
 //  * K is consumed in steps of 64 through two LDS stages of 2 x 32 KB. Every operand tile goes global -> LDS directly
-//    (global_load_lds_dwordx4, 1 KB per wavefront instruction, no staging registers), in one of two layouts:
+//    (buffer_load_dwordx4 ... lds, 1 KB per wavefront instruction, no staging registers; the buffer descriptor's range
+//    check zero-fills rows and reduction steps past the edge of a group), in one of two layouts:
 //      - an operand whose reduction dimension is contiguous in memory is kept as [row][64 k] (128-byte rows); row r,
 //        16-byte chunk c sits at phys_row(r)*128 + ((c ^ (r & 7)) << 4), phys_row rotating the low four row bits
 //        left by one, and an MFMA fragment (32 rows x 16 k) is one ds_read_b128 per lane;
@@ -89,99 +90,100 @@ __device__ __forceinline__ float round_bf16(float x) {
     return (float)b;
 }
 
-// ---- direct global -> LDS loader, operand with the reduction dimension contiguous: tile [256 rows][64 k] ------
-// A wavefront instruction moves 8 physical rows (1 KB); NI instructions per wavefront and K step.
-template <int NW>
+// ---- direct global -> LDS loaders ---------------------------------------------------------------------------------
+// Every load is a buffer load to LDS (buffer_load_dwordx4 ... lds): the address is a 128-bit buffer descriptor held in
+// scalar registers plus one per-lane byte offset that stays the same for the whole tile plus a scalar offset per
+// instruction, so the K loop spends no vector instructions or registers on addresses. The descriptor's size field does
+// the edge handling: a dword whose offset (lane + scalar part) is not below it is not read and lands in LDS as zero.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const uint16_t* p, uint32_t bytes) {
+    // stride 0 (raw buffer), 32-bit data format
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint32_t uniform(uint32_t x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ uint64_t uniform(uint64_t x) {
+    return ((uint64_t)uniform((uint32_t)(x >> 32)) << 32) | uniform((uint32_t)x);
+}
+constexpr uint32_t kOutOfRange = 0x80000000u;  // lane offset no descriptor of this kernel reaches (sizes stay < 2^31)
+
+// Operand with the reduction dimension contiguous: tile [256 rows][64 k]. A wavefront instruction moves 8 physical rows
+// (1 KB); NI instructions per wavefront and K step. SPLIT: tile rows 128..255 come from a second row range (base1).
+template <int NW, bool SPLIT>
 struct LoaderK {
     static constexpr int NI = 32 / NW;
-    const uint16_t* gp[NI];  // this lane's source of each instruction at k0 = 0
-    uint32_t chunk;          // this lane's logical 16-byte chunk (the same for every instruction: NW is even)
+    static constexpr uint32_t kRowsPerInst = NW * 8;
+    const uint16_t* base0;  // first element of tile row 0
+    const uint16_t* base1;  // SPLIT: first element of tile row 128
+    uint32_t bytes;         // valid bytes from a base: rows inside the operand x row pitch
+    uint32_t ldb;           // row pitch in bytes
+    uint32_t voff;          // this lane's offset: its row of instruction 0, its 16-byte chunk
+    uint32_t chunk;         // this lane's logical chunk (the same for every instruction)
     uint32_t kdim;
     uint32_t wave;
 
-    // row_of(r): global row index of tile row r (already clamped into the valid range)
-    template <typename RowFn>
-    __device__ __forceinline__ void setup(const uint16_t* base, uint64_t ld, uint32_t kdim_, uint32_t wave_,
-                                          uint32_t lane, RowFn row_of) {
+    // rows_valid: rows of the tile (of each half when SPLIT) that exist in the operand; the rest arrives as zeros
+    __device__ __forceinline__ void setup(const uint16_t* b0, const uint16_t* b1, uint32_t rows_valid, uint32_t kdim_,
+                                          uint32_t wave_, uint32_t lane) {
         static_assert(NW % 2 == 0, "chunk is per lane only for an even number of wavefronts");
+        base0 = b0;
+        base1 = b1;
         kdim = kdim_;
         wave = wave_;
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const uint32_t pr = (uint32_t)(i * NW + wave_) * 8u + (lane >> 3);
-            const uint32_t r = logical_row(pr);
-            chunk = (lane & 7u) ^ (r & 7u);
-            gp[i] = base + (uint64_t)row_of(r) * ld + chunk * 8u;
-        }
+        ldb = kdim_ * 2u;
+        bytes = rows_valid * ldb;
+        const uint32_t r = logical_row(wave_ * 8u + (lane >> 3));
+        chunk = (lane & 7u) ^ (r & 7u);
+        voff = r * ldb + chunk * 16u;
     }
 
-    __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0, uint32_t lane) const {
-        if (k0 + BK <= kdim) {
+    __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0) const {
+        uint32_t v = voff;
+        // last, partial K step: chunks past the end of K are pushed out of range, which zero-fills them
+        if (k0 + BK > kdim && k0 + chunk * 8u >= kdim) v = kOutOfRange;
+        const __amdgpu_buffer_rsrc_t r0 = make_rsrc(base0, bytes);
+        const __amdgpu_buffer_rsrc_t r1 = make_rsrc(SPLIT ? base1 : base0, bytes);
 #pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                __builtin_amdgcn_global_load_lds(gp[i] + k0, (lds_void*)(tile + (i * NW + wave) * 1024), 16, 0, 0);
-            }
-        } else {
-            // last, partial K step: chunks past the end of K are zero-filled instead of loaded
-            const bool valid = k0 + chunk * 8u < kdim;
-#pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                uint8_t* dst = tile + (i * NW + wave) * 1024;
-                if (valid) {
-                    __builtin_amdgcn_global_load_lds(gp[i] + k0, (lds_void*)dst, 16, 0, 0);
-                } else {
-                    *reinterpret_cast<uint4*>(dst + lane * 16u) = make_uint4(0, 0, 0, 0);
-                }
-            }
+        for (int i = 0; i < NI; ++i) {
+            const bool second = SPLIT && i >= NI / 2;
+            const uint32_t row = (uint32_t)(second ? i - NI / 2 : i) * kRowsPerInst;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(second ? r1 : r0, (lds_void*)(tile + (i * NW + wave) * 1024), 16, v,
+                                                     k0 * 2u + row * ldb, 0, 0);
         }
     }
 };
 
-// ---- direct global -> LDS loader, operand stored [reduction][out] (out contiguous): tile [64 k][256 out] -------
-// A wavefront instruction moves two k rows (2 x 512 B).
+// Operand stored [reduction][out] (out contiguous): tile [64 k][256 out]. A wavefront instruction moves two k rows
+// (2 x 512 B). Rows past the end of the reduction are out of the descriptor's range (zeros); columns past the end of
+// the operand's rows read whatever follows, which only reaches outputs that are never stored.
 template <int NW>
 struct LoaderT {
     static constexpr int NI = 32 / NW;
-    const uint16_t* gp[NI];  // this lane's source of each instruction at k0 = 0
-    uint64_t ld;
+    const uint16_t* base;  // row 0 of the group's operand, first column of the tile
+    uint32_t ldb;          // row pitch in bytes
+    uint32_t col_bytes;    // byte offset of the tile's first column inside a row
+    uint32_t voff;
     uint32_t kdim;
     uint32_t wave;
-    uint32_t khalf;  // which of the two rows of an instruction this lane loads
 
-    __device__ __forceinline__ void setup(const uint16_t* base, uint64_t ld_, uint32_t kdim_, uint32_t out0,
-                                          uint32_t out_total, uint32_t wave_, uint32_t lane) {
-        ld = ld_;
+    __device__ __forceinline__ void setup(const uint16_t* group_base, uint32_t ld, uint32_t kdim_, uint32_t out0,
+                                          uint32_t wave_, uint32_t lane) {
+        base = group_base + out0;
+        ldb = ld * 2u;
+        col_bytes = out0 * 2u;
         kdim = kdim_;
         wave = wave_;
-        khalf = lane >> 5;
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const uint32_t krow = (uint32_t)(i * NW + wave_) * 2u + khalf;
-            const uint32_t chunk = (lane & 31u) ^ (4u * (krow & 3u));
-            uint32_t col = out0 + chunk * 8u;
-            if (col + 8u > out_total) col = out_total - 8u;  // columns past the edge: results are never stored
-            gp[i] = base + (uint64_t)krow * ld_ + col;
-        }
+        const uint32_t khalf = lane >> 5;  // which of the two rows of an instruction this lane loads
+        const uint32_t krow = wave_ * 2u + khalf;
+        voff = khalf * ldb + (((lane & 31u) ^ (4u * (krow & 3u))) << 4);
     }
 
-    __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0, uint32_t lane) const {
-        const uint64_t adv = (uint64_t)k0 * ld;
-        if (k0 + BK <= kdim) {
+    __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0) const {
+        // rows of this K step that exist (none at all when the step lies past the end: everything is zero-filled)
+        const uint32_t rows = k0 >= kdim ? 0u : (kdim - k0 < (uint32_t)BK ? kdim - k0 : (uint32_t)BK);
+        const __amdgpu_buffer_rsrc_t r = make_rsrc(base + (uint64_t)k0 * (ldb / 2u), rows ? rows * ldb - col_bytes : 0u);
 #pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                __builtin_amdgcn_global_load_lds(gp[i] + adv, (lds_void*)(tile + (i * NW + wave) * 1024), 16, 0, 0);
-            }
-        } else {
-            // last, partial K step: rows past the end of the reduction are zero-filled instead of loaded
-#pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                uint8_t* dst = tile + (i * NW + wave) * 1024;
-                if (k0 + (uint32_t)(i * NW + wave) * 2u + khalf < kdim) {
-                    __builtin_amdgcn_global_load_lds(gp[i] + adv, (lds_void*)dst, 16, 0, 0);
-                } else {
-                    *reinterpret_cast<uint4*>(dst + lane * 16u) = make_uint4(0, 0, 0, 0);
-                }
-            }
+        for (int i = 0; i < NI; ++i) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(tile + (i * NW + wave) * 1024), 16, voff,
+                                                     (uint32_t)(i * NW + wave) * 2u * ldb, 0, 0);
         }
     }
 };
@@ -263,6 +265,16 @@ __device__ __forceinline__ void interleave_mfma_lds() {
         interleave_mfma_lds<R + 1, MFMAS, READS>();
     } else if constexpr (MFMAS - kPairs > 0) {
         __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - kPairs, 0);
+    }
+}
+
+// Scheduling hint: MFMAS matrix instructions with LOADS buffer loads placed one after each of the first MFMAs.
+template <int R, int MFMAS, int LOADS>
+__device__ __forceinline__ void spread_mfma_vmem() {
+    if constexpr (R < MFMAS) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if constexpr (R < LOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        spread_mfma_vmem<R + 1, MFMAS, LOADS>();
     }
 }
 
@@ -399,7 +411,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             if (s_tile_start[mid + 1] <= v) lo = mid + 1;
             else hi = mid;
         }
-        const uint32_t e = lo;
+        const uint32_t e = uniform(lo);
         const uint32_t Me = group_m(e), Ne = group_n(e), Ke = group_k(e);
         const uint32_t n_span = EPI == EPI_SWIGLU ? Ne / 2 : Ne;  // columns the tile grid runs over
         constexpr uint32_t TN = EPI == EPI_SWIGLU ? BN / 2 : BN;  // of which one tile covers this many
@@ -420,16 +432,19 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         const uint32_t n0 = nt * TN;
 #endif
 
-        const uint16_t* Ae = args.A + s_off_a[e];
-        const uint16_t* Be = args.B + s_off_b[e];
-        const uint64_t off_d = s_off_d[e];
+        const uint64_t off_a = uniform(s_off_a[e]), off_b = uniform(s_off_b[e]);
+        const uint16_t* Ae = args.A + off_a;
+        const uint16_t* Be = args.B + off_b;
+        const uint64_t off_d = uniform(s_off_d[e]);
 
         // 16-byte accesses need: every contiguous dimension a multiple of 8 elements (K for an operand whose
         // reduction dim is contiguous, M / N for one stored reduction-major, N for the output rows) and packed
         // group bases that stayed multiples of 8. A ragged reduction length is fine for reduction-major operands.
-        bool fast = (Ne % 8u == 0) && (s_off_a[e] % 8u == 0) && (s_off_b[e] % 8u == 0) && (off_d % 8u == 0);
-        if (A_KC || B_KC) fast = fast && (Ke % 8u == 0);
-        if (!A_KC) fast = fast && (Me % 8u == 0);
+        // The loaders address a tile with 32-bit byte offsets below 2^31: 256 rows of K elements, or 64 rows of M / N.
+        bool fast = (Ne % 8u == 0) && (off_a % 8u == 0) && (off_b % 8u == 0) && (off_d % 8u == 0);
+        if (A_KC || B_KC) fast = fast && (Ke % 8u == 0) && (Ke < (1u << 21));
+        if (!A_KC) fast = fast && (Me % 8u == 0) && (Me < (1u << 23));
+        if (!B_KC) fast = fast && (Ne < (1u << 23));
         if (EPI == EPI_SWIGLU) fast = fast && (n_span % 8u == 0);
 
         __syncthreads();  // every wavefront is done with the previous tile's LDS stages
@@ -442,40 +457,33 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         }
 
         // ---- loaders ----
-        LoaderK<NW> lk_a, lk_b;
+        LoaderK<NW, false> lk_a;
+        LoaderK<NW, EPI == EPI_SWIGLU> lk_b;
         LoaderT<NW> lt_a, lt_b;
         if constexpr (A_KC) {
-            lk_a.setup(Ae, Ke, Ke, wave, lane, [&](uint32_t r) {
-                const uint32_t m = m0 + r;
-                return m < Me ? m : Me - 1;
-            });
+            lk_a.setup(Ae + (uint64_t)m0 * Ke, nullptr, Me - m0 < (uint32_t)BM ? Me - m0 : (uint32_t)BM, Ke, wave, lane);
         } else {
-            lt_a.setup(Ae, Me, Ke, m0, Me, wave, lane);
+            lt_a.setup(Ae, Me, Ke, m0, wave, lane);
         }
         if constexpr (B_KC) {
-            lk_b.setup(Be, Ke, Ke, wave, lane, [&](uint32_t r) {
-                uint32_t n;
-                if constexpr (EPI == EPI_SWIGLU) {
-                    // rows 0..127: "up" rows n0 + r; rows 128..255: "gate" rows I + n0 + (r - 128)
-                    const uint32_t c = n0 + (r & (BN / 2 - 1));
-                    n = (c < n_span ? c : n_span - 1) + (r >= BN / 2 ? n_span : 0u);
-                } else {
-                    n = n0 + r;
-                    n = n < Ne ? n : Ne - 1;
-                }
-                return n;
-            });
+            if constexpr (EPI == EPI_SWIGLU) {
+                // tile rows 0..127: "up" rows n0.. of the weight; rows 128..255: "gate" rows I + n0..
+                const uint32_t rows = n_span - n0 < (uint32_t)(BN / 2) ? n_span - n0 : (uint32_t)(BN / 2);
+                lk_b.setup(Be + (uint64_t)n0 * Ke, Be + (uint64_t)(n_span + n0) * Ke, rows, Ke, wave, lane);
+            } else {
+                lk_b.setup(Be + (uint64_t)n0 * Ke, nullptr, Ne - n0 < (uint32_t)BN ? Ne - n0 : (uint32_t)BN, Ke, wave, lane);
+            }
         } else {
-            lt_b.setup(Be, Ne, Ke, n0, Ne, wave, lane);
+            lt_b.setup(Be, Ne, Ke, n0, wave, lane);
         }
         auto issue = [&](int stage, uint32_t k0) {
 #if defined(FMA_EXPERIMENT_SKIP_LOADS)
             if (k0 >= 2 * BK) return;  // diagnostic build: steady-state loads removed (results are wrong)
 #endif
-            if constexpr (A_KC) lk_a.issue(stage ? s_a1 : s_a0, k0, lane);
-            else lt_a.issue(stage ? s_a1 : s_a0, k0, lane);
-            if constexpr (B_KC) lk_b.issue(stage ? s_b1 : s_b0, k0, lane);
-            else lt_b.issue(stage ? s_b1 : s_b0, k0, lane);
+            if constexpr (A_KC) lk_a.issue(stage ? s_a1 : s_a0, k0);
+            else lt_a.issue(stage ? s_a1 : s_a0, k0);
+            if constexpr (B_KC) lk_b.issue(stage ? s_b1 : s_b0, k0);
+            else lt_b.issue(stage ? s_b1 : s_b0, k0);
         };
 
         f32x16 acc[FM][FN];
@@ -536,16 +544,12 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             // unconditional (after the last step the fragments are simply not used): straight-line code lets the
             // compiler count outstanding LDS reads exactly, so the MFMAs below do not wait for these reads
             load_frags(stage ^ 1, 0, 0);
-            // The loads of step kt+2 go out before the last MFMA group for NT (a quarter of a step more time in flight:
-            // measured +2.5 points of peak) and after it for the other layouts (NN measured -1.5, TN within noise).
-            constexpr bool kIssueEarly = A_KC && B_KC;
-            if constexpr (kIssueEarly) {
-                if (kt + 2 < KT) issue(stage, (kt + 2) * BK);
-            }
+            // the loads of step kt+2 go out one per MFMA (a burst of loads stalls the wavefront's instruction issue);
+            // past the end of K they are all out of range (zero-fill), which keeps the loop body free of branches
+            issue(stage, (kt + 2) * BK);
             mma(1);
-            if constexpr (!kIssueEarly) {
-                if (kt + 2 < KT) issue(stage, (kt + 2) * BK);
-            }
+            __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
+            spread_mfma_vmem<0, FM * FN, 2 * (32 / NW)>();
         };
         if (KT > 0) {
             issue(0, 0);
@@ -558,18 +562,26 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                 step(0, kt);
                 if (kt + 1 < KT) step(1, kt + 1);
             }
+            // the zero-fill loads issued past the end of K must have landed before the stages are reused below
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
         }
 
         // ---- epilogue ----
         // Past the last barrier of the K loop nobody reads the LDS stages any more; each wavefront takes its own 16 KB
         // slice of them as staging space (the barrier at the top of the next tile keeps the next loads away from it).
         // A lane holds row (lane & 31), columns q*8 + (lane >> 5)*4 + 0..3 of each 32x32 accumulator block.
-        static_assert(WM * WN * 2 == 16384 && NW == 8, "staging slices are sized for eight 128x64 wave tiles");
+        static_assert((WM * WN * 2 == 16384 && NW == 8) || (WM * WN * 2 == 32768 && NW == 4),
+                      "staging slices are sized for eight 128x64 or four 128x128 wave tiles");
         // the lane id is made opaque here so that the epilogue's per-lane address arithmetic is redone per tile instead
         // of being hoisted out of the tile loop, where it would occupy registers throughout the K loop
         uint32_t el = lane;
         asm volatile("" : "+v"(el));
-        uint8_t* const img = (wave < 2 ? s_a0 : wave < 4 ? s_b0 : wave < 6 ? s_a1 : s_b1) + (wave & 1u) * 16384u;
+        constexpr uint32_t kPerArray = NW / 4;  // wavefronts that share one 32 KB stage array
+        const uint32_t arr = wave / kPerArray;
+        uint8_t* const img = (arr == 0 ? s_a0 : arr == 1 ? s_b0 : arr == 2 ? s_a1 : s_b1) +
+                             (wave % kPerArray) * (uint32_t)(WM * WN * 2);
         const float alpha = args.alpha;
         const uint32_t row0 = m0 + wm * WM;  // first output row of this wavefront
         if constexpr (EPI == EPI_PLAIN) {
