@@ -538,7 +538,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             mma(0);
             interleave_reads();
             // every load of step kt+1 has landed and every LDS read of this stage has returned
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(0x0070);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             // unconditional (after the last step the fragments are simply not used): straight-line code lets the
@@ -554,16 +554,20 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         if (KT > 0) {
             issue(0, 0);
             if (KT > 1) issue(1, BK);
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(0x0070);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             load_frags(0, 0, 0);
-            for (uint32_t kt = 0; kt < KT; kt += 2) {
+            // two steps per iteration without a branch between them (a branch there makes the compiler wait for the
+            // loads in flight before every LDS read at the top of the loop); an odd last step is peeled
+            uint32_t kt = 0;
+            for (; kt + 1 < KT; kt += 2) {
                 step(0, kt);
-                if (kt + 1 < KT) step(1, kt + 1);
+                step(1, kt + 1);
             }
+            if (kt < KT) step(0, kt);
             // the zero-fill loads issued past the end of K must have landed before the stages are reused below
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(0x0f70);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
         }
