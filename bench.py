@@ -31,6 +31,13 @@ WORKLOADS = {
 }
 
 
+# Bytes per launch of the up-projection forward kernel crossing the L2 <-> fabric boundary, from two rocprofv3 --pmc runs
+# (FETCH_SIZE 6.7125e6 KiB, WRITE_SIZE 2.8927e6 KiB per dispatch) scaled by what the same counters read for a 1 GiB
+# device copy (FETCH_SIZE 0.50, WRITE_SIZE 1.00 of the true bytes); profiles/grouped_gemm_mixtral_counters.txt holds
+# the runs. Measured for the mixtral workload only.
+MEASURED_TRAFFIC_BYTES = {"mixtral": (2 * 6.7125e6 + 2.8927e6) * 1024}
+
+
 def parse_args():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
@@ -279,7 +286,7 @@ def main():
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": dominant["frac"],
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
         }
         del xg, h, a, o, dh, y, d_o, da, dxg, dw1, dw2, blk
 
