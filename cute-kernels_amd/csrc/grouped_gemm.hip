@@ -1,5 +1,5 @@
-// Grouped GEMM over ragged expert groups for gfx950: bf16 operands, fp32 accumulation on the matrix cores
-// (v_mfma_f32_32x32x16_bf16), optional SwiGLU epilogue.
+// Grouped GEMM over ragged expert groups for gfx950: bf16 or fp16 operands, fp32 accumulation on the matrix cores
+// (v_mfma_f32_32x32x16_bf16 / _f16), optional SwiGLU epilogue.
 //
 // Shape of the kernel
 //  * Persistent: the grid is one workgroup per compute unit. Each workgroup builds the group table (tile
@@ -79,16 +79,37 @@ __device__ __forceinline__ uint32_t mc_frag_off(uint32_t r0, uint32_t lane) {
     return (8u * (g >> 1) + kr) * kTRowBytes + ((chunk ^ (4u * kr)) << 4) + (q & 1u) * 8u;
 }
 
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    f32x2 f = {lo, hi};
-    bf16x2 b = __builtin_convertvector(f, bf16x2);
-    return __builtin_bit_cast(uint32_t, b);
-}
+// ---- the two 16-bit element types: conversions and the matrix instruction ------------------------------------------
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 
-__device__ __forceinline__ float round_bf16(float x) {
-    const __bf16 b = (__bf16)x;
-    return (float)b;
-}
+struct ElemBf16 {
+    using frag = bf16x8;
+    using act_t = bf16_t;  // selects the activation's arithmetic (the one swiglu_forward uses for this dtype)
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {  // round to nearest even, lo in the low half
+        f32x2 f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+    }
+    static __device__ __forceinline__ float round(float x) { return (float)(__bf16)x; }
+    static __device__ __forceinline__ float from_bits(uint16_t b) { return bf16_bits_to_float(b); }
+    static __device__ __forceinline__ f32x16 mfma(frag a, frag b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+
+struct ElemF16 {
+    using frag = f16x8;
+    using act_t = f16_t;
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        f32x2 f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+    }
+    static __device__ __forceinline__ float round(float x) { return (float)(_Float16)x; }
+    static __device__ __forceinline__ float from_bits(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+    static __device__ __forceinline__ f32x16 mfma(frag a, frag b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
 
 // ---- direct global -> LDS loaders ---------------------------------------------------------------------------------
 // Every load is a buffer load to LDS (buffer_load_dwordx4 ... lds): the address is a 128-bit buffer descriptor held in
@@ -188,13 +209,12 @@ struct LoaderT {
     }
 };
 
-__device__ __forceinline__ bf16x8 read_kc_frag(const uint8_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ s16x8 read_kc_frag(const uint8_t* p) { return *reinterpret_cast<const s16x8*>(p); }
 
-__device__ __forceinline__ bf16x8 read_tr_frag(const uint8_t* p) {
+__device__ __forceinline__ s16x8 read_tr_frag(const uint8_t* p) {
     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p);
     const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p + 4 * kTRowBytes));
-    const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(bf16x8, v);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
 // ---- epilogue staging: a wavefront transposes its accumulator sub-tile through a private 16 KB slice of LDS ----
@@ -279,7 +299,7 @@ __device__ __forceinline__ void spread_mfma_vmem() {
 }
 
 // Slow, layout-agnostic path for a group whose contiguous dimensions are not multiples of 8 elements.
-template <bool A_KC, bool B_KC>
+template <typename EL, bool A_KC, bool B_KC>
 __device__ void scalar_tile(const uint16_t* Ae, const uint16_t* Be, uint16_t* De, uint32_t Me, uint32_t Ne,
                             uint32_t Ke, uint32_t m0, uint32_t n0, float alpha, uint32_t nthreads) {
     for (uint32_t idx = threadIdx.x; idx < (uint32_t)(BM * BN); idx += nthreads) {
@@ -290,13 +310,13 @@ __device__ void scalar_tile(const uint16_t* Ae, const uint16_t* Be, uint16_t* De
         for (uint32_t k = 0; k < Ke; ++k) {
             const uint16_t a = A_KC ? Ae[(uint64_t)m * Ke + k] : Ae[(uint64_t)k * Me + m];
             const uint16_t b = B_KC ? Be[(uint64_t)n * Ke + k] : Be[(uint64_t)k * Ne + n];
-            acc = fmaf(bf16_bits_to_float(a), bf16_bits_to_float(b), acc);
+            acc = fmaf(EL::from_bits(a), EL::from_bits(b), acc);
         }
-        De[(uint64_t)m * Ne + n] = (uint16_t)(pack_bf16x2(alpha * acc, 0.0f) & 0xffffu);
+        De[(uint64_t)m * Ne + n] = (uint16_t)(EL::pack2(alpha * acc, 0.0f) & 0xffffu);
     }
 }
 
-template <int NWM, int NWN, bool A_KC, bool B_KC, int EPI>
+template <typename EL, int NWM, int NWN, bool A_KC, bool B_KC, int EPI>
 __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmArgs args) {
     constexpr int NW = NWM * NWN;
     constexpr int NT = NW * 64;
@@ -451,7 +471,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
 
         if (!fast) {
             if constexpr (EPI == EPI_PLAIN) {
-                scalar_tile<A_KC, B_KC>(Ae, Be, args.D + off_d, Me, Ne, Ke, m0, n0, args.alpha, NT);
+                scalar_tile<EL, A_KC, B_KC>(Ae, Be, args.D + off_d, Me, Ne, Ke, m0, n0, args.alpha, NT);
             }
             continue;
         }
@@ -495,19 +515,19 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                 for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.0f;
 
         // MFMA operand fragments of one 16-wide k slice, double buffered in registers
-        bf16x8 fa[2][FM], fb[2][FN];
+        typename EL::frag fa[2][FM], fb[2][FN];
         auto load_frags = [&](int stage, int ks, int buf) {
             const uint8_t* ta = stage ? s_a1 : s_a0;
             const uint8_t* tb = stage ? s_b1 : s_b0;
 #pragma unroll
             for (int i = 0; i < FM; ++i) {
-                if constexpr (A_KC) fa[buf][i] = read_kc_frag(ta + a_off[i] + kc_slice[ks]);
-                else fa[buf][i] = read_tr_frag(ta + a_off[i] + ks * 16 * kTRowBytes);
+                if constexpr (A_KC) fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_kc_frag(ta + a_off[i] + kc_slice[ks]));
+                else fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_tr_frag(ta + a_off[i] + ks * 16 * kTRowBytes));
             }
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
-                if constexpr (B_KC) fb[buf][j] = read_kc_frag(tb + b_off[j] + kc_slice[ks]);
-                else fb[buf][j] = read_tr_frag(tb + b_off[j] + ks * 16 * kTRowBytes);
+                if constexpr (B_KC) fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_kc_frag(tb + b_off[j] + kc_slice[ks]));
+                else fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_tr_frag(tb + b_off[j] + ks * 16 * kTRowBytes));
             }
         };
         auto mma = [&](int buf) {
@@ -515,7 +535,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             for (int i = 0; i < FM; ++i)
 #pragma unroll
                 for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = EL::mfma(fb[buf][j], fa[buf][i], acc[i][j]);
         };
         // ask the scheduler to alternate the MFMAs of one slice with the LDS reads of the next
         constexpr int kReads = (A_KC ? FM : 2 * FM) + (B_KC ? FN : 2 * FN);
@@ -596,8 +616,8 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         uint2 w;
-                        w.x = pack_bf16x2(alpha * acc[i][j][q * 4 + 0], alpha * acc[i][j][q * 4 + 1]);
-                        w.y = pack_bf16x2(alpha * acc[i][j][q * 4 + 2], alpha * acc[i][j][q * 4 + 3]);
+                        w.x = EL::pack2(alpha * acc[i][j][q * 4 + 0], alpha * acc[i][j][q * 4 + 1]);
+                        w.y = EL::pack2(alpha * acc[i][j][q * 4 + 2], alpha * acc[i][j][q * 4 + 3]);
                         stage_put<WN * 2>(img, i * 32 + (el & 31u), j * 32 + q * 8 + (el >> 5) * 4, w);
                     }
             stage_flush<WN * 2, WM>(img, args.D + off_d, Ne, row0, Me, n0 + wn * WN, Ne, el);
@@ -617,24 +637,24 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                         float u[4], g[4], y[4];
 #pragma unroll
                         for (int x = 0; x < 4; ++x) {
-                            u[x] = round_bf16(alpha * acc[i][j][q * 4 + x]);
-                            g[x] = round_bf16(alpha * acc[i][j + FN / 2][q * 4 + x]);
-                            y[x] = u[x] * g[x] * sigmoid_for<bf16_t>(g[x]);
+                            u[x] = EL::round(alpha * acc[i][j][q * 4 + x]);
+                            g[x] = EL::round(alpha * acc[i][j + FN / 2][q * 4 + x]);
+                            y[x] = u[x] * g[x] * sigmoid_for<typename EL::act_t>(g[x]);
                         }
                         const uint32_t m = i * 32 + (el & 31u);
                         const uint32_t c = j * 32 + q * 8 + (el >> 5) * 4;
                         uint2 wy;
-                        wy.x = pack_bf16x2(y[0], y[1]);
-                        wy.y = pack_bf16x2(y[2], y[3]);
+                        wy.x = EL::pack2(y[0], y[1]);
+                        wy.y = EL::pack2(y[2], y[3]);
                         // the packed activation waits in two accumulator registers until h has left the staging slice
                         acc[i][j][q * 4 + 0] = __uint_as_float(wy.x);
                         acc[i][j][q * 4 + 1] = __uint_as_float(wy.y);
                         if (He) {
                             uint2 wu, wg;
-                            wu.x = pack_bf16x2(u[0], u[1]);
-                            wu.y = pack_bf16x2(u[2], u[3]);
-                            wg.x = pack_bf16x2(g[0], g[1]);
-                            wg.y = pack_bf16x2(g[2], g[3]);
+                            wu.x = EL::pack2(u[0], u[1]);
+                            wu.y = EL::pack2(u[2], u[3]);
+                            wg.x = EL::pack2(g[0], g[1]);
+                            wg.y = EL::pack2(g[2], g[3]);
                             stage_put<HB>(img, m, c, wu);
                             stage_put<HB>(img, m, WN / 2 + c, wg);
                         }
@@ -664,19 +684,31 @@ constexpr int kWavesM = 2;
 constexpr int kWavesN = FMA_GEMM_WAVES_N;
 
 // every instantiation the entry points launch (explicit, so that host stub and device code are both emitted)
-template __global__ void grouped_gemm_kernel<kWavesM, kWavesN, true, true, EPI_PLAIN>(const GemmArgs);
-template __global__ void grouped_gemm_kernel<kWavesM, kWavesN, true, false, EPI_PLAIN>(const GemmArgs);
-template __global__ void grouped_gemm_kernel<kWavesM, kWavesN, false, true, EPI_PLAIN>(const GemmArgs);
-template __global__ void grouped_gemm_kernel<kWavesM, kWavesN, false, false, EPI_PLAIN>(const GemmArgs);
-template __global__ void grouped_gemm_kernel<kWavesM, kWavesN, true, true, EPI_SWIGLU>(const GemmArgs);
+#define FMA_GEMM_INSTANTIATE(EL)                                                                             \
+    template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, true, true, EPI_PLAIN>(const GemmArgs);  \
+    template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, true, false, EPI_PLAIN>(const GemmArgs); \
+    template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, false, true, EPI_PLAIN>(const GemmArgs); \
+    template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, false, false, EPI_PLAIN>(const GemmArgs); \
+    template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, true, true, EPI_SWIGLU>(const GemmArgs);
+FMA_GEMM_INSTANTIATE(ElemBf16)
+FMA_GEMM_INSTANTIATE(ElemF16)
+#undef FMA_GEMM_INSTANTIATE
 
-template <int NWM, int NWN, bool A_KC, bool B_KC, int EPI>
+template <typename EL, bool A_KC, bool B_KC, int EPI>
 int launch(const GemmArgs& args, hipStream_t st) {
     int cus = num_compute_units();
     if (cus <= 0) cus = 256;
-    hipLaunchKernelGGL((grouped_gemm_kernel<NWM, NWN, A_KC, B_KC, EPI>), dim3((uint32_t)cus), dim3(NWM * NWN * 64), 0,
-                       st, args);
+    hipLaunchKernelGGL((grouped_gemm_kernel<EL, kWavesM, kWavesN, A_KC, B_KC, EPI>), dim3((uint32_t)cus),
+                       dim3(kWavesM * kWavesN * 64), 0, st, args);
     return launch_status("grouped_gemm");
+}
+
+template <typename EL>
+int launch_plain(const GemmArgs& args, bool a_kc, bool b_kc, hipStream_t st) {
+    if (a_kc && b_kc) return launch<EL, true, true, EPI_PLAIN>(args, st);
+    if (a_kc && !b_kc) return launch<EL, true, false, EPI_PLAIN>(args, st);
+    if (!a_kc && b_kc) return launch<EL, false, true, EPI_PLAIN>(args, st);
+    return launch<EL, false, false, EPI_PLAIN>(args, st);
 }
 
 }  // namespace gemm
@@ -689,8 +721,8 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
                      void* stream) {
     using namespace fmahip;
     using namespace fmahip::gemm;
-    FMA_REQUIRE(dtype == FMA_BF16, dtype_bytes(dtype) ? FMA_ERR_UNSUPPORTED : FMA_ERR_BAD_DTYPE,
-                "grouped_gemm: only bf16 operands are implemented (dtype code %d)", dtype);
+    FMA_REQUIRE(dtype == FMA_BF16 || dtype == FMA_F16, dtype_bytes(dtype) ? FMA_ERR_UNSUPPORTED : FMA_ERR_BAD_DTYPE,
+                "grouped_gemm: bf16 and fp16 operands are implemented (dtype code %d)", dtype);
     FMA_REQUIRE(E >= 0, FMA_ERR_BAD_SIZE, "grouped_gemm: negative group count %lld", (long long)E);
     FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "grouped_gemm: E=%lld exceeds the limit %d",
                 (long long)E, FMA_MAX_GROUPS);
@@ -711,18 +743,15 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
     hipStream_t st = (hipStream_t)stream;
     const bool a_kc = trans_a == 0;  // A stored [M, K]: reduction dim contiguous
     const bool b_kc = trans_b != 0;  // B stored [N, K]: reduction dim contiguous
-    if (a_kc && b_kc) return launch<kWavesM, kWavesN, true, true, EPI_PLAIN>(args, st);
-    if (a_kc && !b_kc) return launch<kWavesM, kWavesN, true, false, EPI_PLAIN>(args, st);
-    if (!a_kc && b_kc) return launch<kWavesM, kWavesN, false, true, EPI_PLAIN>(args, st);
-    return launch<kWavesM, kWavesN, false, false, EPI_PLAIN>(args, st);
+    return dtype == FMA_BF16 ? launch_plain<ElemBf16>(args, a_kc, b_kc, st) : launch_plain<ElemF16>(args, a_kc, b_kc, st);
 }
 
 int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, const uint32_t* M_arr, int64_t E,
                             int64_t I, int64_t K, int dtype, void* stream) {
     using namespace fmahip;
     using namespace fmahip::gemm;
-    FMA_REQUIRE(dtype == FMA_BF16, dtype_bytes(dtype) ? FMA_ERR_UNSUPPORTED : FMA_ERR_BAD_DTYPE,
-                "grouped_gemm_swiglu: only bf16 operands are implemented (dtype code %d)", dtype);
+    FMA_REQUIRE(dtype == FMA_BF16 || dtype == FMA_F16, dtype_bytes(dtype) ? FMA_ERR_UNSUPPORTED : FMA_ERR_BAD_DTYPE,
+                "grouped_gemm_swiglu: bf16 and fp16 operands are implemented (dtype code %d)", dtype);
     FMA_REQUIRE(E >= 0, FMA_ERR_BAD_SIZE, "grouped_gemm_swiglu: negative group count %lld", (long long)E);
     FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "grouped_gemm_swiglu: E=%lld exceeds the limit %d",
                 (long long)E, FMA_MAX_GROUPS);
@@ -746,7 +775,8 @@ int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, co
     args.const_n = (uint32_t)(2 * I);
     args.const_k = (uint32_t)K;
     args.alpha = 1.0f;
-    return launch<kWavesM, kWavesN, true, true, EPI_SWIGLU>(args, (hipStream_t)stream);
+    return dtype == FMA_BF16 ? launch<ElemBf16, true, true, EPI_SWIGLU>(args, (hipStream_t)stream)
+                             : launch<ElemF16, true, true, EPI_SWIGLU>(args, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -131,3 +131,45 @@ def test_fused_swiglu_equals_gemm_then_swiglu(M_list, I, K):
     act_only = torch.empty_like(act)
     grouped_gemm_swiglu_cuda(x, w, M, None, act_only)
     assert torch.equal(act_only, act)
+
+
+@pytest.mark.parametrize("tA,tB", [(False, True), (False, False), (True, False), (True, True)])
+def test_fp16_integer_known_answer(tA, tB):
+    # fp16 operands: integers in [-3, 3], K = 200, so every sum (|sum| <= 1800 < 2048) is exact in fp16
+    M_list, N, K = [264, 0, 8, 520, 1000], 264, 200
+    E = len(M_list)
+    g = torch.Generator().manual_seed(11)
+    As = [torch.randint(-3, 4, (K, M) if tA else (M, K), generator=g).to(torch.float16) for M in M_list]
+    Bs = [torch.randint(-3, 4, (N, K) if tB else (K, N), generator=g).to(torch.float16) for _ in M_list]
+    A = torch.cat([a.reshape(-1) for a in As])
+    B = torch.cat([b.reshape(-1) for b in Bs])
+    expect = O.grouped_gemm(A, B, M_list, [N] * E, [K] * E, tA, tB)
+    got = grouped_gemm(
+        A=A.to(DEV), B=B.to(DEV), C=None, M_array=_u32(M_list), N_array=_u32([N] * E), K_array=_u32([K] * E),
+        output_shape=(sum(M_list) * N,), is_A_transposed=tA, is_B_transposed=tB,
+    )
+    assert got.dtype == torch.float16
+    assert float((got.cpu().float() - expect.float()).abs().max()) == 0
+
+
+def test_fp16_random_operands_and_fused_swiglu():
+    # fp16 N(0,1) x 0.1 operands: one fp16 ulp (2^-11) of the largest output against fp32 math; the fused SwiGLU
+    # epilogue equals GEMM followed by swiglu_packed bit for bit, as for bf16
+    torch.manual_seed(6)
+    M_list, I, K = [300, 0, 513, 1], 264, 520
+    E, R = len(M_list), sum(M_list)
+    x = torch.randn(R, K).half().to(DEV)
+    w = (torch.randn(E, 2 * I, K) * 0.1).half().to(DEV)
+    M = _u32(M_list)
+    h_ref = grouped_gemm(
+        A=x, B=w, C=None, M_array=M, N_array=_u32([2 * I] * E), K_array=_u32([K] * E), output_shape=(R, 2 * I),
+        is_A_transposed=False, is_B_transposed=True,
+    )
+    expect = O.grouped_gemm(x.cpu().float(), w.cpu().float(), M_list, [2 * I] * E, [K] * E, False, True).reshape(R, 2 * I)
+    max_rel, frob_rel = rel_err(h_ref, expect)
+    assert max_rel <= 2**-11 and frob_rel <= 2**-11
+    h = torch.empty(R, 2 * I, dtype=torch.float16, device=DEV)
+    act = torch.empty(R, I, dtype=torch.float16, device=DEV)
+    grouped_gemm_swiglu_cuda(x, w, M, h, act)
+    assert torch.equal(h, h_ref)
+    assert torch.equal(act, swiglu_packed(h_ref))

@@ -101,6 +101,26 @@ def test_moe_reference_cases(E, k, H, I, act_name):
         assert max_rel <= 3e-2 and frob_rel <= 1.5e-2, f"{name}: max_rel={max_rel:.4g} frob_rel={frob_rel:.4g}"
 
 
+@pytest.mark.parametrize("act_name", ["swiglu_fused", "glu"])
+def test_moe_fp16(act_name):
+    # the reference's kernel-backend rows in fp16 (tests/modules/moe_test.py:106-150: output atol 4e-3, rtol 0) at T=7;
+    # gradients against the fp32 oracle relative to each tensor's largest value (fp16 has 11 mantissa bits)
+    torch.manual_seed(42)
+    E, k, H, I = 8, 2, 2048, 8192
+    act = {"swiglu_fused": swiglu_packed, "glu": nn.GLU()}[act_name]
+    oracle_act = {"swiglu_fused": O.swiglu_packed, "glu": _glu}[act_name]
+    moe = MoE(E, k, H, I, act, True, False, 0.02).to(torch.float16).to(DEV)
+    x = torch.randn(7, H).half().to(DEV).requires_grad_()
+    y, _ = moe(x, kernel_backend=KernelBackend.cuda)
+    y.sum().backward()
+    got = [y, x.grad, moe.c_fc.weight.grad, moe.c_proj.weight.grad]
+    ref32 = _oracle_grads(moe, x, oracle_act, torch.float32)
+    assert float((y.detach().cpu().float() - ref32[0]).abs().max()) <= 4e-3
+    for name, a, b in zip(["output", "input gradient", "c_fc weight gradient", "c_proj weight gradient"], got, ref32):
+        max_rel, frob_rel = rel_err(a.detach(), b)
+        assert max_rel <= 4e-3 and frob_rel <= 2e-3, f"{name}: max_rel={max_rel:.4g} frob_rel={frob_rel:.4g}"
+
+
 def test_moe_plumbing_config_against_golden_fixture():
     # BASELINE configuration 1 (T=512, H=256, I=512, E=8, k=2): expected values were written by the fp32 oracle
     # (tests/golden/make_golden.py); the HIP path runs it in bf16
