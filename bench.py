@@ -47,6 +47,8 @@ def parse_args():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     p.add_argument("--no-kernels", action="store_true", help="skip the per-kernel measurements")
     p.add_argument("--no-layer", action="store_true", help="skip the whole-layer timing (for short profiler runs)")
+    p.add_argument("--fuse-swiglu", type=int, default=-1, choices=[-1, 0, 1],
+                   help="1 / 0: compute SwiGLU inside / after the up-projection kernel; -1: the module's default")
     p.add_argument("--only", default="", help="comma-separated substrings: measure only the kernels whose name matches")
     return p.parse_args()
 
@@ -108,6 +110,8 @@ def main():
     torch.manual_seed(42)
     with torch.device(dev):
         moe = MoE(E, k, H, I, swiglu_packed, True, False, 0.02).to(torch.bfloat16)
+    if args.fuse_swiglu >= 0:
+        moe.fuse_swiglu = bool(args.fuse_swiglu)
     selected_d = selected.to(dev)
     weights_d = weights.bfloat16().to(dev)
 

@@ -428,7 +428,13 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     const uint32_t per_xcd = grid / kXcds;
     const uint32_t slot = (grid % kXcds == 0) ? (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds : blockIdx.x;
 
-    for (uint32_t v = slot; v < total_tiles; v += grid) {
+    // Rounds of `grid` tiles are dealt in alternating directions (slot s takes tile s of even rounds and tile
+    // grid-1-s of odd ones): when the tiles get cheaper along the tile order (groups with shrinking reduction length, as in
+    // weight gradients under skewed routing) a workgroup that drew an expensive tile in one round draws a cheap one in the
+    // next. Blocks of 32 neighbouring tiles still go to one XCD.
+    for (uint32_t round = 0; round * grid < total_tiles; ++round) {
+        const uint32_t v = round * grid + ((round & 1u) ? grid - 1u - slot : slot);
+        if (v >= total_tiles) continue;
         // ---- which group, which tile ----
         uint32_t lo = 0, hi = E;
         while (lo < hi) {
