@@ -121,6 +121,30 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const uint16_t* p, u
     // stride 0 (raw buffer), 32-bit data format
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, (int)bytes, 0x00020000);
 }
+// The same load written in assembly, with its M0 set-up (M0 holds the LDS address the wavefront's 1 KB goes to). The
+// compiler does not see that it writes LDS, so it places no waits of its own for it: the first loads of a tile are
+// issued this way, partly while the previous tile's epilogue is still running, and waited for with an exact count.
+__device__ __forceinline__ void buffer_load_lds_quiet(u32x4 rsrc, uint32_t voff, uint32_t soff, uint32_t lds_addr) {
+    // M0 is put back afterwards: the compiler keeps its own values in it and does not honour a clobber of it
+    uint32_t saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
+                 "s_mov_b32 m0, %0"
+                 : "=&s"(saved_m0)
+                 : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr));
+}
+__device__ __forceinline__ uint32_t lds_address(const uint8_t* p) {
+    return (uint32_t)(uintptr_t)(lds_void*)const_cast<uint8_t*>(p);
+}
+// the descriptor make_rsrc() builds, as four plain words in scalar registers (p and bytes are the same in every lane)
+__device__ __forceinline__ u32x4 make_rsrc_words(const uint16_t* p, uint32_t bytes) {
+    const uint64_t a = (uint64_t)(uintptr_t)p;
+    u32x4 r;
+    r.x = (uint32_t)a;
+    r.y = (uint32_t)(a >> 32) & 0xffffu;
+    r.z = bytes;
+    r.w = 0x00020000u;
+    return r;
+}
 __device__ __forceinline__ uint32_t uniform(uint32_t x) { return __builtin_amdgcn_readfirstlane(x); }
 __device__ __forceinline__ uint64_t uniform(uint64_t x) {
     return ((uint64_t)uniform((uint32_t)(x >> 32)) << 32) | uniform((uint32_t)x);
@@ -171,6 +195,20 @@ struct LoaderK {
                                                      k0 * 2u + row * ldb, 0, 0);
         }
     }
+    // the same NI loads through buffer_load_lds_quiet
+    __device__ __forceinline__ void issue_quiet(uint8_t* tile, uint32_t k0) const {
+        uint32_t v = voff;
+        if (k0 + BK > kdim && k0 + chunk * 8u >= kdim) v = kOutOfRange;
+        const u32x4 r0 = make_rsrc_words(base0, bytes);
+        const u32x4 r1 = make_rsrc_words(SPLIT ? base1 : base0, bytes);
+        const uint32_t lds0 = lds_address(tile) + wave * 1024u;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const bool second = SPLIT && i >= NI / 2;
+            const uint32_t row = (uint32_t)(second ? i - NI / 2 : i) * kRowsPerInst;
+            buffer_load_lds_quiet(second ? r1 : r0, v, k0 * 2u + row * ldb, lds0 + (uint32_t)(i * NW) * 1024u);
+        }
+    }
 };
 
 // Operand stored [reduction][out] (out contiguous): tile [64 k][256 out]. A wavefront instruction moves two k rows
@@ -208,6 +246,15 @@ struct LoaderT {
                                                      (uint32_t)(i * NW + wave) * 2u * ldb, 0, 0);
         }
     }
+    __device__ __forceinline__ void issue_quiet(uint8_t* tile, uint32_t k0) const {
+        const uint32_t rows = k0 >= kdim ? 0u : (kdim - k0 < (uint32_t)BK ? kdim - k0 : (uint32_t)BK);
+        const u32x4 r = make_rsrc_words(base + (uint64_t)k0 * (ldb / 2u), rows ? rows * ldb - col_bytes : 0u);
+        const uint32_t lds0 = lds_address(tile) + wave * 1024u;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            buffer_load_lds_quiet(r, voff, (uint32_t)(i * NW + wave) * 2u * ldb, lds0 + (uint32_t)(i * NW) * 1024u);
+        }
+    }
 };
 
 __device__ __forceinline__ s16x8 read_kc_frag(const uint8_t* p) { return *reinterpret_cast<const s16x8*>(p); }
@@ -224,10 +271,13 @@ __device__ __forceinline__ s16x8 read_tr_frag(const uint8_t* p) {
 // instruction writes 16 bytes per lane and whole 64- or 128-byte row segments.
 // Row m, 16-byte chunk c of the image sits at m*ROWB + ((c ^ key(m)) << 4), key(m) = (m / rows-per-256-B) mod chunks:
 // the 8-byte writes of 32 consecutive rows conflict at most two ways, the 16-byte reads not at all.
-// 16-byte store with the non-temporal hint: the output tile is not read again by this kernel, and a workgroup's 128 KB
-// of results should not push operand panels out of the L2 (measured: +0.5 to +1.5 points of peak over plain stores)
-__device__ __forceinline__ void store_streaming(uint16_t* p, uint4 v) {
-    __builtin_nontemporal_store(__builtin_bit_cast(u32x4, v), reinterpret_cast<u32x4*>(p));
+// 16-byte buffer store with the non-temporal hint: the output tile is not read again by this kernel, and a workgroup's
+// 128 KB of results should not push operand panels out of the L2 (measured: +0.5 to +1.5 points of peak over plain
+// stores). A lane whose offset is not below the descriptor's size stores nothing, so every lane always executes the
+// instruction: the number of stores a wavefront issues per tile is a compile-time constant, which the wait for the next
+// tile's first loads relies on.
+__device__ __forceinline__ void store_streaming(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint4 v) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc, (int)voff, 0, /*nt*/ 2);
 }
 template <int ROWB>
 __device__ __forceinline__ uint32_t stage_off(uint32_t m, uint32_t chunk16) {
@@ -235,46 +285,62 @@ __device__ __forceinline__ uint32_t stage_off(uint32_t m, uint32_t chunk16) {
     constexpr uint32_t kRowsPer256 = 256 / ROWB;
     return m * ROWB + ((chunk16 ^ ((m / kRowsPer256) & (kChunks - 1))) << 4);
 }
+// A wavefront's staging slice is made of the 1 KB pieces of LDS stage 1 that the wavefront itself fills when it loads
+// operands (pieces wave, wave + NW, ... of the A array, then of the B array), so only its own loads ever overwrite its
+// image and no workgroup barrier is needed between an epilogue and the next tile's loads into stage 1.
+template <int NW>
+struct StagingSlice {
+    uint8_t* a;  // LDS stage 1, A array, this wavefront's first piece
+    uint8_t* b;  // the same of the B array
+    __device__ __forceinline__ uint8_t* at(uint32_t off) const {  // byte `off` of the image
+        constexpr uint32_t kPieces = 32 / NW;                    // pieces per array
+        const uint32_t piece = off >> 10;
+        return (piece < kPieces ? a : b) + (piece % kPieces) * (uint32_t)(NW * 1024) + (off & 1023u);
+    }
+};
 // lane's 4 columns [col, col+4) of image row m
-template <int ROWB>
-__device__ __forceinline__ void stage_put(uint8_t* img, uint32_t m, uint32_t col, uint2 v) {
-    *reinterpret_cast<uint2*>(img + stage_off<ROWB>(m, col >> 3) + ((col >> 2) & 1u) * 8u) = v;
+template <int ROWB, typename Slice>
+__device__ __forceinline__ void stage_put(const Slice& img, uint32_t m, uint32_t col, uint2 v) {
+    *reinterpret_cast<uint2*>(img.at(stage_off<ROWB>(m, col >> 3) + ((col >> 2) & 1u) * 8u)) = v;
 }
-// Stores the image (rows x ROWB/2 columns) to out[(row0 + r) * ld + col0 + c], rows >= row_end and columns >= col_end
-// masked. col0, ld and col_end are multiples of 8 elements, so every 16-byte piece is wholly inside or outside.
-template <int ROWB, int ROWS>
-__device__ __forceinline__ void stage_flush(const uint8_t* img, uint16_t* out, uint64_t ld, uint32_t row0,
-                                            uint32_t row_end, uint32_t col0, uint32_t col_end, uint32_t lane) {
-    constexpr uint32_t kChunks = ROWB / 16;      // 16-byte pieces per image row
+// Stores the image (ROWS rows of ROWB/2 columns) to origin[r * ld + c]; only the first rows_valid rows and cols_valid
+// columns exist in the output (both may be 0). ld and cols_valid are multiples of 8 elements, so every 16-byte piece
+// is wholly inside or outside. Issues exactly ROWS * ROWB / 1024 store instructions.
+template <int ROWB, int ROWS, typename Slice>
+__device__ __forceinline__ void stage_flush(const Slice& img, uint16_t* origin, uint32_t ld, uint32_t rows_valid,
+                                            uint32_t cols_valid, uint32_t lane) {
+    constexpr uint32_t kChunks = ROWB / 16;  // 16-byte pieces per image row
     constexpr uint32_t kRowsPerInst = 64 / kChunks;
     const uint32_t c16 = lane % kChunks;
-    const uint32_t col = col0 + c16 * 8u;
+    const uint32_t ldb = ld * 2u;
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(origin, rows_valid * ldb);
+    const bool col_ok = c16 * 8u < cols_valid;
 #pragma unroll
     for (uint32_t it = 0; it < ROWS / kRowsPerInst; ++it) {
         const uint32_t r = it * kRowsPerInst + lane / kChunks;
-        const uint4 v = *reinterpret_cast<const uint4*>(img + stage_off<ROWB>(r, c16));
-        if (row0 + r < row_end && col < col_end) store_streaming(out + (uint64_t)(row0 + r) * ld + col, v);
+        const uint4 v = *reinterpret_cast<const uint4*>(img.at(stage_off<ROWB>(r, c16)));
+        store_streaming(rsrc, col_ok ? r * ldb + c16 * 16u : kOutOfRange, v);
     }
 }
 
-// Like stage_flush for an image whose row holds two windows of HALF columns each: window 0 goes to columns
-// col0.., window 1 to columns second0 + col0.. of the same output row (the "up" and "gate" halves of h).
-template <int ROWB, int ROWS, int HALF>
-__device__ __forceinline__ void stage_flush_split(const uint8_t* img, uint16_t* out, uint64_t ld, uint32_t row0,
-                                                  uint32_t row_end, uint32_t col0, uint32_t col_end, uint32_t second0,
-                                                  uint32_t lane) {
+// Like stage_flush for an image whose row holds two windows of HALF columns each: window 0 goes to columns 0.. of the
+// origin's row, window 1 to columns second0.. of the same row (the "up" and "gate" halves of h).
+template <int ROWB, int ROWS, int HALF, typename Slice>
+__device__ __forceinline__ void stage_flush_split(const Slice& img, uint16_t* origin, uint32_t ld, uint32_t rows_valid,
+                                                  uint32_t cols_valid, uint32_t second0, uint32_t lane) {
     constexpr uint32_t kChunks = ROWB / 16;
     constexpr uint32_t kRowsPerInst = 64 / kChunks;
     const uint32_t c16 = lane % kChunks;
     const uint32_t in_window = (c16 * 8u) % HALF;
     const uint32_t window = (c16 * 8u) / HALF;
-    const uint32_t col = col0 + in_window;
+    const uint32_t ldb = ld * 2u;
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(origin, rows_valid * ldb);
+    const bool col_ok = in_window < cols_valid;
 #pragma unroll
     for (uint32_t it = 0; it < ROWS / kRowsPerInst; ++it) {
         const uint32_t r = it * kRowsPerInst + lane / kChunks;
-        const uint4 v = *reinterpret_cast<const uint4*>(img + stage_off<ROWB>(r, c16));
-        if (row0 + r < row_end && col < col_end)
-            store_streaming(out + (uint64_t)(row0 + r) * ld + window * second0 + col, v);
+        const uint4 v = *reinterpret_cast<const uint4*>(img.at(stage_off<ROWB>(r, c16)));
+        store_streaming(rsrc, col_ok ? r * ldb + (window * second0 + in_window) * 2u : kOutOfRange, v);
     }
 }
 
@@ -349,9 +415,13 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     const uint32_t wn = wave % NWN;
     const uint32_t E = args.E;
 
-    auto group_m = [&](uint32_t e) { return args.M_arr[e]; };
-    auto group_n = [&](uint32_t e) { return args.N_arr ? args.N_arr[e] : args.const_n; };
-    auto group_k = [&](uint32_t e) { return args.K_arr ? args.K_arr[e] : args.const_k; };
+    // The size arrays are read through the constant address space: with a wavefront-uniform index that is a scalar
+    // load (nothing writes the arrays while the kernel runs), not a vector load that every tile would wait for.
+    typedef const __attribute__((address_space(4))) uint32_t* const_u32_ptr;
+    const const_u32_ptr m_arr = (const_u32_ptr)args.M_arr, n_arr = (const_u32_ptr)args.N_arr, k_arr = (const_u32_ptr)args.K_arr;
+    auto group_m = [&](uint32_t e) { return m_arr[e]; };
+    auto group_n = [&](uint32_t e) { return n_arr ? n_arr[e] : args.const_n; };
+    auto group_k = [&](uint32_t e) { return k_arr ? k_arr[e] : args.const_k; };
     // n-extent covered by the tile grid: for the SwiGLU epilogue a tile spans 128 up + 128 gate columns
     auto tiles_of = [&](uint32_t m, uint32_t n) -> uint32_t {
         if (m == 0 || n == 0) return 0;
@@ -428,14 +498,21 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     const uint32_t per_xcd = grid / kXcds;
     const uint32_t slot = (grid % kXcds == 0) ? (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds : blockIdx.x;
 
+    // Everything that identifies one output tile; the same in every lane.
+    struct Tile {
+        bool valid, fast;
+        uint32_t Me, Ne, Ke, n_span, m0, n0;
+        uint64_t off_a, off_b, off_d;
+    };
+    constexpr uint32_t TN = EPI == EPI_SWIGLU ? BN / 2 : BN;  // columns of the tile grid one tile covers
     // Rounds of `grid` tiles are dealt in alternating directions (slot s takes tile s of even rounds and tile
     // grid-1-s of odd ones): when the tiles get cheaper along the tile order (groups with shrinking reduction length, as in
     // weight gradients under skewed routing) a workgroup that drew an expensive tile in one round draws a cheap one in the
-    // next. Blocks of 32 neighbouring tiles still go to one XCD.
-    for (uint32_t round = 0; round * grid < total_tiles; ++round) {
+    // next. Blocks of 32 neighbouring tiles still go to one XCD. Only the last round can leave a slot without a tile.
+    auto lookup = [&](uint32_t round) -> Tile {
+        Tile t{};
         const uint32_t v = round * grid + ((round & 1u) ? grid - 1u - slot : slot);
-        if (v >= total_tiles) continue;
-        // ---- which group, which tile ----
+        if ((uint64_t)round * grid >= total_tiles || v >= total_tiles) return t;
         uint32_t lo = 0, hi = E;
         while (lo < hi) {
             const uint32_t mid = (lo + hi) >> 1;
@@ -443,80 +520,119 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             else hi = mid;
         }
         const uint32_t e = uniform(lo);
-        const uint32_t Me = group_m(e), Ne = group_n(e), Ke = group_k(e);
-        const uint32_t n_span = EPI == EPI_SWIGLU ? Ne / 2 : Ne;  // columns the tile grid runs over
-        constexpr uint32_t TN = EPI == EPI_SWIGLU ? BN / 2 : BN;  // of which one tile covers this many
-        const uint32_t tiles_m = (Me + BM - 1) / BM;
-        const uint32_t tiles_n = (n_span + TN - 1) / TN;
-        const uint32_t local = v - s_tile_start[e];
+        t.valid = true;
+        t.Me = group_m(e);
+        t.Ne = group_n(e);
+        t.Ke = group_k(e);
+        t.n_span = EPI == EPI_SWIGLU ? t.Ne / 2 : t.Ne;  // columns the tile grid runs over
+        const uint32_t tiles_m = (t.Me + BM - 1) / BM;
+        const uint32_t tiles_n = (t.n_span + TN - 1) / TN;
+        const uint32_t local = v - uniform(s_tile_start[e]);
         const uint32_t band = kGroupM * tiles_n;
         const uint32_t first_m = (local / band) * kGroupM;
         const uint32_t band_m = tiles_m - first_m < (uint32_t)kGroupM ? tiles_m - first_m : (uint32_t)kGroupM;
         const uint32_t mt = first_m + (local % band) % band_m;
         const uint32_t nt = (local % band) / band_m;
 #if defined(FMA_EXPERIMENT_SAME_TILE)
-        const uint32_t m0 = 0, n0 = 0;  // diagnostic build: every workgroup reads the same, cache-resident tile
+        t.m0 = 0, t.n0 = 0;  // diagnostic build: every workgroup reads the same, cache-resident tile
         (void)mt;
         (void)nt;
 #else
-        const uint32_t m0 = mt * BM;
-        const uint32_t n0 = nt * TN;
+        t.m0 = mt * BM;
+        t.n0 = nt * TN;
 #endif
-
-        const uint64_t off_a = uniform(s_off_a[e]), off_b = uniform(s_off_b[e]);
-        const uint16_t* Ae = args.A + off_a;
-        const uint16_t* Be = args.B + off_b;
-        const uint64_t off_d = uniform(s_off_d[e]);
-
+        t.off_a = uniform(s_off_a[e]);
+        t.off_b = uniform(s_off_b[e]);
+        t.off_d = uniform(s_off_d[e]);
         // 16-byte accesses need: every contiguous dimension a multiple of 8 elements (K for an operand whose
         // reduction dim is contiguous, M / N for one stored reduction-major, N for the output rows) and packed
         // group bases that stayed multiples of 8. A ragged reduction length is fine for reduction-major operands.
-        // The loaders address a tile with 32-bit byte offsets below 2^31: 256 rows of K elements, or 64 rows of M / N.
-        bool fast = (Ne % 8u == 0) && (off_a % 8u == 0) && (off_b % 8u == 0) && (off_d % 8u == 0);
-        if (A_KC || B_KC) fast = fast && (Ke % 8u == 0) && (Ke < (1u << 21));
-        if (!A_KC) fast = fast && (Me % 8u == 0) && (Me < (1u << 23));
-        if (!B_KC) fast = fast && (Ne < (1u << 23));
-        if (EPI == EPI_SWIGLU) fast = fast && (n_span % 8u == 0);
+        // Loads and stores address a tile with 32-bit byte offsets below 2^31: 256 rows of K elements, 64 rows of M / N.
+        bool fast = (t.Ne % 8u == 0) && (t.Ne < (1u << 23)) && (t.off_a % 8u == 0) && (t.off_b % 8u == 0) &&
+                    (t.off_d % 8u == 0);
+        if (A_KC || B_KC) fast = fast && (t.Ke % 8u == 0) && (t.Ke < (1u << 21));
+        if (!A_KC) fast = fast && (t.Me % 8u == 0) && (t.Me < (1u << 23));
+        if (EPI == EPI_SWIGLU) fast = fast && (t.n_span % 8u == 0);
+        t.fast = fast;
+        return t;
+    };
 
-        __syncthreads();  // every wavefront is done with the previous tile's LDS stages
-
-        if (!fast) {
-            if constexpr (EPI == EPI_PLAIN) {
-                scalar_tile<EL, A_KC, B_KC>(Ae, Be, args.D + off_d, Me, Ne, Ke, m0, n0, args.alpha, NT);
-            }
-            continue;
-        }
-
-        // ---- loaders ----
-        LoaderK<NW, false> lk_a;
-        LoaderK<NW, EPI == EPI_SWIGLU> lk_b;
-        LoaderT<NW> lt_a, lt_b;
+    // ---- loaders (state of the tile whose operands are being loaded) ----
+    LoaderK<NW, false> lk_a;
+    LoaderK<NW, EPI == EPI_SWIGLU> lk_b;
+    LoaderT<NW> lt_a, lt_b;
+    auto setup_loaders = [&](const Tile& t) {
+        const uint16_t* Ae = args.A + t.off_a;
+        const uint16_t* Be = args.B + t.off_b;
         if constexpr (A_KC) {
-            lk_a.setup(Ae + (uint64_t)m0 * Ke, nullptr, Me - m0 < (uint32_t)BM ? Me - m0 : (uint32_t)BM, Ke, wave, lane);
+            lk_a.setup(Ae + (uint64_t)t.m0 * t.Ke, nullptr, t.Me - t.m0 < (uint32_t)BM ? t.Me - t.m0 : (uint32_t)BM, t.Ke,
+                       wave, lane);
         } else {
-            lt_a.setup(Ae, Me, Ke, m0, wave, lane);
+            lt_a.setup(Ae, t.Me, t.Ke, t.m0, wave, lane);
         }
         if constexpr (B_KC) {
             if constexpr (EPI == EPI_SWIGLU) {
                 // tile rows 0..127: "up" rows n0.. of the weight; rows 128..255: "gate" rows I + n0..
-                const uint32_t rows = n_span - n0 < (uint32_t)(BN / 2) ? n_span - n0 : (uint32_t)(BN / 2);
-                lk_b.setup(Be + (uint64_t)n0 * Ke, Be + (uint64_t)(n_span + n0) * Ke, rows, Ke, wave, lane);
+                const uint32_t rows = t.n_span - t.n0 < (uint32_t)(BN / 2) ? t.n_span - t.n0 : (uint32_t)(BN / 2);
+                lk_b.setup(Be + (uint64_t)t.n0 * t.Ke, Be + (uint64_t)(t.n_span + t.n0) * t.Ke, rows, t.Ke, wave, lane);
             } else {
-                lk_b.setup(Be + (uint64_t)n0 * Ke, nullptr, Ne - n0 < (uint32_t)BN ? Ne - n0 : (uint32_t)BN, Ke, wave, lane);
+                lk_b.setup(Be + (uint64_t)t.n0 * t.Ke, nullptr, t.Ne - t.n0 < (uint32_t)BN ? t.Ne - t.n0 : (uint32_t)BN,
+                           t.Ke, wave, lane);
             }
         } else {
-            lt_b.setup(Be, Ne, Ke, n0, wave, lane);
+            lt_b.setup(Be, t.Ne, t.Ke, t.n0, wave, lane);
         }
-        auto issue = [&](int stage, uint32_t k0) {
+    };
+    // loads of the K step at k0 into `stage`: inside the K loop (compiler-visible, placed by the scheduling hints) ...
+    auto issue = [&](int stage, uint32_t k0) {
 #if defined(FMA_EXPERIMENT_SKIP_LOADS)
-            if (k0 >= 2 * BK) return;  // diagnostic build: steady-state loads removed (results are wrong)
+        if (k0 >= 2 * BK) return;  // diagnostic build: steady-state loads removed (results are wrong)
 #endif
-            if constexpr (A_KC) lk_a.issue(stage ? s_a1 : s_a0, k0);
-            else lt_a.issue(stage ? s_a1 : s_a0, k0);
-            if constexpr (B_KC) lk_b.issue(stage ? s_b1 : s_b0, k0);
-            else lt_b.issue(stage ? s_b1 : s_b0, k0);
-        };
+        if constexpr (A_KC) lk_a.issue(stage ? s_a1 : s_a0, k0);
+        else lt_a.issue(stage ? s_a1 : s_a0, k0);
+        if constexpr (B_KC) lk_b.issue(stage ? s_b1 : s_b0, k0);
+        else lt_b.issue(stage ? s_b1 : s_b0, k0);
+    };
+    // ... and at the head of a tile
+    auto issue_quiet = [&](int stage, uint32_t k0) {
+        if constexpr (A_KC) lk_a.issue_quiet(stage ? s_a1 : s_a0, k0);
+        else lt_a.issue_quiet(stage ? s_a1 : s_a0, k0);
+        if constexpr (B_KC) lk_b.issue_quiet(stage ? s_b1 : s_b0, k0);
+        else lt_b.issue_quiet(stage ? s_b1 : s_b0, k0);
+    };
+    constexpr uint32_t kStepLoads = 2 * (32 / NW);  // load instructions per wavefront and K step
+    // store instructions per wavefront and tile (stage_flush issues a fixed number)
+    const uint32_t tile_stores = EPI == EPI_PLAIN ? WM * WN * 2 / 1024 : (args.D ? WM * WN * 2 / 1024 : 0) + WM * WN / 1024;
+    // waits until at most n of this wavefront's loads and stores are outstanding (they complete in issue order)
+    auto wait_outstanding = [&](uint32_t n) {
+        if (n >= 40) __builtin_amdgcn_s_waitcnt(0x8f78);       // vmcnt(40)
+        else if (n >= 32) __builtin_amdgcn_s_waitcnt(0x8f70);  // vmcnt(32)
+        else if (n >= 24) __builtin_amdgcn_s_waitcnt(0x4f78);  // vmcnt(24)
+        else if (n >= 16) __builtin_amdgcn_s_waitcnt(0x4f70);  // vmcnt(16)
+        else if (n >= 8) __builtin_amdgcn_s_waitcnt(0x0f78);   // vmcnt(8)
+        else __builtin_amdgcn_s_waitcnt(0x0f70);               // vmcnt(0)
+    };
 
+    uint32_t round = 0;
+    Tile cur = lookup(0);
+    // prefetched: the loaders are set up for `cur` and the loads of its first K step went out (into stage 0) before the
+    // epilogue of the previous tile, followed by exactly tile_stores stores
+    bool prefetched = false;
+    while (cur.valid) {
+        const uint32_t Me = cur.Me, Ne = cur.Ne, Ke = cur.Ke, n_span = cur.n_span, m0 = cur.m0, n0 = cur.n0;
+        const uint64_t off_d = cur.off_d;
+
+        if (!prefetched) {
+            if (!cur.fast) {
+                if constexpr (EPI == EPI_PLAIN) {
+                    scalar_tile<EL, A_KC, B_KC>(args.A + cur.off_a, args.B + cur.off_b, args.D + off_d, Me, Ne, Ke, m0, n0,
+                                                args.alpha, NT);
+                }
+                cur = lookup(++round);
+                continue;
+            }
+            setup_loaders(cur);
+        }
         f32x16 acc[FM][FN];
 #pragma unroll
         for (int i = 0; i < FM; ++i)
@@ -557,7 +673,6 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         // k slice and the MFMAs of that slice: once it is passed, the stage just read is free (the loads of step kt+2
         // are issued into it) and the other stage is complete (its first fragments are fetched), and both overlap
         // with the MFMAs still to be issued, so the matrix pipe has work while the barrier's latencies play out.
-        const uint32_t KT = (Ke + BK - 1) / BK;
         auto step = [&](int stage, uint32_t kt) {
             load_frags(stage, 1, 1);
             mma(0);
@@ -582,10 +697,15 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
             spread_mfma_vmem<0, FM * FN, 2 * (32 / NW)>();
         };
+        const uint32_t KT = (Ke + BK - 1) / BK;
+        Tile nxt{};
+        if (KT == 0) nxt = lookup(++round);
         if (KT > 0) {
-            issue(0, 0);
-            if (KT > 1) issue(1, BK);
-            __builtin_amdgcn_s_waitcnt(0x0070);
+            if (!prefetched) issue_quiet(0, 0);
+            if (KT > 1) issue_quiet(1, BK);
+            nxt = lookup(++round);  // in the shadow of the loads
+            // the first K step's loads have landed; the second step's, and the previous tile's stores, may still be out
+            wait_outstanding((prefetched ? tile_stores : 0u) + (KT > 1 ? kStepLoads : 0u));
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             load_frags(0, 0, 0);
@@ -603,87 +723,99 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             asm volatile("" ::: "memory");
         }
 
+        // ---- next tile: its first loads go out now, into stage 0, and fly while this tile's results are stored ----
+        prefetched = nxt.valid && nxt.fast && nxt.Ke > 0;
+        if (prefetched) {
+            setup_loaders(nxt);
+            issue_quiet(0, 0);
+        }
+
         // ---- epilogue ----
-        // Past the last barrier of the K loop nobody reads the LDS stages any more; each wavefront takes its own 16 KB
-        // slice of them as staging space (the barrier at the top of the next tile keeps the next loads away from it).
+        // Past the last barrier of the K loop nobody reads the LDS stages any more. Stage 1 is the staging space: each
+        // wavefront takes a private slice of it for half of its sub-tile at a time.
         // A lane holds row (lane & 31), columns q*8 + (lane >> 5)*4 + 0..3 of each 32x32 accumulator block.
-        static_assert((WM * WN * 2 == 16384 && NW == 8) || (WM * WN * 2 == 32768 && NW == 4),
-                      "staging slices are sized for eight 128x64 or four 128x128 wave tiles");
+        static_assert(FM % 2 == 0 && WM * WN == 2 * (32 / NW) * 1024, "two passes over the slices of one LDS stage");
         // the lane id is made opaque here so that the epilogue's per-lane address arithmetic is redone per tile instead
         // of being hoisted out of the tile loop, where it would occupy registers throughout the K loop
         uint32_t el = lane;
         asm volatile("" : "+v"(el));
-        constexpr uint32_t kPerArray = NW / 4;  // wavefronts that share one 32 KB stage array
-        const uint32_t arr = wave / kPerArray;
-        uint8_t* const img = (arr == 0 ? s_a0 : arr == 1 ? s_b0 : arr == 2 ? s_a1 : s_b1) +
-                             (wave % kPerArray) * (uint32_t)(WM * WN * 2);
+        const StagingSlice<NW> img{s_a1 + wave * 1024u, s_b1 + wave * 1024u};
         const float alpha = args.alpha;
-        const uint32_t row0 = m0 + wm * WM;  // first output row of this wavefront
-        if constexpr (EPI == EPI_PLAIN) {
+        constexpr int HM = WM / 2;  // rows per pass
+        constexpr int HF = FM / 2;  // accumulator row blocks per pass
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
+        for (int pass = 0; pass < 2; ++pass) {
+            const uint32_t row0 = m0 + wm * WM + pass * HM;  // first output row of this pass
+            const uint32_t rows_valid = row0 < Me ? (Me - row0 < (uint32_t)HM ? Me - row0 : (uint32_t)HM) : 0u;
+            if constexpr (EPI == EPI_PLAIN) {
+                const uint32_t col0 = n0 + wn * WN;
+                const uint32_t cols_valid = col0 < Ne ? Ne - col0 : 0u;
 #pragma unroll
-                for (int j = 0; j < FN; ++j)
+                for (int i = 0; i < HF; ++i)
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        uint2 w;
-                        w.x = EL::pack2(alpha * acc[i][j][q * 4 + 0], alpha * acc[i][j][q * 4 + 1]);
-                        w.y = EL::pack2(alpha * acc[i][j][q * 4 + 2], alpha * acc[i][j][q * 4 + 3]);
-                        stage_put<WN * 2>(img, i * 32 + (el & 31u), j * 32 + q * 8 + (el >> 5) * 4, w);
-                    }
-            stage_flush<WN * 2, WM>(img, args.D + off_d, Ne, row0, Me, n0 + wn * WN, Ne, el);
-        } else {
-            // first the rounded pre-activation (32 "up" columns | 32 "gate" columns per row), then the activation
-            constexpr int HB = WN * 2;  // bytes per staged row of h: 32 "up" columns | 32 "gate" columns
-            constexpr int YB = WN;      // bytes per staged row of the activation
-            uint16_t* He = args.D ? args.D + off_d : nullptr;
-            uint16_t* Ce = args.ACT + off_d / 2;
-            const uint32_t ncol0 = n0 + wn * (WN / 2);
+                    for (int j = 0; j < FN; ++j)
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
-#pragma unroll
-                for (int j = 0; j < FN / 2; ++j)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        float u[4], g[4], y[4];
-#pragma unroll
-                        for (int x = 0; x < 4; ++x) {
-                            u[x] = EL::round(alpha * acc[i][j][q * 4 + x]);
-                            g[x] = EL::round(alpha * acc[i][j + FN / 2][q * 4 + x]);
-                            y[x] = u[x] * g[x] * sigmoid_for<typename EL::act_t>(g[x]);
+                        for (int q = 0; q < 4; ++q) {
+                            const f32x16& c = acc[pass * HF + i][j];
+                            uint2 w;
+                            w.x = EL::pack2(alpha * c[q * 4 + 0], alpha * c[q * 4 + 1]);
+                            w.y = EL::pack2(alpha * c[q * 4 + 2], alpha * c[q * 4 + 3]);
+                            stage_put<WN * 2>(img, i * 32 + (el & 31u), j * 32 + q * 8 + (el >> 5) * 4, w);
                         }
-                        const uint32_t m = i * 32 + (el & 31u);
-                        const uint32_t c = j * 32 + q * 8 + (el >> 5) * 4;
-                        uint2 wy;
-                        wy.x = EL::pack2(y[0], y[1]);
-                        wy.y = EL::pack2(y[2], y[3]);
-                        // the packed activation waits in two accumulator registers until h has left the staging slice
-                        acc[i][j][q * 4 + 0] = __uint_as_float(wy.x);
-                        acc[i][j][q * 4 + 1] = __uint_as_float(wy.y);
-                        if (He) {
-                            uint2 wu, wg;
-                            wu.x = EL::pack2(u[0], u[1]);
-                            wu.y = EL::pack2(u[2], u[3]);
-                            wg.x = EL::pack2(g[0], g[1]);
-                            wg.y = EL::pack2(g[2], g[3]);
-                            stage_put<HB>(img, m, c, wu);
-                            stage_put<HB>(img, m, WN / 2 + c, wg);
+                stage_flush<WN * 2, HM>(img, args.D + off_d + (uint64_t)row0 * Ne + col0, Ne, rows_valid, cols_valid, el);
+            } else {
+                // first the rounded pre-activation (32 "up" columns | 32 "gate" columns per row), then the activation
+                constexpr int HB = WN * 2;  // bytes per staged row of h: 32 "up" columns | 32 "gate" columns
+                constexpr int YB = WN;      // bytes per staged row of the activation
+                const uint32_t col0 = n0 + wn * (WN / 2);
+                const uint32_t cols_valid = col0 < n_span ? n_span - col0 : 0u;
+                uint32_t ypack[HF][FN / 2][4][2];  // the packed activation waits here until h has left the staging slice
+#pragma unroll
+                for (int i = 0; i < HF; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN / 2; ++j)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            float u[4], g[4], y[4];
+#pragma unroll
+                            for (int x = 0; x < 4; ++x) {
+                                u[x] = EL::round(alpha * acc[pass * HF + i][j][q * 4 + x]);
+                                g[x] = EL::round(alpha * acc[pass * HF + i][j + FN / 2][q * 4 + x]);
+                                y[x] = u[x] * g[x] * sigmoid_for<typename EL::act_t>(g[x]);
+                            }
+                            ypack[i][j][q][0] = EL::pack2(y[0], y[1]);
+                            ypack[i][j][q][1] = EL::pack2(y[2], y[3]);
+                            if (args.D) {
+                                const uint32_t m = i * 32 + (el & 31u);
+                                const uint32_t c = j * 32 + q * 8 + (el >> 5) * 4;
+                                uint2 wu, wg;
+                                wu.x = EL::pack2(u[0], u[1]);
+                                wu.y = EL::pack2(u[2], u[3]);
+                                wg.x = EL::pack2(g[0], g[1]);
+                                wg.y = EL::pack2(g[2], g[3]);
+                                stage_put<HB>(img, m, c, wu);
+                                stage_put<HB>(img, m, WN / 2 + c, wg);
+                            }
                         }
-                    }
-            if (He) stage_flush_split<HB, WM, WN / 2>(img, He, Ne, row0, Me, ncol0, n_span, n_span, el);
+                if (args.D)
+                    stage_flush_split<HB, HM, WN / 2>(img, args.D + off_d + (uint64_t)row0 * Ne + col0, Ne, rows_valid,
+                                                      cols_valid, n_span, el);
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
+                for (int i = 0; i < HF; ++i)
 #pragma unroll
-                for (int j = 0; j < FN / 2; ++j)
+                    for (int j = 0; j < FN / 2; ++j)
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        uint2 wy;
-                        wy.x = __float_as_uint(acc[i][j][q * 4 + 0]);
-                        wy.y = __float_as_uint(acc[i][j][q * 4 + 1]);
-                        stage_put<YB>(img, i * 32 + (el & 31u), j * 32 + q * 8 + (el >> 5) * 4, wy);
-                    }
-            stage_flush<YB, WM>(img, Ce, n_span, row0, Me, ncol0, n_span, el);
+                        for (int q = 0; q < 4; ++q) {
+                            uint2 wy;
+                            wy.x = ypack[i][j][q][0];
+                            wy.y = ypack[i][j][q][1];
+                            stage_put<YB>(img, i * 32 + (el & 31u), j * 32 + q * 8 + (el >> 5) * 4, wy);
+                        }
+                stage_flush<YB, HM>(img, args.ACT + off_d / 2 + (uint64_t)row0 * n_span + col0, n_span, rows_valid,
+                                    cols_valid, el);
+            }
         }
+        cur = nxt;
     }
 }
 
