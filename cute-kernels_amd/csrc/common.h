@@ -78,6 +78,22 @@ struct alignas(16) Vec16 {
     T v[N];
 };
 
+// 16-byte store with the non-temporal hint, for outputs much larger than the caches that the kernel does not read back
+template <typename V>
+__device__ __forceinline__ void store_streaming16(V* p, const V& v) {
+    static_assert(sizeof(V) == 16, "16-byte vectors only");
+    typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+    __builtin_nontemporal_store(__builtin_bit_cast(u32x4, v), reinterpret_cast<u32x4*>(p));
+}
+
+// 16-byte load with the non-temporal hint, for inputs that are read exactly once
+template <typename V>
+__device__ __forceinline__ V load_streaming16(const V* p) {
+    static_assert(sizeof(V) == 16, "16-byte vectors only");
+    typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+    return __builtin_bit_cast(V, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)));
+}
+
 // sigmoid with the argument clamped to +-88.3762626647949 (the reference's fma/include/activations.h:9-22),
 // which keeps expf finite and changes no finite result.
 __device__ __forceinline__ float sigmoid_clamped(float x) {

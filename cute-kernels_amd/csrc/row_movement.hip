@@ -27,7 +27,7 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_kernel(const uint4* _
         for (int r = 0; r < kGatherRows; ++r) t[r] = src[r][v];
 #pragma unroll
         for (int r = 0; r < kGatherRows; ++r) {
-            if (i0 + r < R) out[(i0 + r) * vecs + v] = t[r];
+            if (i0 + r < R) store_streaming16(out + (i0 + r) * vecs + v, t[r]);
         }
     }
 }
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(kRowThreads) void dispatch_rows_kernel(const uint4*
         for (int u = 0; u < kDispatchTokens; ++u) {
             if (t0 + u < T) {
                 const int32_t* dst = inv + (t0 + u) * k;
-                for (int64_t j = 0; j < k; ++j) out[(int64_t)dst[j] * vecs + v] = row[u];
+                for (int64_t j = 0; j < k; ++j) store_streaming16(out + (int64_t)dst[j] * vecs + v, row[u]);
             }
         }
     }
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(kRowThreads) void combine_kernel(const Vec16<T>* __
             float g[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                r[u] = o[(int64_t)my_inv[j + u] * vecs + v];
+                r[u] = load_streaming16(o + (int64_t)my_inv[j + u] * vecs + v);
                 g[u] = my_gates ? Num<T>::up(my_gates[j + u]) : 1.0f;
             }
 #pragma unroll
@@ -126,13 +126,13 @@ __global__ __launch_bounds__(kRowThreads) void combine_bwd_kernel(const Vec16<T>
         auto one = [&](int64_t v, const Vec16<T>& d) {
             Vec16<T> w;
             if (d_gates) {
-                const Vec16<T> ov = o[row * vecs + v];
+                const Vec16<T> ov = load_streaming16(o + row * vecs + v);
 #pragma unroll
                 for (int c = 0; c < N; ++c) dot = fmaf(Num<T>::up(d.v[c]), Num<T>::up(ov.v[c]), dot);
             }
 #pragma unroll
             for (int c = 0; c < N; ++c) w.v[c] = Num<T>::down(g * Num<T>::up(d.v[c]));
-            d_o[row * vecs + v] = w;
+            store_streaming16(d_o + row * vecs + v, w);
         };
         if constexpr (CACHED) {
 #pragma unroll
