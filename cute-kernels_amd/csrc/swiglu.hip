@@ -28,6 +28,25 @@ struct Strides5 {
     int64_t gate, up, dy, dgate, dup;
 };
 
+// Position of a thread's current 16-byte vector in a rows x cvec grid of vectors, advanced by a fixed number of vectors
+// per iteration without a division inside the loop.
+struct VecCursor {
+    int64_t i, r, c;   // flat index, row, vector column
+    int64_t di, dr, dc;
+    __device__ __forceinline__ VecCursor(int64_t first, int64_t stride, int64_t cvec)
+        : i(first), r(first / cvec), c(first - (first / cvec) * cvec), di(stride), dr(stride / cvec),
+          dc(stride - (stride / cvec) * cvec) {}
+    __device__ __forceinline__ void advance(int64_t cvec) {
+        i += di;
+        r += dr;
+        c += dc;
+        if (c >= cvec) {
+            c -= cvec;
+            ++r;
+        }
+    }
+};
+
 template <typename T, bool VEC>
 __global__ __launch_bounds__(kSwThreads) void swiglu_fwd_kernel(const T* __restrict__ gate, const T* __restrict__ up,
                                                                 T* __restrict__ out, int64_t rows, int64_t cols,
@@ -35,17 +54,38 @@ __global__ __launch_bounds__(kSwThreads) void swiglu_fwd_kernel(const T* __restr
     constexpr int N = VEC ? Vec16<T>::N : 1;
     const int64_t cvec = cols / N;
     const int64_t total = rows * cvec;
-    for (int64_t i = (int64_t)blockIdx.x * kSwThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kSwThreads) {
-        const int64_t r = i / cvec;
-        const int64_t c = (i - r * cvec) * N;
-        if constexpr (VEC) {
-            const Vec16<T> g = *reinterpret_cast<const Vec16<T>*>(gate + r * s.gate + c);
-            const Vec16<T> u = *reinterpret_cast<const Vec16<T>*>(up + r * s.up + c);
-            Vec16<T> y;
+    if constexpr (VEC) {
+        typedef Vec16<T> V;
+        auto compute = [](const V& g, const V& u) {
+            V y;
 #pragma unroll
             for (int e = 0; e < N; ++e) y.v[e] = Num<T>::down(swiglu_f<T>(Num<T>::up(g.v[e]), Num<T>::up(u.v[e])));
-            *reinterpret_cast<Vec16<T>*>(out + r * s.out + c) = y;
-        } else {
+            return y;
+        };
+        VecCursor p((int64_t)blockIdx.x * kSwThreads + threadIdx.x, (int64_t)gridDim.x * kSwThreads, cvec);
+        // two vectors per iteration: four loads in flight per thread
+        while (p.i + p.di < total) {
+            const int64_t r0 = p.r, c0 = p.c * N;
+            p.advance(cvec);
+            const int64_t r1 = p.r, c1 = p.c * N;
+            p.advance(cvec);
+            const V g0 = *reinterpret_cast<const V*>(gate + r0 * s.gate + c0);
+            const V u0 = *reinterpret_cast<const V*>(up + r0 * s.up + c0);
+            const V g1 = *reinterpret_cast<const V*>(gate + r1 * s.gate + c1);
+            const V u1 = *reinterpret_cast<const V*>(up + r1 * s.up + c1);
+            *reinterpret_cast<V*>(out + r0 * s.out + c0) = compute(g0, u0);
+            *reinterpret_cast<V*>(out + r1 * s.out + c1) = compute(g1, u1);
+        }
+        if (p.i < total) {
+            const int64_t r0 = p.r, c0 = p.c * N;
+            const V g0 = *reinterpret_cast<const V*>(gate + r0 * s.gate + c0);
+            const V u0 = *reinterpret_cast<const V*>(up + r0 * s.up + c0);
+            *reinterpret_cast<V*>(out + r0 * s.out + c0) = compute(g0, u0);
+        }
+    } else {
+        for (int64_t i = (int64_t)blockIdx.x * kSwThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kSwThreads) {
+            const int64_t r = i / cvec;
+            const int64_t c = i - r * cvec;
             out[r * s.out + c] = Num<T>::down(swiglu_f<T>(Num<T>::up(gate[r * s.gate + c]), Num<T>::up(up[r * s.up + c])));
         }
     }
@@ -59,14 +99,9 @@ __global__ __launch_bounds__(kSwThreads) void swiglu_bwd_kernel(const T* __restr
     constexpr int N = VEC ? Vec16<T>::N : 1;
     const int64_t cvec = cols / N;
     const int64_t total = rows * cvec;
-    for (int64_t i = (int64_t)blockIdx.x * kSwThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kSwThreads) {
-        const int64_t r = i / cvec;
-        const int64_t c = (i - r * cvec) * N;
-        if constexpr (VEC) {
-            const Vec16<T> g = *reinterpret_cast<const Vec16<T>*>(gate + r * s.gate + c);
-            const Vec16<T> u = *reinterpret_cast<const Vec16<T>*>(up + r * s.up + c);
-            const Vec16<T> d = *reinterpret_cast<const Vec16<T>*>(dy + r * s.dy + c);
-            Vec16<T> og, ou;
+    if constexpr (VEC) {
+        typedef Vec16<T> V;
+        auto compute = [](const V& g, const V& u, const V& d, V& og, V& ou) {
 #pragma unroll
             for (int e = 0; e < N; ++e) {
                 float a, b;
@@ -74,9 +109,42 @@ __global__ __launch_bounds__(kSwThreads) void swiglu_bwd_kernel(const T* __restr
                 og.v[e] = Num<T>::down(a);
                 ou.v[e] = Num<T>::down(b);
             }
-            *reinterpret_cast<Vec16<T>*>(dgate + r * s.dgate + c) = og;
-            *reinterpret_cast<Vec16<T>*>(dup + r * s.dup + c) = ou;
-        } else {
+        };
+        VecCursor p((int64_t)blockIdx.x * kSwThreads + threadIdx.x, (int64_t)gridDim.x * kSwThreads, cvec);
+        // two vectors per iteration: six loads in flight per thread
+        while (p.i + p.di < total) {
+            const int64_t r0 = p.r, c0 = p.c * N;
+            p.advance(cvec);
+            const int64_t r1 = p.r, c1 = p.c * N;
+            p.advance(cvec);
+            const V g0 = *reinterpret_cast<const V*>(gate + r0 * s.gate + c0);
+            const V u0 = *reinterpret_cast<const V*>(up + r0 * s.up + c0);
+            const V d0 = *reinterpret_cast<const V*>(dy + r0 * s.dy + c0);
+            const V g1 = *reinterpret_cast<const V*>(gate + r1 * s.gate + c1);
+            const V u1 = *reinterpret_cast<const V*>(up + r1 * s.up + c1);
+            const V d1 = *reinterpret_cast<const V*>(dy + r1 * s.dy + c1);
+            V og, ou;
+            compute(g0, u0, d0, og, ou);
+            *reinterpret_cast<V*>(dgate + r0 * s.dgate + c0) = og;
+            *reinterpret_cast<V*>(dup + r0 * s.dup + c0) = ou;
+            compute(g1, u1, d1, og, ou);
+            *reinterpret_cast<V*>(dgate + r1 * s.dgate + c1) = og;
+            *reinterpret_cast<V*>(dup + r1 * s.dup + c1) = ou;
+        }
+        if (p.i < total) {
+            const int64_t r0 = p.r, c0 = p.c * N;
+            const V g0 = *reinterpret_cast<const V*>(gate + r0 * s.gate + c0);
+            const V u0 = *reinterpret_cast<const V*>(up + r0 * s.up + c0);
+            const V d0 = *reinterpret_cast<const V*>(dy + r0 * s.dy + c0);
+            V og, ou;
+            compute(g0, u0, d0, og, ou);
+            *reinterpret_cast<V*>(dgate + r0 * s.dgate + c0) = og;
+            *reinterpret_cast<V*>(dup + r0 * s.dup + c0) = ou;
+        }
+    } else {
+        for (int64_t i = (int64_t)blockIdx.x * kSwThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kSwThreads) {
+            const int64_t r = i / cvec;
+            const int64_t c = i - r * cvec;
             float a, b;
             swiglu_b<T>(Num<T>::up(gate[r * s.gate + c]), Num<T>::up(up[r * s.up + c]), Num<T>::up(dy[r * s.dy + c]), a, b);
             dgate[r * s.dgate + c] = Num<T>::down(a);
