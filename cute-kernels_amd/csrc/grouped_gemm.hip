@@ -271,13 +271,16 @@ __device__ __forceinline__ s16x8 read_tr_frag(const uint8_t* p) {
 // instruction writes 16 bytes per lane and whole 64- or 128-byte row segments.
 // Row m, 16-byte chunk c of the image sits at m*ROWB + ((c ^ key(m)) << 4), key(m) = (m / rows-per-256-B) mod chunks:
 // the 8-byte writes of 32 consecutive rows conflict at most two ways, the 16-byte reads not at all.
-// 16-byte buffer store with the non-temporal hint: the output tile is not read again by this kernel, and a workgroup's
-// 128 KB of results should not push operand panels out of the L2 (measured: +0.5 to +1.5 points of peak over plain
-// stores). A lane whose offset is not below the descriptor's size stores nothing, so every lane always executes the
+// 16-byte buffer store, with the non-temporal hint where possible: the output tile is not read again by this kernel,
+// and a workgroup's 128 KB of results should not push operand panels out of the L2 (measured: +0.5 to +1.5 points of
+// peak over plain stores). A lane whose offset is not below the descriptor's size stores nothing, so every lane always executes the
 // instruction: the number of stores a wavefront issues per tile is a compile-time constant, which the wait for the next
 // tile's first loads relies on.
-__device__ __forceinline__ void store_streaming(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint4 v) {
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc, (int)voff, 0, /*nt*/ 2);
+// NT only where a store instruction covers whole 128-byte lines: streamed 64-byte pieces are not merged in the L2 and
+// cost a read-modify-write each (measured on the SwiGLU epilogue: +35 % fetched and +28 % written bytes).
+template <bool NT>
+__device__ __forceinline__ void store_tile16(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint4 v) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc, (int)voff, 0, NT ? 2 : 0);
 }
 template <int ROWB>
 __device__ __forceinline__ uint32_t stage_off(uint32_t m, uint32_t chunk16) {
@@ -319,7 +322,7 @@ __device__ __forceinline__ void stage_flush(const Slice& img, uint16_t* origin, 
     for (uint32_t it = 0; it < ROWS / kRowsPerInst; ++it) {
         const uint32_t r = it * kRowsPerInst + lane / kChunks;
         const uint4 v = *reinterpret_cast<const uint4*>(img.at(stage_off<ROWB>(r, c16)));
-        store_streaming(rsrc, col_ok ? r * ldb + c16 * 16u : kOutOfRange, v);
+        store_tile16<(ROWB >= 128)>(rsrc, col_ok ? r * ldb + c16 * 16u : kOutOfRange, v);
     }
 }
 
@@ -340,7 +343,7 @@ __device__ __forceinline__ void stage_flush_split(const Slice& img, uint16_t* or
     for (uint32_t it = 0; it < ROWS / kRowsPerInst; ++it) {
         const uint32_t r = it * kRowsPerInst + lane / kChunks;
         const uint4 v = *reinterpret_cast<const uint4*>(img.at(stage_off<ROWB>(r, c16)));
-        store_streaming(rsrc, col_ok ? r * ldb + (window * second0 + in_window) * 2u : kOutOfRange, v);
+        store_tile16<(HALF * 2 >= 128)>(rsrc, col_ok ? r * ldb + (window * second0 + in_window) * 2u : kOutOfRange, v);
     }
 }
 
