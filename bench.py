@@ -204,13 +204,16 @@ def main():
         def want(name):
             return not only or any(w in name for w in only)
 
-        def mfma(name, flops, fn, n=iters):
+        def mfma(name, flops, fn, n=iters, nbytes=None):
             if not want(name):
                 return
             t = time_gpu(fn, n, blocker=blocker)
             tf = flops / (t[0] * 1e-3) / 1e12
             kernels[name] = {"ms": t[0], "ms_mean": t[1], "bound": "mfma", "achieved": tf, "peak": PEAK_BF16_TFLOPS,
                              "unit": "TFLOP/s", "frac": tf / PEAK_BF16_TFLOPS, "flop": flops}
+            if nbytes is not None:  # the second roof: operands read once, output written once
+                kernels[name]["hbm_bytes"] = nbytes
+                kernels[name]["hbm_frac"] = nbytes / (t[0] * 1e-3) / 1e9 / PEAK_HBM_GBS
 
         def hbm(name, nbytes, fn, n=20, warmup=3):
             if not want(name):
@@ -220,16 +223,24 @@ def main():
             kernels[name] = {"ms": t[0], "ms_mean": t[1], "bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS,
                              "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "bytes": nbytes}
 
+        w1_b, w2_b = E * 2 * I * H * s, E * H * I * s  # bytes of the two weight tensors
         mfma("up_projection_swiglu_fwd(NT)", 2.0 * R * 2 * I * H,
              lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), h.data_ptr(), a.data_ptr(),
-                                                      counts.data_ptr(), E, I, H, BF16, stream)))
+                                                      counts.data_ptr(), E, I, H, BF16, stream)),
+             nbytes=R * H * s + w1_b + R * 3 * I * s)
         # the unfused pair the fused kernel above replaces (same bits): plain up-projection, then swiglu_forward below
-        mfma("up_projection_plain_fwd(NT)", 2.0 * R * 2 * I * H, lambda i: gemm(xg, w1, h, counts, N_fc, K_fc, 0, 1))
-        mfma("down_projection_fwd(NT)", 2.0 * R * I * H, lambda i: gemm(a, w2, o, counts, N_pj, K_pj, 0, 1))
-        mfma("down_projection_dgrad(NN)", 2.0 * R * I * H, lambda i: gemm(d_o, w2, da, counts, K_pj, N_pj, 0, 0))
-        mfma("down_projection_wgrad(TN)", 2.0 * R * I * H, lambda i: gemm(d_o, a, dw2, N_pj, K_pj, counts, 1, 0))
-        mfma("up_projection_dgrad(NN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, w1, dxg, counts, K_fc, N_fc, 0, 0))
-        mfma("up_projection_wgrad(TN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, xg, dw1, N_fc, K_fc, counts, 1, 0))
+        mfma("up_projection_plain_fwd(NT)", 2.0 * R * 2 * I * H, lambda i: gemm(xg, w1, h, counts, N_fc, K_fc, 0, 1),
+             nbytes=R * H * s + w1_b + R * 2 * I * s)
+        mfma("down_projection_fwd(NT)", 2.0 * R * I * H, lambda i: gemm(a, w2, o, counts, N_pj, K_pj, 0, 1),
+             nbytes=R * I * s + w2_b + R * H * s)
+        mfma("down_projection_dgrad(NN)", 2.0 * R * I * H, lambda i: gemm(d_o, w2, da, counts, K_pj, N_pj, 0, 0),
+             nbytes=R * H * s + w2_b + R * I * s)
+        mfma("down_projection_wgrad(TN)", 2.0 * R * I * H, lambda i: gemm(d_o, a, dw2, N_pj, K_pj, counts, 1, 0),
+             nbytes=R * H * s + R * I * s + w2_b)
+        mfma("up_projection_dgrad(NN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, w1, dxg, counts, K_fc, N_fc, 0, 0),
+             nbytes=R * 2 * I * s + w1_b + R * H * s)
+        mfma("up_projection_wgrad(TN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, xg, dw1, N_fc, K_fc, counts, 1, 0),
+             nbytes=R * 2 * I * s + R * H * s + w1_b)
 
         # calibration for the profiler's FETCH_SIZE / WRITE_SIZE counters: a plain device copy of known size (ATen's
         # elementwise copy kernel): reads 1 GiB, writes 1 GiB
@@ -312,11 +323,19 @@ def main():
             y_c = O.moe_experts(x_c, w_c, sel_c, w1_c, w2_c)
             y_c.backward(dy_c)
 
+        def progress(msg):  # keeps a watchdog that looks for output quiet during the CPU leg
+            print(f"bench.py: cpu baseline: {msg}", file=sys.stderr, flush=True)
+
+        progress(f"{T_cpu} tokens on {cores} threads, warm-up step")
+        t0 = time.perf_counter()
         cpu_step()
+        first = time.perf_counter() - t0
         n, t0 = 0, time.perf_counter()
-        while n < 3 or (time.perf_counter() - t0 < 10 and n < 50):
+        # about 10 s of timed work, at least 2 steps (1 if a single step already takes more than 20 s)
+        while n < (1 if first > 20 else 2) or (time.perf_counter() - t0 < 10 and n < 50):
             cpu_step()
             n += 1
+            progress(f"step {n}, {time.perf_counter() - t0:.1f} s")
         cpu_s = (time.perf_counter() - t0) / n
         result["cpu_baseline"] = {
             "value": T_cpu / cpu_s,
@@ -326,6 +345,14 @@ def main():
             "sample": f"first {T_cpu} of {T} tokens of the same workload (same H, I, E, k, same routing), fp32 eager "
             f"torch on the host CPU, forward + backward, mean of {n} steps",
         }
+        # continuous_count beside it: the oracle's histogram of the same 16 Mi int32 ids on the host
+        ids_c = O.make_ids(16 << 20, 64, "uniform", seed=100)
+        O.continuous_count(ids_c, 64)
+        t0 = time.perf_counter()
+        for _ in range(3):
+            O.continuous_count(ids_c, 64)
+        cnt_s = (time.perf_counter() - t0) / 3
+        result["cpu_baseline"]["continuous_count_16Mi"] = {"ms": cnt_s * 1e3, "GB/s": ids_c.nbytes / cnt_s / 1e9, "cores": 1}
 
     print(json.dumps(result))
 
