@@ -49,6 +49,8 @@ def parse_args():
     p.add_argument("--no-layer", action="store_true", help="skip the whole-layer timing (for short profiler runs)")
     p.add_argument("--fuse-swiglu", type=int, default=-1, choices=[-1, 0, 1],
                    help="1 / 0: compute SwiGLU inside / after the up-projection kernel; -1: the module's default")
+    p.add_argument("--permute-experts", action="store_true",
+                   help="relabel the experts by a fixed random permutation (skewed routing no longer sorted by expert id)")
     p.add_argument("--only", default="", help="comma-separated substrings: measure only the kernels whose name matches")
     return p.parse_args()
 
@@ -105,6 +107,8 @@ def main():
     # ---- synthetic inputs (seeded on the CPU generator, then moved: identical bits for every consumer) ----
     g = torch.Generator().manual_seed(42)
     selected, weights = O.make_routing(T, E, k, c["kind"], seed=17, empty_tail=c["empty"])
+    if args.permute_experts:
+        selected = torch.randperm(E, generator=torch.Generator().manual_seed(5))[selected]
     x = torch.randn(T, H, generator=g).bfloat16().to(dev)
     dy = torch.randn(T, H, generator=g).bfloat16().to(dev)
     torch.manual_seed(42)

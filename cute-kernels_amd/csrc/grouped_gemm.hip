@@ -406,7 +406,8 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     __shared__ __attribute__((aligned(1024))) uint8_t s_b0[kTileBytes];
     __shared__ __attribute__((aligned(1024))) uint8_t s_a1[kTileBytes];
     __shared__ __attribute__((aligned(1024))) uint8_t s_b1[kTileBytes];
-    __shared__ uint32_t s_tile_start[FMA_MAX_GROUPS + 1];
+    __shared__ uint32_t s_tile_start[FMA_MAX_GROUPS + 1];  // first tile of the group at position p of the tile sequence
+    __shared__ uint16_t s_order[FMA_MAX_GROUPS];           // which group that is
     __shared__ uint64_t s_off_a[FMA_MAX_GROUPS + 1];
     __shared__ uint64_t s_off_b[FMA_MAX_GROUPS + 1];
     __shared__ uint64_t s_off_d[FMA_MAX_GROUPS + 1];
@@ -432,19 +433,51 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         return ((m + BM - 1) / BM) * tn;
     };
 
-    // ---- group table: exclusive prefixes of tiles and of packed element counts, built by wavefront 0 ----
+    // ---- order of the groups in the tile sequence: by K steps per tile, longest first ----
+    // With the reduction length varying between groups (weight gradients: it is the number of rows routed to the expert)
+    // tiles differ in cost; handing them out expensive-first, in alternating directions (below), keeps the workgroups'
+    // totals close. Ranks come from an all-pairs comparison over keys parked in the (still unused) LDS stages; groups of
+    // equal cost keep their order, and when every group costs the same the order is the identity.
+    {
+        uint32_t* const key = reinterpret_cast<uint32_t*>(s_a0);  // K steps per tile of group e; 0 if it has no tiles
+        const uint32_t key0 = tiles_of(group_m(0), group_n(0)) ? (group_k(0) + BK - 1) / BK : 0u;
+        bool differs = false;
+        for (uint32_t e = tid; e < E; e += NT) {
+            const uint32_t k = tiles_of(group_m(e), group_n(e)) ? (group_k(e) + BK - 1) / BK : 0u;
+            key[e] = k;
+            differs = differs || k != key0;
+        }
+        if (__syncthreads_or(differs)) {
+            for (uint32_t e = tid; e < E; e += NT) {
+                const uint32_t mine = key[e];
+                uint32_t rank = 0;
+                for (uint32_t j = 0; j < E; ++j) {
+                    const uint32_t other = key[j];
+                    rank += (other > mine || (other == mine && j < e)) ? 1u : 0u;
+                }
+                s_order[rank] = (uint16_t)e;
+            }
+        } else {
+            for (uint32_t e = tid; e < E; e += NT) s_order[e] = (uint16_t)e;
+        }
+        __syncthreads();
+    }
+
+    // ---- group table, built by wavefront 0: exclusive prefix of tiles over the order above, exclusive prefixes of the
+    // packed element counts over the groups as they lie in memory ----
     if (wave == 0) {
         uint32_t carry_t = 0;
         uint64_t carry_a = 0, carry_b = 0, carry_d = 0;
         for (uint32_t base = 0; base < E; base += 64) {
             const uint32_t e = base + lane;
-            uint32_t m = 0, n = 0, k = 0;
+            uint32_t m = 0, n = 0, k = 0, t = 0;
             if (e < E) {
                 m = group_m(e);
                 n = group_n(e);
                 k = group_k(e);
+                const uint32_t at = s_order[e];  // the group at position e of the tile sequence
+                t = tiles_of(group_m(at), group_n(at));
             }
-            const uint32_t t = tiles_of(m, n);
             const uint64_t sa = (uint64_t)m * k, sb = (uint64_t)k * n, sd = (uint64_t)m * n;
             const uint32_t it = wave_inclusive_scan<uint32_t>(t);
             const uint64_t ia = wave_inclusive_scan<uint64_t>(sa);
@@ -522,7 +555,8 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             if (s_tile_start[mid + 1] <= v) lo = mid + 1;
             else hi = mid;
         }
-        const uint32_t e = uniform(lo);
+        const uint32_t pos = uniform(lo);
+        const uint32_t e = uniform((uint32_t)s_order[pos]);
         t.valid = true;
         t.Me = group_m(e);
         t.Ne = group_n(e);
@@ -530,7 +564,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         t.n_span = EPI == EPI_SWIGLU ? t.Ne / 2 : t.Ne;  // columns the tile grid runs over
         const uint32_t tiles_m = (t.Me + BM - 1) / BM;
         const uint32_t tiles_n = (t.n_span + TN - 1) / TN;
-        const uint32_t local = v - uniform(s_tile_start[e]);
+        const uint32_t local = v - uniform(s_tile_start[pos]);
         const uint32_t band = kGroupM * tiles_n;
         const uint32_t first_m = (local / band) * kGroupM;
         const uint32_t band_m = tiles_m - first_m < (uint32_t)kGroupM ? tiles_m - first_m : (uint32_t)kGroupM;

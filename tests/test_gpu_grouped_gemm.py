@@ -173,3 +173,18 @@ def test_fp16_random_operands_and_fused_swiglu():
     grouped_gemm_swiglu_cuda(x, w, M, h, act)
     assert torch.equal(h, h_ref)
     assert torch.equal(act, swiglu_packed(h_ref))
+
+
+def test_weight_gradient_layout_with_shuffled_ragged_reduction_lengths():
+    # TN with a different reduction length per group, in no particular order, zeros included: the kernel orders the
+    # groups by cost internally, the results must not depend on that
+    g = torch.Generator().manual_seed(3)
+    K_list = [0, 8, 4000, 64, 0, 1032, 72, 8, 2048, 136, 520, 8, 264, 1000, 0, 200] * 3
+    E, M, N = len(K_list), 264, 520
+    A, B = _integer_operands([M] * E, [N] * E, K_list, True, False, seed=13)
+    expect = O.grouped_gemm(A, B, [M] * E, [N] * E, K_list, True, False)
+    got = grouped_gemm(
+        A=A.to(DEV), B=B.to(DEV), C=None, M_array=_u32([M] * E), N_array=_u32([N] * E), K_array=_u32(K_list),
+        output_shape=(E * M * N,), is_A_transposed=True, is_B_transposed=False,
+    )
+    assert float((got.cpu().float() - expect.float()).abs().max()) == 0
