@@ -4,8 +4,10 @@
 // Shape of the kernel
 //  * Persistent: the grid is one workgroup per compute unit. Each workgroup builds the group table (tile
 //    prefix and packed element offsets of every group) in LDS from the device-side M/N/K arrays, then walks
-//    256x256 output tiles. Tile ids are handed out so that the 32 workgroups of one XCD (workgroup id mod 8)
-//    always hold a compact 8x4 block of tiles of the same group: they share A and B panels in that XCD's L2.
+//    256x256 output tiles. Groups enter the tile sequence longest reduction first and rounds of tiles are dealt in
+//    alternating directions (balance under ragged reduction lengths); within a round the 32 workgroups of one XCD
+//    (workgroup id mod 8) hold a compact 8x4 block of tiles of the same group: they share A and B panels in that
+//    XCD's L2.
 //  * K is consumed in steps of 64 through two LDS stages of 2 x 32 KB. Every operand tile goes global -> LDS directly
 //    (buffer_load_dwordx4 ... lds, 1 KB per wavefront instruction, no staging registers; the buffer descriptor's range
 //    check zero-fills rows and reduction steps past the edge of a group), in one of two layouts:
@@ -21,7 +23,8 @@
 //  * Fragments are double buffered in registers and the workgroup barrier of a K step sits before the MFMAs of its
 //    last k slice, so the LDS and barrier latencies are covered by matrix work.
 //  * The MFMA is issued with B as the first operand, so a lane ends up holding four consecutive output
-//    columns of one output row and stores them as one 8-byte word.
+//    columns of one output row. The epilogue transposes the wavefront's sub-tile through LDS (stage 1) and stores
+//    whole 128-byte row segments; the next tile's first loads are already on their way into stage 0 by then.
 #include "common.h"
 
 namespace fmahip {
@@ -265,19 +268,20 @@ __device__ __forceinline__ s16x8 read_tr_frag(const uint8_t* p) {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-// ---- epilogue staging: a wavefront transposes its accumulator sub-tile through a private 16 KB slice of LDS ----
+// ---- epilogue staging: a wavefront transposes its accumulator sub-tile, half at a time, through 8 KB of LDS ----
 // The MFMA leaves a lane with 4 consecutive columns of one row per 32x32 block, so storing straight from registers
 // writes 8-byte pieces of 32 different rows per instruction. Staged through LDS as rows of ROWB bytes, every store
 // instruction writes 16 bytes per lane and whole 64- or 128-byte row segments.
 // Row m, 16-byte chunk c of the image sits at m*ROWB + ((c ^ key(m)) << 4), key(m) = (m / rows-per-256-B) mod chunks:
 // the 8-byte writes of 32 consecutive rows conflict at most two ways, the 16-byte reads not at all.
-// 16-byte buffer store, with the non-temporal hint where possible: the output tile is not read again by this kernel,
-// and a workgroup's 128 KB of results should not push operand panels out of the L2 (measured: +0.5 to +1.5 points of
-// peak over plain stores). A lane whose offset is not below the descriptor's size stores nothing, so every lane always executes the
-// instruction: the number of stores a wavefront issues per tile is a compile-time constant, which the wait for the next
-// tile's first loads relies on.
-// NT only where a store instruction covers whole 128-byte lines: streamed 64-byte pieces are not merged in the L2 and
-// cost a read-modify-write each (measured on the SwiGLU epilogue: +35 % fetched and +28 % written bytes).
+
+// 16-byte buffer store of a staged piece. A lane whose offset is not below the descriptor's size stores nothing, so
+// every lane always executes the instruction: the number of stores a wavefront issues per tile is a compile-time
+// constant, which the wait for the next tile's first loads relies on.
+// NT = the non-temporal hint: the output tile is not read again by this kernel, and a workgroup's 128 KB of results
+// should not push operand panels out of the L2 (measured: +0.5 to +1.5 points of peak over plain stores). Only where a
+// store instruction covers whole 128-byte lines: streamed 64-byte pieces are not merged in the L2 and cost a
+// read-modify-write each (measured on the SwiGLU epilogue: +35 % fetched and +28 % written bytes).
 template <bool NT>
 __device__ __forceinline__ void store_tile16(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint4 v) {
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc, (int)voff, 0, NT ? 2 : 0);
