@@ -781,7 +781,14 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         uint32_t el = lane;
         asm volatile("" : "+v"(el));
         const StagingSlice<NW> img{s_a1 + wave * 1024u, s_b1 + wave * 1024u};
-        const float alpha = args.alpha;
+        // alpha is applied up front, and only when it is not 1 (the usual case, and always so for the SwiGLU epilogue)
+        if (EPI == EPI_PLAIN && args.alpha != 1.0f) {
+            const float alpha = args.alpha;
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j) acc[i][j] *= alpha;
+        }
         constexpr int HM = WM / 2;  // rows per pass
         constexpr int HF = FM / 2;  // accumulator row blocks per pass
 #pragma unroll
@@ -799,8 +806,8 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                         for (int q = 0; q < 4; ++q) {
                             const f32x16& c = acc[pass * HF + i][j];
                             uint2 w;
-                            w.x = EL::pack2(alpha * c[q * 4 + 0], alpha * c[q * 4 + 1]);
-                            w.y = EL::pack2(alpha * c[q * 4 + 2], alpha * c[q * 4 + 3]);
+                            w.x = EL::pack2(c[q * 4 + 0], c[q * 4 + 1]);
+                            w.y = EL::pack2(c[q * 4 + 2], c[q * 4 + 3]);
                             stage_put<WN * 2>(img, i * 32 + (el & 31u), j * 32 + q * 8 + (el >> 5) * 4, w);
                         }
                 stage_flush<WN * 2, HM>(img, args.D + off_d + (uint64_t)row0 * Ne + col0, Ne, rows_valid, cols_valid, el);
@@ -820,8 +827,8 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                             float u[4], g[4], y[4];
 #pragma unroll
                             for (int x = 0; x < 4; ++x) {
-                                u[x] = EL::round(alpha * acc[pass * HF + i][j][q * 4 + x]);
-                                g[x] = EL::round(alpha * acc[pass * HF + i][j + FN / 2][q * 4 + x]);
+                                u[x] = EL::round(acc[pass * HF + i][j][q * 4 + x]);
+                                g[x] = EL::round(acc[pass * HF + i][j + FN / 2][q * 4 + x]);
                                 y[x] = u[x] * g[x] * sigmoid_for<typename EL::act_t>(g[x]);
                             }
                             ypack[i][j][q][0] = EL::pack2(y[0], y[1]);

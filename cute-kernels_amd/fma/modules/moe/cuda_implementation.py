@@ -53,7 +53,7 @@ def moe_build_index_cuda(
 def gather_rows_cuda(x: torch.Tensor, idx: torch.Tensor, divisor: int, output: torch.Tensor) -> None:
     _lib.require_gpu(x, idx, output)
     assert x.dim() == 2 and output.dim() == 2 and x.size(1) == output.size(1) and x.dtype == output.dtype
-    assert idx.dtype == torch.int32 and idx.numel() == output.size(0)
+    assert idx.dtype == torch.int32 and idx.numel() == output.size(0)  # x may have more rows than are gathered
     assert x.is_contiguous() and output.is_contiguous() and idx.is_contiguous()
     with torch.cuda.device(x.device):
         rc = _lib.load().fma_gather_rows(
@@ -67,7 +67,8 @@ def gather_rows_cuda(x: torch.Tensor, idx: torch.Tensor, divisor: int, output: t
 def dispatch_rows_cuda(x: torch.Tensor, inv: torch.Tensor, top_k: int, output: torch.Tensor) -> None:
     _lib.require_gpu(x, inv, output)
     T, H = x.shape
-    assert output.shape == (T * top_k, H) and x.dtype == output.dtype
+    # at least one destination row per (token, choice); more when the destination is a padded layout
+    assert output.dim() == 2 and output.size(0) >= T * top_k and output.size(1) == H and x.dtype == output.dtype
     assert inv.dtype == torch.int32 and inv.numel() == T * top_k
     assert x.is_contiguous() and output.is_contiguous() and inv.is_contiguous()
     with torch.cuda.device(x.device):
@@ -333,6 +334,151 @@ class _UpProjectionSwiglu(torch.autograd.Function):
                 output_shape=weight.size(), is_A_transposed=True, is_B_transposed=False,
             )
         return x_grad, weight_grad, None, None, None
+
+
+# ---- the reference's padded grouping interface -------------------------------------------------------
+# The MoE module above does not pad (the grouped GEMM masks ragged group edges). These keep the call signatures of
+# fma/modules/moe/cuda_implementation/__init__.py:83-280 for code that calls them directly; the row movement itself is
+# the dispatch / gather / combine kernels with a destination index that includes the padding offsets.
+
+
+@torch.no_grad()
+def _get_expert_padding_offset(
+    expert_frequency: torch.Tensor, E: int, pad_to_multiple_of: int
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """pad[e] = p - (M_e mod p), in [1, p] (an expert whose count is a multiple of p still gets p rows of padding);
+    returns (M_e + pad[e] as uint32[E], [0, cumsum(pad)] as int64[E + 1])
+    (fma/modules/moe/cuda_implementation/__init__.py:83-104, padded_expert_frequency_kernel.py:14-24)."""
+    assert expert_frequency.numel() == E
+    frequency = expert_frequency.to(torch.int64)
+    padding = pad_to_multiple_of - frequency % pad_to_multiple_of
+    padded_expert_frequency = (frequency + padding).to(torch.uint32)
+    expert_padding_offset = torch.cat([padding.new_zeros(1), padding.cumsum(-1)])
+    return padded_expert_frequency, expert_padding_offset
+
+
+def _padded_row_of_slot(
+    expert_padding_offset: torch.Tensor | None, sorted_idxs: torch.Tensor, scattered_idxs: torch.Tensor
+) -> torch.Tensor:
+    """int32[R]: the (padded) grouped row that holds slot s. sorted_idxs[i] is the expert of grouped row i,
+    scattered_idxs[i] the slot it comes from (group_kernel.py:26-74: row i of expert e lands at i + offset[e])."""
+    R = scattered_idxs.numel()
+    rows = torch.arange(R, device=scattered_idxs.device, dtype=torch.int64)
+    if expert_padding_offset is not None:
+        rows = rows + expert_padding_offset.to(torch.int64)[sorted_idxs.long()]
+    row_of_slot = torch.empty(R, device=scattered_idxs.device, dtype=torch.int32)
+    row_of_slot[scattered_idxs.long()] = rows.to(torch.int32)
+    return row_of_slot
+
+
+class _GroupWithPadding(torch.autograd.Function):
+    @staticmethod
+    @ensure_contiguous
+    def forward(
+        ctx,
+        x: torch.Tensor,
+        expert_frequency: torch.Tensor,
+        sorted_idxs: torch.Tensor,
+        scattered_idxs: torch.Tensor,
+        top_k: int,
+        pad_to_multiple_of: int,
+    ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
+        assert x.dim() == 2
+        T, H = x.size()
+        E = expert_frequency.size(0)
+        assert H % 8 == 0
+
+        if pad_to_multiple_of == 1:
+            output = torch.empty(T * top_k, H, device=x.device, dtype=x.dtype)
+            padded_expert_frequency = expert_frequency
+            expert_padding_offset = None
+        else:
+            # the data-independent upper bound on the padded row count, zero-filled (the reference's shape)
+            rows = (-(-(T * top_k) // pad_to_multiple_of) + E) * pad_to_multiple_of
+            output = torch.zeros(rows, H, device=x.device, dtype=x.dtype)
+            padded_expert_frequency, expert_padding_offset = _get_expert_padding_offset(
+                expert_frequency=expert_frequency, E=E, pad_to_multiple_of=pad_to_multiple_of
+            )
+
+        row_of_slot = _padded_row_of_slot(expert_padding_offset, sorted_idxs, scattered_idxs)
+        dispatch_rows_cuda(x, row_of_slot, top_k, output)
+
+        ctx.save_for_backward(row_of_slot)
+        ctx.T = T
+        ctx.K = top_k
+        return output, padded_expert_frequency, expert_padding_offset
+
+    @staticmethod
+    @ensure_contiguous
+    def backward(ctx, output_grad: torch.Tensor, _: torch.Tensor, __: torch.Tensor) -> tuple[torch.Tensor | None]:
+        (row_of_slot,) = ctx.saved_tensors
+        # fp32 accumulation over the top_k rows of a token in a fixed order (the reference: fp32 atomics, then a cast)
+        x_grad = torch.empty(ctx.T, output_grad.size(-1), device=output_grad.device, dtype=output_grad.dtype)
+        combine_cuda(output_grad, row_of_slot, None, ctx.K, x_grad)
+        return x_grad, *[None] * 5
+
+
+class _UngroupWithPadding(torch.autograd.Function):
+    @staticmethod
+    @ensure_contiguous
+    def forward(
+        ctx,
+        x: torch.Tensor,
+        expert_padding_offset: torch.Tensor | None,
+        sorted_idxs: torch.Tensor,
+        scattered_idxs: torch.Tensor,
+        top_k: int,
+        num_tokens: int,
+        pad_to_multiple_of: int,
+    ) -> torch.Tensor:
+        assert x.dim() == 2
+        H = x.size(-1)
+        assert H % 8 == 0
+        output = torch.empty(num_tokens, top_k, H, device=x.device, dtype=x.dtype)
+
+        row_of_slot = _padded_row_of_slot(expert_padding_offset, sorted_idxs, scattered_idxs)
+        gather_rows_cuda(x, row_of_slot, 1, output.view(num_tokens * top_k, H))
+
+        ctx.save_for_backward(row_of_slot)
+        ctx.x_shape = x.size()
+        ctx.pad_to_multiple_of = pad_to_multiple_of
+        return output
+
+    @staticmethod
+    @ensure_contiguous
+    def backward(ctx, output_grad: torch.Tensor) -> tuple[torch.Tensor | None]:
+        (row_of_slot,) = ctx.saved_tensors
+        T, K, H = output_grad.size()
+        x_grad = (torch.empty if ctx.pad_to_multiple_of == 1 else torch.zeros)(
+            *ctx.x_shape, device=output_grad.device, dtype=output_grad.dtype
+        )
+        dispatch_rows_cuda(output_grad.view(T * K, H), row_of_slot, 1, x_grad)
+        return x_grad, *[None] * 6
+
+
+def group_with_padding(
+    x: torch.Tensor,
+    expert_frequency: torch.Tensor,
+    sorted_idxs: torch.Tensor,
+    scattered_idxs: torch.Tensor,
+    top_k: int,
+    pad_to_multiple_of: int = 1,
+) -> torch.Tensor:
+    return _GroupWithPadding.apply(x, expert_frequency, sorted_idxs, scattered_idxs, top_k, pad_to_multiple_of)
+
+
+def ungroup_with_padding(
+    x: torch.Tensor,
+    expert_padding_offset: torch.Tensor,
+    sorted_idxs: torch.Tensor,
+    scattered_idxs: torch.Tensor,
+    top_k: int,
+    num_tokens: int,
+    pad_to_multiple_of: int,
+) -> torch.Tensor:
+    return _UngroupWithPadding.apply(
+        x, expert_padding_offset, sorted_idxs, scattered_idxs, top_k, num_tokens, pad_to_multiple_of
+    )
 
 
 def gather_rows(x: torch.Tensor, perm: torch.Tensor, inv: torch.Tensor, top_k: int) -> torch.Tensor:
