@@ -946,10 +946,11 @@ int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, co
     FMA_REQUIRE(E >= 0, FMA_ERR_BAD_SIZE, "grouped_gemm_swiglu: negative group count %lld", (long long)E);
     FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "grouped_gemm_swiglu: E=%lld exceeds the limit %d",
                 (long long)E, FMA_MAX_GROUPS);
-    FMA_REQUIRE(I >= 8 && I % 8 == 0 && I <= 0x3fffffffll, FMA_ERR_BAD_SIZE,
-                "grouped_gemm_swiglu: intermediate size %lld must be a positive multiple of 8", (long long)I);
-    FMA_REQUIRE(K >= 8 && K % 8 == 0 && K <= 0x7fffffffll, FMA_ERR_BAD_SIZE,
-                "grouped_gemm_swiglu: K=%lld must be a positive multiple of 8", (long long)K);
+    // the upper bounds are those of the kernel's 32-bit tile offsets; this entry point has no scalar path beyond them
+    FMA_REQUIRE(I >= 8 && I % 8 == 0 && 2 * I < (1ll << 23), FMA_ERR_BAD_SIZE,
+                "grouped_gemm_swiglu: intermediate size %lld must be a positive multiple of 8 below 2^22", (long long)I);
+    FMA_REQUIRE(K >= 8 && K % 8 == 0 && K < (1ll << 21), FMA_ERR_BAD_SIZE,
+                "grouped_gemm_swiglu: K=%lld must be a positive multiple of 8 below 2^21", (long long)K);
     if (E == 0) return FMA_OK;
     FMA_REQUIRE(x && W && act && M_arr, FMA_ERR_NULL_POINTER, "grouped_gemm_swiglu: NULL pointer");
     FMA_REQUIRE(aligned16(x) && aligned16(W) && aligned16(act) && aligned16(h), FMA_ERR_MISALIGNED,

@@ -161,7 +161,7 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
  *   h_e   = x_e[M_e, K] * W_e[2I, K]^T            (rounded to dtype; written to h if h != NULL)
  *   act_e = h_e[:, :I] * silu(h_e[:, I:])         (first half "up", second half "gate")
  * computed from the ROUNDED h so the result equals fma_grouped_gemm followed by fma_swiglu_forward bit for
- * bit. W: [E, 2I, K] row-major; h: [R, 2I]; act: [R, I]; I % 8 == 0, K % 8 == 0.
+ * bit. W: [E, 2I, K] row-major; h: [R, 2I]; act: [R, I]; I % 8 == 0, K % 8 == 0, I < 2^22, K < 2^21.
  * Fuses _GroupedGemmExperts.forward (fma/modules/moe/cuda_implementation/__init__.py:28-38) with
  * swiglu_packed (fma/ops/swiglu/__init__.py:133-164, up/gate = chunk(2, -1) at :153). */
 int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, const uint32_t* M_arr,

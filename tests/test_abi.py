@@ -91,6 +91,8 @@ def test_swiglu_and_gemm_validation(lib):
     assert lib.fma_grouped_gemm(p, p, p, p, p, p, 0, 0, 1, 1.0, 2, None) == 0
     assert lib.fma_grouped_gemm_swiglu(p, p, p, p, p, 4, 12, 64, 2, None) == -3  # I % 8 != 0
     assert lib.fma_grouped_gemm_swiglu(p, p, p, p, p, 4, 16, 60, 2, None) == -3  # K % 8 != 0
+    assert lib.fma_grouped_gemm_swiglu(p, p, p, p, p, 4, 1 << 22, 64, 2, None) == -3  # beyond the 32-bit tile offsets
+    assert lib.fma_grouped_gemm_swiglu(p, p, p, p, p, 4, 16, 1 << 21, 2, None) == -3
 
 
 def test_check_raises_runtime_error(lib):
