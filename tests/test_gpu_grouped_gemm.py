@@ -188,3 +188,20 @@ def test_weight_gradient_layout_with_shuffled_ragged_reduction_lengths():
         output_shape=(E * M * N,), is_A_transposed=True, is_B_transposed=False,
     )
     assert float((got.cpu().float() - expect.float()).abs().max()) == 0
+
+
+@pytest.mark.parametrize("tA,tB", [(False, True), (True, False)])
+def test_maximum_group_count(tA, tB):
+    # 1024 groups (the limit), sizes that vary per group in every dimension, many empty
+    g = torch.Generator().manual_seed(21)
+    E = 1024
+    M_list = (torch.randint(0, 5, (E,), generator=g) * 8).tolist()
+    N_list = (torch.randint(1, 4, (E,), generator=g) * 8).tolist()
+    K_list = (torch.randint(0, 20, (E,), generator=g) * 8).tolist()
+    A, B = _integer_operands(M_list, N_list, K_list, tA, tB, seed=22)
+    expect = O.grouped_gemm(A, B, M_list, N_list, K_list, tA, tB)
+    got = grouped_gemm(
+        A=A.to(DEV), B=B.to(DEV), C=None, M_array=_u32(M_list), N_array=_u32(N_list), K_array=_u32(K_list),
+        output_shape=(sum(m * n for m, n in zip(M_list, N_list)),), is_A_transposed=tA, is_B_transposed=tB,
+    )
+    assert float((got.cpu().float() - expect.float()).abs().max()) == 0
