@@ -205,3 +205,66 @@ def test_maximum_group_count(tA, tB):
         output_shape=(sum(m * n for m, n in zip(M_list, N_list)),), is_A_transposed=tA, is_B_transposed=tB,
     )
     assert float((got.cpu().float() - expect.float()).abs().max()) == 0
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_problem_shapes(seed):
+    # seeded random problems: every layout, group counts 1..40, ragged / empty / one-row groups, reduction lengths from 0
+    # to 17 K steps (even and odd step counts, partial last step), sizes off the 8-element grid now and then (scalar
+    # path). Integer operands, so the fp32 sums are exact in any order and the bf16 result must match bit for bit.
+    g = torch.Generator().manual_seed(1000 + seed)
+
+    def draw(hi, grid):
+        v = int(torch.randint(0, hi + 1, (1,), generator=g))
+        return v if int(torch.randint(0, 8, (1,), generator=g)) == 0 and not grid else (v // 8) * 8
+
+    for _ in range(6):
+        tA, tB = bool(torch.randint(0, 2, (1,), generator=g)), bool(torch.randint(0, 2, (1,), generator=g))
+        E = int(torch.randint(1, 41, (1,), generator=g))
+        same_nk = bool(torch.randint(0, 2, (1,), generator=g))
+        N0, K0 = max(8, draw(600, True)), draw(1100, True)
+        M_list = [draw(700, False) for _ in range(E)]
+        N_list = [N0 if same_nk else max(1, draw(600, False)) for _ in range(E)]
+        K_list = [K0 if same_nk else draw(1100, False) for _ in range(E)]
+        As, Bs, Ds = [], [], []
+        for M, N, K in zip(M_list, N_list, K_list):
+            a = torch.randint(-4, 5, (K, M) if tA else (M, K), generator=g).to(torch.bfloat16).to(DEV)
+            b = torch.randint(-4, 5, (N, K) if tB else (K, N), generator=g).to(torch.bfloat16).to(DEV)
+            As.append(a.reshape(-1))
+            Bs.append(b.reshape(-1))
+            Ds.append(((a.T if tA else a).float() @ (b.T if tB else b).float()).to(torch.bfloat16).reshape(-1))
+        total = sum(m * n for m, n in zip(M_list, N_list))
+        if total == 0:
+            continue
+        got = grouped_gemm(
+            A=torch.cat(As), B=torch.cat(Bs), C=None, M_array=_u32(M_list), N_array=_u32(N_list), K_array=_u32(K_list),
+            output_shape=(total,), is_A_transposed=tA, is_B_transposed=tB,
+        )
+        diff = float((got.float() - torch.cat(Ds).float()).abs().max())
+        assert diff == 0, f"tA={tA} tB={tB} M={M_list} N={N_list} K={K_list}: max |diff| = {diff}"
+
+
+@pytest.mark.parametrize("tA,tB", [(False, True), (False, False), (True, False)])
+def test_random_problems_with_several_tiles_per_workgroup(tA, tB):
+    # more tiles than workgroups, so every workgroup walks through tiles of different groups with different reduction
+    # lengths (and reaches the next tile's first loads before it has stored the previous one)
+    g = torch.Generator().manual_seed(77 + 2 * tA + tB)
+    E = 24
+    M_list = [int(v) * 8 for v in torch.randint(0, 1000, (E,), generator=g)]
+    N_list = [int(v) * 8 for v in torch.randint(20, 130, (E,), generator=g)]
+    K_list = [int(v) * 8 for v in torch.randint(0, 160, (E,), generator=g)]
+    M_list[3], K_list[5] = 0, 0
+    As, Bs, Ds = [], [], []
+    for M, N, K in zip(M_list, N_list, K_list):
+        a = torch.randint(-4, 5, (K, M) if tA else (M, K), generator=g).to(torch.bfloat16).to(DEV)
+        b = torch.randint(-4, 5, (N, K) if tB else (K, N), generator=g).to(torch.bfloat16).to(DEV)
+        As.append(a.reshape(-1))
+        Bs.append(b.reshape(-1))
+        Ds.append(((a.T if tA else a).float() @ (b.T if tB else b).float()).to(torch.bfloat16).reshape(-1))
+    tiles = sum(-(-m // 256) * -(-n // 256) for m, n in zip(M_list, N_list))
+    assert tiles > 3 * 256
+    got = grouped_gemm(
+        A=torch.cat(As), B=torch.cat(Bs), C=None, M_array=_u32(M_list), N_array=_u32(N_list), K_array=_u32(K_list),
+        output_shape=(sum(m * n for m, n in zip(M_list, N_list)),), is_A_transposed=tA, is_B_transposed=tB,
+    )
+    assert float((got.float() - torch.cat(Ds).float()).abs().max()) == 0
