@@ -108,7 +108,10 @@ def test_random_operands_within_bf16_rounding(tA, tB):
     assert max_rel <= 2**-8 and frob_rel <= 2**-8
 
 
-@pytest.mark.parametrize("M_list,I,K", [([100, 0, 300, 1], 128, 64), ([512, 260], 1408, 256), ([40] * 16, 72, 520)])
+@pytest.mark.parametrize(
+    "M_list,I,K",
+    [([100, 0, 300, 1], 128, 64), ([512, 260], 1408, 256), ([40] * 16, 72, 520), ([3000, 0, 5000, 7000, 1, 4999], 1408, 520)],
+)
 def test_fused_swiglu_equals_gemm_then_swiglu(M_list, I, K):
     torch.manual_seed(I)
     E, R = len(M_list), sum(M_list)
