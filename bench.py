@@ -272,6 +272,37 @@ def main():
         hbm("swiglu_backward", 5 * R * I * s,
             lambda i: ok(lib.fma_swiglu_backward(h.data_ptr() + I * s, h.data_ptr(), da.data_ptr(), dh.data_ptr() + I * s,
                                                  dh.data_ptr(), R, I, es, es, I, es, es, BF16, stream)), n=10)
+        # router: x and the gate weight read once, logits / weights / choice / histogram written. Three copies of x
+        # (together larger than the 256 MiB last-level cache) are rotated so that every launch reads from HBM.
+        if want("router"):
+            wg = moe.gate.weight.detach()
+            xs3 = [x] + [x.clone() for _ in range(2)]
+            lg = torch.empty(T, E, **bf)
+            rw = torch.empty(T, k, **bf)
+            sel32 = torch.empty(T, k, dtype=torch.int32, device=dev)
+            cnt = torch.empty(E, dtype=torch.uint32, device=dev)
+            # as the MoE module calls it: without the optional histogram (which costs one more small launch)
+            hbm("router_topk", T * H * s + E * H * s + T * E * s + T * k * (s + 4),
+                lambda i: ok(lib.fma_router_topk(xs3[i % 3].data_ptr(), wg.data_ptr(), T, H, E, k, lg.data_ptr(),
+                                                 rw.data_ptr(), sel32.data_ptr(), None, BF16, stream)))
+            ok(lib.fma_router_topk(x.data_ptr(), wg.data_ptr(), T, H, E, k, lg.data_ptr(), rw.data_ptr(),
+                                   sel32.data_ptr(), cnt.data_ptr(), BF16, stream))
+            assert int(cnt.view(torch.int32).sum()) == T * k, "router histogram does not sum to T * top_k"
+
+            def aten_router(i):  # the same results from library calls: gate linear, top-k, fp32 softmax, cast
+                logits = torch.nn.functional.linear(xs3[i % 3], wg)
+                values, _ = logits.topk(k, dim=-1)
+                torch.softmax(values.float(), dim=-1).to(torch.bfloat16)
+
+            t = time_gpu(aten_router, 20, blocker=blocker)
+            kernels["router_aten(linear+topk+softmax, 4+ launches)"] = {"ms": t[0], "ms_mean": t[1]}
+            dlg = torch.randn(T, E, device=dev).bfloat16()
+            drw = torch.randn(T, k, device=dev).bfloat16()
+            dlg_out = torch.empty(T, E, **bf)
+            hbm("router_topk_backward", 3 * T * E * s + T * k * (s + 4),
+                lambda i: ok(lib.fma_router_topk_bwd(lg.data_ptr(), sel32.data_ptr(), drw.data_ptr(), dlg.data_ptr(), T,
+                                                     E, k, dlg_out.data_ptr(), BF16, stream)))
+            del xs3
         if want("build_routing_index"):
             ws_idx = torch.empty(max(lib.fma_moe_build_index_workspace_bytes(R, E), 4) // 4, dtype=torch.int32, device=dev)
             t = time_gpu(lambda i: ok(lib.fma_moe_build_index(selected_d.data_ptr(), 8, R, E, counts.data_ptr(),

@@ -43,6 +43,8 @@ SIGNATURES = {
     "fma_swiglu_backward": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _p]),
     "fma_grouped_gemm": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _i32, _i32, _f32, _i32, _p]),
     "fma_grouped_gemm_swiglu": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
+    "fma_router_topk": (_i32, [_p, _p, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _i32, _p]),
+    "fma_router_topk_bwd": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _p, _i32, _p]),
 }
 
 _lib = None

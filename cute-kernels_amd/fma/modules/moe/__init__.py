@@ -16,6 +16,7 @@ from ...ops.swiglu import swiglu_packed
 from .cuda_implementation import (
     build_routing_index,
     combine,
+    fused_router,
     gather_rows,
     grouped_gemm_experts,
     up_projection_swiglu_experts,
@@ -100,6 +101,8 @@ class MoE(nn.Module):
         self.intermediate_size = intermediate_size
 
         self.gate = nn.Linear(in_features=self.hidden_size, out_features=num_experts, bias=False)
+        # gate GEMM, top-k and softmax in one kernel wherever that kernel applies (16-bit activations on the GPU)
+        self.fuse_router = True
 
         self.c_fc = Experts(
             num_experts=num_experts,
@@ -139,7 +142,22 @@ class MoE(nn.Module):
 
         return hidden_states, router_logits
 
+    def _router_is_fusable(self, hidden_states: torch.Tensor) -> bool:
+        return (
+            self.fuse_router
+            and hidden_states.is_cuda
+            and hidden_states.dtype in (torch.bfloat16, torch.float16)
+            and self.gate.weight.dtype == hidden_states.dtype
+            and self.hidden_size % 8 == 0
+            and self.num_experts <= 1024
+            and self.top_k <= 64
+        )
+
     def _compute_routing_weights(self, hidden_states: torch.Tensor) -> tuple[torch.Tensor]:
+        if self._router_is_fusable(hidden_states):
+            # same three results; selected_experts comes back as int32, sorted by descending logit
+            return fused_router(hidden_states, self.gate.weight, self.top_k)
+
         router_logits = self.gate(hidden_states)
         router_weights, selected_experts = self._get_topk(router_logits)
 

@@ -146,6 +146,58 @@ def grouped_gemm_swiglu_cuda(
     _lib.check(rc, "grouped_gemm_swiglu_cuda")
 
 
+@custom_op(f"{LIBRARY_NAME}::router_topk_cuda", mutates_args={"logits", "weights", "selected", "counts"})
+def router_topk_cuda(
+    x: torch.Tensor,
+    gate_weight: torch.Tensor,
+    top_k: int,
+    logits: torch.Tensor,
+    weights: torch.Tensor,
+    selected: torch.Tensor,
+    counts: torch.Tensor | None,
+) -> None:
+    _lib.require_gpu(x, gate_weight, logits, weights, selected, counts)
+    T, H = x.shape
+    E = gate_weight.size(0)
+    assert gate_weight.shape == (E, H) and logits.shape == (T, E)
+    assert weights.shape == (T, top_k) and selected.shape == (T, top_k)
+    assert x.dtype == gate_weight.dtype == logits.dtype == weights.dtype and selected.dtype == torch.int32
+    assert counts is None or (counts.dtype == torch.uint32 and counts.numel() == E)
+    for t in (x, gate_weight, logits, weights, selected, counts):
+        assert t is None or t.is_contiguous()
+    with torch.cuda.device(x.device):
+        rc = _lib.load().fma_router_topk(
+            x.data_ptr(), gate_weight.data_ptr(), T, H, E, top_k, logits.data_ptr(), weights.data_ptr(),
+            selected.data_ptr(), _lib.ptr(counts), _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
+        )
+    _lib.check(rc, "router_topk_cuda")
+
+
+@custom_op(f"{LIBRARY_NAME}::router_topk_backward_cuda", mutates_args={"logits_grad"})
+def router_topk_backward_cuda(
+    logits: torch.Tensor,
+    selected: torch.Tensor,
+    weights_grad: torch.Tensor | None,
+    logits_output_grad: torch.Tensor | None,
+    logits_grad: torch.Tensor,
+) -> None:
+    _lib.require_gpu(logits, selected, weights_grad, logits_output_grad, logits_grad)
+    T, E = logits.shape
+    top_k = selected.size(1)
+    assert selected.shape == (T, top_k) and selected.dtype == torch.int32 and logits_grad.shape == (T, E)
+    assert logits_grad.dtype == logits.dtype
+    assert weights_grad is None or (weights_grad.shape == (T, top_k) and weights_grad.dtype == logits.dtype)
+    assert logits_output_grad is None or (logits_output_grad.shape == (T, E) and logits_output_grad.dtype == logits.dtype)
+    for t in (logits, selected, weights_grad, logits_output_grad, logits_grad):
+        assert t is None or t.is_contiguous()
+    with torch.cuda.device(logits.device):
+        rc = _lib.load().fma_router_topk_bwd(
+            logits.data_ptr(), selected.data_ptr(), _lib.ptr(weights_grad), _lib.ptr(logits_output_grad), T, E, top_k,
+            logits_grad.data_ptr(), _lib.dtype_code(logits.dtype), _lib.current_stream(logits.device),
+        )
+    _lib.check(rc, "router_topk_backward_cuda")
+
+
 # ---- index construction -----------------------------------------------------------------------------
 
 
@@ -173,6 +225,42 @@ def build_routing_index(
 
 
 # ---- autograd functions -----------------------------------------------------------------------------
+
+
+class _FusedRouter(torch.autograd.Function):
+    """(router_logits, router_weights, selected_experts) of MoE._compute_routing_weights
+    (fma/modules/moe/__init__.py:191-204) from one kernel. The backward forms the logits' gradient (softmax and top-k
+    backward plus whatever arrives for the logits themselves) in one kernel; the two products with it are GEMMs with
+    one tiny dimension (E) and go to the BLAS library like the backward of the reference's nn.Linear gate."""
+
+    @staticmethod
+    @ensure_contiguous
+    def forward(ctx, x: torch.Tensor, gate_weight: torch.Tensor, top_k: int):
+        T, E = x.size(0), gate_weight.size(0)
+        logits = torch.empty(T, E, device=x.device, dtype=x.dtype)
+        weights = torch.empty(T, top_k, device=x.device, dtype=x.dtype)
+        selected = torch.empty(T, top_k, device=x.device, dtype=torch.int32)
+        router_topk_cuda(x, gate_weight, top_k, logits, weights, selected, None)
+        ctx.save_for_backward(x, gate_weight, logits, selected)
+        ctx.mark_non_differentiable(selected)
+        ctx.set_materialize_grads(False)
+        return logits, weights, selected
+
+    @staticmethod
+    @ensure_contiguous
+    def backward(ctx, logits_output_grad, weights_grad, _):
+        x, gate_weight, logits, selected = ctx.saved_tensors
+        if logits_output_grad is None and weights_grad is None:
+            return None, None, None
+        logits_grad = torch.empty_like(logits)
+        router_topk_backward_cuda(logits, selected, weights_grad, logits_output_grad, logits_grad)
+        x_grad = logits_grad @ gate_weight if ctx.needs_input_grad[0] else None
+        gate_weight_grad = logits_grad.t() @ x if ctx.needs_input_grad[1] else None
+        return x_grad, gate_weight_grad, None
+
+
+def fused_router(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int):
+    return _FusedRouter.apply(x, gate_weight, top_k)
 
 
 class _GatherRows(torch.autograd.Function):

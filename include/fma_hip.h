@@ -41,6 +41,8 @@ extern "C" {
 /* limits (same values as the reference's: continuous_count forward.cu:12, grouped_gemm kernel.cu:38) */
 #define FMA_MAX_COUNT_BINS 16384
 #define FMA_MAX_GROUPS 1024
+/* largest top_k of the fused router */
+#define FMA_MAX_ROUTER_TOP_K 64
 
 /* ---- library ---------------------------------------------------------------------------- */
 
@@ -166,6 +168,34 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
  * swiglu_packed (fma/ops/swiglu/__init__.py:133-164, up/gate = chunk(2, -1) at :153). */
 int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, const uint32_t* M_arr,
                             int64_t E, int64_t I, int64_t K, int dtype, void* stream);
+
+/* ---- router ---------------------------------------------------------------------------------- */
+
+/* The router in one pass over x[T, H]:
+ *   logits[t, e]  = <x[t, :], gate_weight[e, :]>          fp32 accumulation, rounded to dtype   ([T, E])
+ *   selected[t, :] = the top_k columns of logits[t, :] (the rounded values), largest first; equal values
+ *                    in ascending column order; NaN ranks above every number                     (int32 [T, top_k])
+ *   weights[t, :] = softmax of those top_k logits, computed in fp32, rounded to dtype           ([T, top_k])
+ *   counts[e]     = #{(t, j) : selected[t, j] == e}   (uint32 [E]; fully overwritten; may be NULL)
+ * gate_weight: [E, H] row-major. dtype: FMA_BF16 or FMA_F16. H % 8 == 0, E <= FMA_MAX_GROUPS,
+ * top_k <= min(E, FMA_MAX_ROUTER_TOP_K). x and gate_weight 16-byte aligned.
+ * Replaces MoE._compute_routing_weights and MoE._get_topk (fma/modules/moe/__init__.py:191-204, 292-298:
+ * `self.gate(hidden_states)`, `topk` / `max`, `F.softmax(router_weights.float(), dim=-1).type_as(...)`); with
+ * counts it also yields what continuous_count(sorted_expert_idxs, num_experts) returns at :215-217. torch.topk
+ * leaves the order of equal values open; the order here is one of the orders it may return. */
+int fma_router_topk(const void* x, const void* gate_weight, int64_t T, int64_t H, int64_t E, int64_t top_k,
+                    void* logits, void* weights, int32_t* selected, uint32_t* counts, int dtype, void* stream);
+
+/* Backward of the top-k + softmax part of fma_router_topk: the gradient with respect to the logits.
+ *   d_out[t, :] = d_logits[t, :]                          (zeros if d_logits == NULL)
+ *   d_out[t, selected[t, j]] += round(s_j * (d_weights[t, j] - sum_i s_i d_weights[t, i]))
+ * with s = the fp32 softmax of the kept logits (recomputed from logits and selected), the product rounded to
+ * dtype and the sum rounded again, which is what autograd does for `softmax(values.float()).type_as(x)` after
+ * `topk` plus a second use of the logits (fma/modules/moe/__init__.py:193-202). d_weights may be NULL (zeros).
+ * d_out must not overlap d_logits. The gradients of x and gate_weight are then plain products with d_out. */
+int fma_router_topk_bwd(const void* logits, const int32_t* selected, const void* d_weights,
+                        const void* d_logits, int64_t T, int64_t E, int64_t top_k, void* d_out, int dtype,
+                        void* stream);
 
 #ifdef __cplusplus
 }

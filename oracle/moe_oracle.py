@@ -12,6 +12,9 @@ pinned (tests/test_oracle.py):
                           E=1 == torch.mm, equal groups == torch.bmm, all four layouts
   swiglu / swiglu_packed  F.silu, closed forms at gate=0, saturation, README derivative vs fp64 autograd
   routing_weights         softmax of top-k logits; k == E reduces to a full softmax
+  topk_lowest_index_first torch.topk's values, torch.sort(descending, stable) order, brute force with ties and NaN
+  router_from_logits      routing_weights on tie-free logits
+  router_logits_grad      closed form s * (dw - <s, dw>) scattered to the kept columns; rows sum to zero
   moe_experts / moe_layer E=1,k=1 collapses to a dense SwiGLU MLP; token-permutation equivariance; zero-token
                           experts get exactly zero weight gradient; fp64 gradcheck on a tiny layer
 No function here is "parity unpinned".
@@ -144,6 +147,51 @@ def routing_weights(
         values, selected = router_logits.topk(top_k, dim=-1)
     weights = F.softmax(values.float(), dim=-1).type_as(hidden_states)
     return router_logits, weights, selected
+
+
+def topk_lowest_index_first(logits: np.ndarray, top_k: int) -> np.ndarray:
+    """int64 [T, k]: columns of the k largest entries of every row, largest first, equal values in ascending column
+    order, NaN ranked above every number. torch.topk / torch.max (fma/modules/moe/__init__.py:292-298) fix the
+    selected VALUES; among equal values they leave the choice and the order open, and this is the one order the
+    fused router kernel is specified to return."""
+    a = np.asarray(logits, dtype=np.float64)
+    key = np.where(np.isnan(a), np.inf, a)
+    # a stable sort of the negated keys keeps equal values in ascending column order
+    return np.argsort(-key, axis=-1, kind="stable")[:, :top_k].astype(np.int64)
+
+
+def router_from_logits(router_logits: torch.Tensor, top_k: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """(router_weights [T,k] in the logits' dtype, selected_experts [T,k] int64) from given logits: the part of
+    MoE._compute_routing_weights after the gate (fma/modules/moe/__init__.py:196-202) with the tie order above."""
+    selected = torch.from_numpy(topk_lowest_index_first(router_logits.detach().float().cpu().numpy(), top_k))
+    values = router_logits.detach().cpu().gather(1, selected)
+    weights = F.softmax(values.float(), dim=-1).to(router_logits.dtype)
+    return weights, selected
+
+
+def router_logits_grad(
+    router_logits: torch.Tensor,
+    selected: torch.Tensor,
+    weights_grad: torch.Tensor | None,
+    logits_output_grad: torch.Tensor | None,
+) -> torch.Tensor:
+    """Gradient reaching router_logits through autograd of fma/modules/moe/__init__.py:196-202 (gather of the kept
+    logits = what topk's backward scatters through, .float(), softmax, cast back) when router_weights receives
+    weights_grad and router_logits itself (returned by MoE.forward for auxiliary losses) receives logits_output_grad."""
+    logits = router_logits.detach().cpu().clone().requires_grad_()
+    values = logits.gather(1, selected.cpu().long())
+    weights = F.softmax(values.float(), dim=-1).to(logits.dtype)
+    outputs, grads = [], []
+    if weights_grad is not None:
+        outputs.append(weights)
+        grads.append(weights_grad.detach().cpu())
+    if logits_output_grad is not None:
+        outputs.append(logits * 1)
+        grads.append(logits_output_grad.detach().cpu())
+    if not outputs:
+        return torch.zeros_like(logits)
+    torch.autograd.backward(outputs, grads)
+    return logits.grad.detach()
 
 
 def moe_experts(

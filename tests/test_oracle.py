@@ -167,6 +167,53 @@ def test_routing_weights_properties():
     assert torch.equal(s1[:, 0], logits.argmax(-1)) and torch.equal(w1, torch.ones(33, 1))
 
 
+def test_topk_order_against_torch_and_brute_force():
+    rng = np.random.default_rng(5)
+    # bf16-like logits with many exact ties
+    logits = np.round(rng.standard_normal((257, 24)) * 4) / 4
+    for k in (1, 2, 5, 24):
+        got = O.topk_lowest_index_first(logits, k)
+        t = torch.from_numpy(logits)
+        # the selected values are what torch.topk selects (the values are unique as a sorted list even with ties)
+        assert torch.equal(t.gather(1, torch.from_numpy(got)), t.topk(k, dim=-1).values)
+        # and the order is that of a stable descending sort
+        assert np.array_equal(got, torch.sort(t, dim=-1, descending=True, stable=True).indices[:, :k].numpy())
+    # brute force: repeatedly take the first maximum
+    for row in logits[:40]:
+        left, expect = list(enumerate(row)), []
+        for _ in range(6):
+            best = max(v for _, v in left)
+            idx = min(i for i, v in left if v == best)
+            expect.append(idx)
+            left = [(i, v) for i, v in left if i != idx]
+        assert list(O.topk_lowest_index_first(row[None], 6)[0]) == expect
+    # NaN ranks first (torch.topk's convention), lowest column first among NaNs
+    nan_row = np.array([[0.5, np.nan, 3.0, np.nan, 3.0]])
+    assert list(O.topk_lowest_index_first(nan_row, 4)[0]) == [1, 3, 2, 4]
+    assert list(torch.from_numpy(nan_row).topk(2).indices[0].sort().values) == [1, 3]
+
+
+def test_router_from_logits_and_its_gradient():
+    torch.manual_seed(4)
+    x, w = torch.randn(50, 32), torch.randn(12, 32)
+    logits, weights, selected = O.routing_weights(x, w, 4)  # continuous random logits: no ties
+    w2, s2 = O.router_from_logits(logits, 4)
+    assert torch.equal(s2, selected) and torch.equal(w2, weights)
+
+    # gradient: closed form of softmax backward scattered to the kept columns, plus the direct term; the softmax
+    # itself runs in fp32 as in the reference (values.float()), hence the 1e-6
+    logits64 = logits.double()
+    dw, dl = torch.randn(50, 4).double(), torch.randn(50, 12).double()
+    got = O.router_logits_grad(logits64, selected, dw, dl)
+    s = F.softmax(logits64.gather(1, selected), dim=-1)
+    ds = s * (dw - (s * dw).sum(-1, keepdim=True))
+    assert torch.allclose(got, dl.clone().scatter_add(1, selected, ds), atol=1e-6, rtol=0)
+    assert torch.allclose(O.router_logits_grad(logits64, selected, dw, None), torch.zeros(50, 12).double().scatter_add(1, selected, ds), atol=1e-6, rtol=0)
+    assert torch.equal(O.router_logits_grad(logits64, selected, None, dl), dl)
+    # shifting all logits of a token leaves the weights unchanged: the rows of the softmax part sum to zero
+    assert float(O.router_logits_grad(logits64, selected, dw, None).sum(-1).abs().max()) < 1e-6
+
+
 def test_layer_collapses_to_dense_mlp():
     # E = 1, k = 1: softmax of one logit is 1, so the layer is linear -> swiglu -> linear
     torch.manual_seed(3)
