@@ -303,6 +303,28 @@ def main():
                 lambda i: ok(lib.fma_router_topk_bwd(lg.data_ptr(), sel32.data_ptr(), drw.data_ptr(), dlg.data_ptr(), T,
                                                      E, k, dlg_out.data_ptr(), BF16, stream)))
             del xs3
+        # residual add + RMSNorm on the layer's residual stream [T, H]: forward reads x and the residual and writes the
+        # normalised activations and the new residual; backward reads the saved residual and both incoming gradients and
+        # writes the two input gradients (plus the per-workgroup partial weight gradients and their sum)
+        if want("rmsnorm"):
+            res_in = torch.randn(T, H, device=dev).bfloat16()
+            nw = (1 + 0.1 * torch.randn(H, device=dev)).bfloat16()
+            n_out, n_added = torch.empty(T, H, **bf), torch.empty(T, H, **bf)
+            n_inv = torch.empty(T, dtype=torch.float32, device=dev)
+            hbm("fused_residual_add_rmsnorm_fwd", 4 * T * H * s + H * s + T * 4,
+                lambda i: ok(lib.fma_fused_residual_add_rmsnorm_fwd(x.data_ptr(), res_in.data_ptr(), nw.data_ptr(),
+                                                                    n_out.data_ptr(), n_added.data_ptr(), n_inv.data_ptr(),
+                                                                    T, H, 1e-5, 1.0, BF16, stream)))
+            ws_n = torch.empty(max(lib.fma_fused_residual_add_rmsnorm_bwd_workspace_bytes(T, H), 4), dtype=torch.uint8,
+                               device=dev)
+            n_dx, n_dres = torch.empty(T, H, **bf), torch.empty(T, H, **bf)
+            n_dw = torch.empty(H, dtype=torch.float32, device=dev)
+            hbm("fused_residual_add_rmsnorm_bwd(2 launches)", 5 * T * H * s + H * (s + 4) + T * 4,
+                lambda i: ok(lib.fma_fused_residual_add_rmsnorm_bwd(n_added.data_ptr(), nw.data_ptr(), dy.data_ptr(),
+                                                                    d_o.data_ptr(), n_inv.data_ptr(), n_dx.data_ptr(),
+                                                                    n_dres.data_ptr(), n_dw.data_ptr(), T, H, 1e-5, 1.0,
+                                                                    ws_n.data_ptr(), ws_n.numel(), BF16, stream)))
+            del res_in, n_out, n_added, n_dx, n_dres, ws_n
         if want("build_routing_index"):
             ws_idx = torch.empty(max(lib.fma_moe_build_index_workspace_bytes(R, E), 4) // 4, dtype=torch.int32, device=dev)
             t = time_gpu(lambda i: ok(lib.fma_moe_build_index(selected_d.data_ptr(), 8, R, E, counts.data_ptr(),

@@ -43,6 +43,8 @@ extern "C" {
 #define FMA_MAX_GROUPS 1024
 /* largest top_k of the fused router */
 #define FMA_MAX_ROUTER_TOP_K 64
+/* longest row of the normalisation kernels (the reference's MAX_TRITON_BLOCK_SIZE, fma/constants.py:17) */
+#define FMA_MAX_NORM_HIDDEN 65536
 
 /* ---- library ---------------------------------------------------------------------------- */
 
@@ -196,6 +198,42 @@ int fma_router_topk(const void* x, const void* gate_weight, int64_t T, int64_t H
 int fma_router_topk_bwd(const void* logits, const int32_t* selected, const void* d_weights,
                         const void* d_logits, int64_t T, int64_t E, int64_t top_k, void* d_out, int dtype,
                         void* stream);
+
+/* ---- residual add + RMSNorm ------------------------------------------------------------------- */
+
+/* For each of the B rows of H elements, in fp32:
+ *   r   = x * multiplier + residual                    -> added_x_residual (rounded to dtype)
+ *   inv = 1 / sqrt(mean(r^2) + eps)  (unrounded r)      -> rmsnorm_denominator[row] (fp32; may be NULL)
+ *   out = r * inv * weight                              -> output (one rounding; weight may be NULL = ones)
+ * multiplier = 1 stands for the reference's `multiplier=None`. Any H in [1, FMA_MAX_NORM_HIDDEN]; rows of a
+ * multiple of 16 bytes (and 16-byte aligned pointers) up to 32 KB take the single-pass kernels.
+ * dtype: FMA_F32 / FMA_F16 / FMA_BF16; weight has the dtype of x.
+ * Replaces fused_residual_add_rmsnorm_forward_triton(x, residual, weight, output, eps, multiplier,
+ * added_x_residual, rmsnorm_denominator) (fma/ops/fused_residual_add_rmsnorm/triton_implementation/forward.py:16-102;
+ * torch formulation at fma/ops/fused_residual_add_rmsnorm/__init__.py:113-120). */
+int fma_fused_residual_add_rmsnorm_fwd(const void* x, const void* residual, const void* weight, void* output,
+                                       void* added_x_residual, float* rmsnorm_denominator, int64_t B, int64_t H,
+                                       float eps, float multiplier, int dtype, void* stream);
+
+/* Bytes of workspace the backward needs when a weight gradient is asked for (no initialisation required). */
+int64_t fma_fused_residual_add_rmsnorm_bwd_workspace_bytes(int64_t B, int64_t H);
+
+/* Backward of the above for the gradients output_grad (of out) and added_x_residual_grad (of r as the second
+ * output; may be NULL = zeros). With g = output_grad * weight and inv from rmsnorm_denominator (NULL: recomputed
+ * from the stored r):
+ *   residual_grad = inv * g - inv^3 / H * r * <g, r> + added_x_residual_grad
+ *   x_grad        = multiplier * residual_grad
+ *   weight_grad[h] = sum over rows of output_grad[., h] * round(r[., h] * inv[.])   (fp32 [H], fully overwritten)
+ * weight and weight_grad are both given or both NULL. The weight gradient is summed in a fixed order (per
+ * workgroup in row order, then over workgroups), so it is the same bits on every run; the reference adds with atomics.
+ * Replaces fused_residual_add_rmsnorm_backward_triton(added_x_residual, weight, output_grad, added_x_residual_grad,
+ * rmsnorm_denominator, x_grad, residual_grad, weight_grad, eps, multiplier)
+ * (fma/ops/fused_residual_add_rmsnorm/triton_implementation/backward.py:15-145). */
+int fma_fused_residual_add_rmsnorm_bwd(const void* added_x_residual, const void* weight, const void* output_grad,
+                                       const void* added_x_residual_grad, const float* rmsnorm_denominator,
+                                       void* x_grad, void* residual_grad, float* weight_grad, int64_t B, int64_t H,
+                                       float eps, float multiplier, void* workspace, int64_t workspace_bytes,
+                                       int dtype, void* stream);
 
 #ifdef __cplusplus
 }

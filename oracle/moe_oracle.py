@@ -17,6 +17,8 @@ pinned (tests/test_oracle.py):
   router_logits_grad      closed form s * (dw - <s, dw>) scattered to the kept columns; rows sum to zero
   moe_experts / moe_layer E=1,k=1 collapses to a dense SwiGLU MLP; token-permutation equivariance; zero-token
                           experts get exactly zero weight gradient; fp64 gradcheck on a tiny layer
+  fused_residual_add_rmsnorm  the definition written out in fp64 (r / sqrt(mean(r^2) + eps) * w), unit RMS of the
+                          unweighted output, invariance to scaling the input (eps = 0), fp64 gradcheck
 No function here is "parity unpinned".
 """
 
@@ -240,6 +242,20 @@ def moe_layer(
     router_logits, weights, selected = routing_weights(x, gate_weight, top_k)
     y = moe_experts(x, weights, selected, w_fc, w_proj, activation)
     return y.reshape(shape), router_logits
+
+
+def fused_residual_add_rmsnorm(
+    x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor | None, eps: float | None, multiplier: float | None = None
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """(normalised activations, updated residual stream): the torch branch of fused_residual_add_rmsnorm
+    (fma/ops/fused_residual_add_rmsnorm/__init__.py:113-120): optional pre-multiplication of x, residual add,
+    F.rms_norm over the last dimension (eps=None means the dtype's machine epsilon, as torch defines it)."""
+    if multiplier not in [None, 1]:
+        x = x * multiplier
+    x = x + residual
+    residual = x
+    x = F.rms_norm(x, (x.size(-1),), weight=weight, eps=eps)
+    return x, residual
 
 
 # ---- synthetic inputs of the benchmark configurations ----------------------------------------------------------

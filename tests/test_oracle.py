@@ -214,6 +214,39 @@ def test_router_from_logits_and_its_gradient():
     assert float(O.router_logits_grad(logits64, selected, dw, None).sum(-1).abs().max()) < 1e-6
 
 
+def test_fused_residual_add_rmsnorm_definition_and_invariants():
+    torch.manual_seed(8)
+    x, res, w = torch.randn(19, 37).double(), torch.randn(19, 37).double(), torch.randn(37).double()
+    for weight in (None, w):
+        for mult in (None, 0.9):
+            out, r = O.fused_residual_add_rmsnorm(x, res, weight, 1e-5, mult)
+            r_expect = x * (1.0 if mult is None else mult) + res
+            assert torch.allclose(r, r_expect, atol=1e-14)
+            expect = r_expect / torch.sqrt((r_expect**2).mean(-1, keepdim=True) + 1e-5)
+            if weight is not None:
+                expect = expect * weight
+            assert torch.allclose(out, expect, atol=1e-12)
+    # brute force on one row
+    out, r = O.fused_residual_add_rmsnorm(x, res, w, 1e-5, 0.9)
+    row = [0.9 * float(a) + float(b) for a, b in zip(x[3], res[3])]
+    inv = (sum(v * v for v in row) / len(row) + 1e-5) ** -0.5
+    assert all(abs(float(out[3, h]) - row[h] * inv * float(w[h])) < 1e-12 for h in range(37))
+    # unweighted output has unit root-mean-square (up to eps); scaling the input changes nothing when eps = 0
+    out, _ = O.fused_residual_add_rmsnorm(x, res, None, 1e-12)
+    assert torch.allclose((out**2).mean(-1), torch.ones(19).double(), atol=1e-9)
+    a, _ = O.fused_residual_add_rmsnorm(x, res, w, 0.0)
+    b, _ = O.fused_residual_add_rmsnorm(7 * x, 7 * res, w, 0.0)
+    assert torch.allclose(a, b, atol=1e-12)
+    # eps=None: the dtype's machine epsilon
+    c, _ = O.fused_residual_add_rmsnorm(x.float(), res.float(), None, None)
+    d, _ = O.fused_residual_add_rmsnorm(x.float(), res.float(), None, torch.finfo(torch.float32).eps)
+    assert torch.equal(c, d)
+    # gradients of both outputs
+    xs, rs, ws = (t[:3, :5].clone().requires_grad_() for t in (x, res, x[:1].expand(3, 37)))
+    wv = w[:5].clone().requires_grad_()
+    assert torch.autograd.gradcheck(lambda a_, b_, c_: O.fused_residual_add_rmsnorm(a_, b_, c_, 1e-5, 0.9), (xs, rs, wv))
+
+
 def test_layer_collapses_to_dense_mlp():
     # E = 1, k = 1: softmax of one logit is 1, so the layer is linear -> swiglu -> linear
     torch.manual_seed(3)
