@@ -325,6 +325,18 @@ def main():
                                                                     n_dres.data_ptr(), n_dw.data_ptr(), T, H, 1e-5, 1.0,
                                                                     ws_n.data_ptr(), ws_n.numel(), BF16, stream)))
             del res_in, n_out, n_added, n_dx, n_dres, ws_n
+        # per-expert bias on the up-projection's output [R, 2I] (layers built with add_bias=True)
+        if want("expert_bias"):
+            b1 = torch.randn(E, 2 * I, device=dev).bfloat16()
+            db1 = torch.empty(E, 2 * I, **bf)
+            ws_b = torch.empty(max(lib.fma_expert_bias_grad_workspace_bytes(E, R, 2 * I), 4), dtype=torch.uint8,
+                               device=dev)
+            hbm("expert_bias_add", 2 * R * 2 * I * s + E * 2 * I * s,
+                lambda i: ok(lib.fma_expert_bias_add(h.data_ptr(), b1.data_ptr(), counts.data_ptr(), E, R, 2 * I, BF16,
+                                                     stream)), n=10)
+            hbm("expert_bias_grad(2 launches)", R * 2 * I * s + E * 2 * I * s,
+                lambda i: ok(lib.fma_expert_bias_grad(dh.data_ptr(), counts.data_ptr(), E, R, 2 * I, db1.data_ptr(),
+                                                      ws_b.data_ptr(), ws_b.numel(), BF16, stream)), n=10)
         if want("build_routing_index"):
             ws_idx = torch.empty(max(lib.fma_moe_build_index_workspace_bytes(R, E), 4) // 4, dtype=torch.int32, device=dev)
             t = time_gpu(lambda i: ok(lib.fma_moe_build_index(selected_d.data_ptr(), 8, R, E, counts.data_ptr(),

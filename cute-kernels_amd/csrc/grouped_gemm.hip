@@ -574,14 +574,8 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         const uint32_t band_m = tiles_m - first_m < (uint32_t)kGroupM ? tiles_m - first_m : (uint32_t)kGroupM;
         const uint32_t mt = first_m + (local % band) % band_m;
         const uint32_t nt = (local % band) / band_m;
-#if defined(FMA_EXPERIMENT_SAME_TILE)
-        t.m0 = 0, t.n0 = 0;  // diagnostic build: every workgroup reads the same, cache-resident tile
-        (void)mt;
-        (void)nt;
-#else
         t.m0 = mt * BM;
         t.n0 = nt * TN;
-#endif
         t.off_a = uniform(s_off_a[e]);
         t.off_b = uniform(s_off_b[e]);
         t.off_d = uniform(s_off_d[e]);
@@ -626,9 +620,6 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     };
     // loads of the K step at k0 into `stage`: inside the K loop (compiler-visible, placed by the scheduling hints) ...
     auto issue = [&](int stage, uint32_t k0) {
-#if defined(FMA_EXPERIMENT_SKIP_LOADS)
-        if (k0 >= 2 * BK) return;  // diagnostic build: steady-state loads removed (results are wrong)
-#endif
         if constexpr (A_KC) lk_a.issue(stage ? s_a1 : s_a0, k0);
         else lt_a.issue(stage ? s_a1 : s_a0, k0);
         if constexpr (B_KC) lk_b.issue(stage ? s_b1 : s_b0, k0);

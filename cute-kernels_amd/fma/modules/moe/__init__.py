@@ -14,6 +14,7 @@ import torch.nn.functional as F
 from ...kernel_backend import KernelBackend, is_hip_kernel_backend
 from ...ops.swiglu import swiglu_packed
 from .cuda_implementation import (
+    add_expert_bias,
     build_routing_index,
     combine,
     fused_router,
@@ -47,15 +48,18 @@ class Experts(nn.Module):
         self.reset_parameters()
 
     def cuda_forward(self, input: torch.Tensor, expert_frequency: torch.Tensor) -> torch.Tensor:
-        # like the reference's cuda_forward (fma/modules/moe/__init__.py:89-92) the grouped GEMM has no bias term
-        assert self.bias is None, "the grouped-GEMM experts do not implement a bias"
-        return grouped_gemm_experts(
+        # the reference's cuda_forward (fma/modules/moe/__init__.py:89-92) silently drops the bias; here it is added
+        # to the rows of every expert, which is what its torch_forward computes (:98-105)
+        output = grouped_gemm_experts(
             x=input, weight=self.weight, M_array=expert_frequency, N_array=self.N_array, K_array=self.K_array
         )
+        if self.bias is not None:
+            output = add_expert_bias(output, self.bias, expert_frequency)
+        return output
 
     def cuda_forward_swiglu(self, input: torch.Tensor, expert_frequency: torch.Tensor) -> torch.Tensor:
         """up-projection with swiglu_packed fused into the GEMM epilogue: returns [sum(M), out_features / 2]"""
-        assert self.bias is None, "the grouped-GEMM experts do not implement a bias"
+        assert self.bias is None, "the fused epilogue has no bias term: use cuda_forward followed by the activation"
         return up_projection_swiglu_experts(
             x=input, weight=self.weight, M_array=expert_frequency, N_array=self.N_array, K_array=self.K_array
         )
@@ -114,7 +118,7 @@ class MoE(nn.Module):
 
         self.act = activation_function
         # swiglu_packed as the activation of a GLU layer is computed inside the up-projection's epilogue
-        self.fuse_swiglu = is_glu and _is_swiglu_packed(activation_function)
+        self.fuse_swiglu = is_glu and _is_swiglu_packed(activation_function) and not add_bias
 
         self.c_proj = Experts(
             num_experts=num_experts,

@@ -146,6 +146,40 @@ def grouped_gemm_swiglu_cuda(
     _lib.check(rc, "grouped_gemm_swiglu_cuda")
 
 
+@custom_op(f"{LIBRARY_NAME}::expert_bias_add_cuda", mutates_args={"y"})
+def expert_bias_add_cuda(y: torch.Tensor, bias: torch.Tensor, M_array: torch.Tensor) -> None:
+    _lib.require_gpu(y, bias, M_array)
+    E, N = bias.shape
+    assert y.dim() == 2 and y.size(1) == N and y.dtype == bias.dtype
+    assert M_array.dtype == torch.uint32 and M_array.numel() == E
+    assert y.is_contiguous() and bias.is_contiguous() and M_array.is_contiguous()
+    with torch.cuda.device(y.device):
+        rc = _lib.load().fma_expert_bias_add(
+            y.data_ptr(), bias.data_ptr(), M_array.data_ptr(), E, y.size(0), N, _lib.dtype_code(y.dtype),
+            _lib.current_stream(y.device),
+        )
+    _lib.check(rc, "expert_bias_add_cuda")
+
+
+@custom_op(f"{LIBRARY_NAME}::expert_bias_grad_cuda", mutates_args={"bias_grad"})
+def expert_bias_grad_cuda(output_grad: torch.Tensor, M_array: torch.Tensor, bias_grad: torch.Tensor) -> None:
+    _lib.require_gpu(output_grad, M_array, bias_grad)
+    E, N = bias_grad.shape
+    assert output_grad.dim() == 2 and output_grad.size(1) == N and output_grad.dtype == bias_grad.dtype
+    assert M_array.dtype == torch.uint32 and M_array.numel() == E
+    assert output_grad.is_contiguous() and bias_grad.is_contiguous() and M_array.is_contiguous()
+    lib = _lib.load()
+    code = _lib.dtype_code(output_grad.dtype)
+    with torch.cuda.device(output_grad.device):
+        nbytes = max(lib.fma_expert_bias_grad_workspace_bytes(E, output_grad.size(0), N), 4)
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=output_grad.device)  # per-slice partial sums
+        rc = lib.fma_expert_bias_grad(
+            output_grad.data_ptr(), M_array.data_ptr(), E, output_grad.size(0), N, bias_grad.data_ptr(),
+            workspace.data_ptr(), nbytes, code, _lib.current_stream(output_grad.device),
+        )
+    _lib.check(rc, "expert_bias_grad_cuda")
+
+
 @custom_op(f"{LIBRARY_NAME}::router_topk_cuda", mutates_args={"logits", "weights", "selected", "counts"})
 def router_topk_cuda(
     x: torch.Tensor,
@@ -375,6 +409,34 @@ class _GroupedGemmExperts(torch.autograd.Function):
             )
 
         return x_grad, weight_grad, None, None, None
+
+
+class _ExpertBias(torch.autograd.Function):
+    """y_e += bias[e] on the packed rows of every expert, in place on the grouped GEMM's fresh output (which no other
+    node needs: the GEMM's backward reads its inputs, not its output); backward sums the rows of every expert."""
+
+    @staticmethod
+    def forward(ctx, y: torch.Tensor, bias: torch.Tensor, M_array: torch.Tensor) -> torch.Tensor:
+        assert y.is_contiguous()
+        expert_bias_add_cuda(y, bias.contiguous(), M_array)
+        ctx.mark_dirty(y)
+        ctx.save_for_backward(M_array)
+        ctx.bias_shape = bias.shape
+        return y
+
+    @staticmethod
+    @ensure_contiguous
+    def backward(ctx, output_grad: torch.Tensor) -> tuple[torch.Tensor | None]:
+        (M_array,) = ctx.saved_tensors
+        bias_grad = None
+        if ctx.needs_input_grad[1]:
+            bias_grad = torch.empty(ctx.bias_shape, device=output_grad.device, dtype=output_grad.dtype)
+            expert_bias_grad_cuda(output_grad, M_array, bias_grad)
+        return output_grad, bias_grad, None
+
+
+def add_expert_bias(y: torch.Tensor, bias: torch.Tensor, M_array: torch.Tensor) -> torch.Tensor:
+    return _ExpertBias.apply(y, bias, M_array)
 
 
 class _UpProjectionSwiglu(torch.autograd.Function):

@@ -171,6 +171,25 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
 int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, const uint32_t* M_arr,
                             int64_t E, int64_t I, int64_t K, int dtype, void* stream);
 
+/* ---- per-expert bias ------------------------------------------------------------------------ */
+
+/* y[i, :] += bias[e, :] for every row i of expert e, rows packed expert by expert with M_arr[e] rows each (device
+ * array, as for fma_grouped_gemm); fp32 addition, one rounding; rows past sum(M_arr) are left alone. y: [R, N],
+ * bias: [E, N], N * element size a multiple of 16. Together with fma_grouped_gemm this is the per-expert
+ * `F.linear(x_e, W[e], bias[e])` of Experts.torch_forward (fma/modules/moe/__init__.py:98-105); the reference's
+ * grouped-GEMM path drops the bias (:89-92) and its Triton path refuses it (:48, :73). */
+int fma_expert_bias_add(void* y, const void* bias, const uint32_t* M_arr, int64_t E, int64_t R, int64_t N, int dtype,
+                        void* stream);
+
+/* Bytes of workspace fma_expert_bias_grad needs (no initialisation required). */
+int64_t fma_expert_bias_grad_workspace_bytes(int64_t E, int64_t R, int64_t N);
+
+/* d_bias[e, :] = sum of the rows dy[i, :] of expert e (zeros for an expert without rows), accumulated in fp32 per
+ * slice of up to 256 rows in row order, slices added in order in fp64, rounded once to dtype: the gradient autograd gives the
+ * bias of `F.linear(x_e, W[e], bias[e])` (fma/modules/moe/__init__.py:98-105). d_bias: [E, N], fully overwritten. */
+int fma_expert_bias_grad(const void* dy, const uint32_t* M_arr, int64_t E, int64_t R, int64_t N, void* d_bias,
+                         void* workspace, int64_t workspace_bytes, int dtype, void* stream);
+
 /* ---- router ---------------------------------------------------------------------------------- */
 
 /* The router in one pass over x[T, H]:

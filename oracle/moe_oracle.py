@@ -203,11 +203,14 @@ def moe_experts(
     w_fc: torch.Tensor,
     w_proj: torch.Tensor,
     activation: Callable[[torch.Tensor], torch.Tensor] = swiglu_packed,
+    b_fc: torch.Tensor | None = None,
+    b_proj: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """The torch branch of MoE._compute_experts (fma/modules/moe/__init__.py:267-286) with Experts.torch_forward
     (:94-110): sort slots by expert, gather x[slot // k], per-expert F.linear, activation, per-expert F.linear,
     scale by the gathered router weights, index_add back to tokens. Differentiable (autograd gives the oracle's
-    gradients). w_fc: [E, 2I or I, H]; w_proj: [E, H, I]; no bias.
+    gradients). w_fc: [E, 2I or I, H]; w_proj: [E, H, I]; optional biases b_fc: [E, 2I or I], b_proj: [E, H]
+    (F.linear(x_e, W[e], bias[e]), :103-105).
     """
     T, H = hidden_states.shape
     E = w_fc.size(0)
@@ -220,9 +223,9 @@ def moe_experts(
     batch_gates = router_weights.flatten()[perm]  # :272-273
     x = hidden_states[fan_in_index]  # :275
     xs = x.split(counts, dim=0)  # :98
-    hs = [F.linear(xs[e], w_fc[e]) for e in range(E)]  # :102-105
+    hs = [F.linear(xs[e], w_fc[e], None if b_fc is None else b_fc[e]) for e in range(E)]  # :102-105
     hs = [activation(h) for h in hs]  # :281
-    ys = torch.cat([F.linear(hs[e], w_proj[e]) for e in range(E)], dim=0)  # :282
+    ys = torch.cat([F.linear(hs[e], w_proj[e], None if b_proj is None else b_proj[e]) for e in range(E)], dim=0)  # :282
     ys = ys * batch_gates.unsqueeze(-1)  # :284
     zeros = torch.zeros((T, H), dtype=ys.dtype, device=ys.device)
     return zeros.index_add(0, fan_in_index, ys)  # :285-286

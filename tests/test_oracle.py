@@ -257,6 +257,18 @@ def test_layer_collapses_to_dense_mlp():
     h = x @ w1[0].T
     dense = (h[:, :I] * F.silu(h[:, I:])) @ w2[0].T
     assert torch.allclose(y, dense, atol=1e-5)
+    # with biases: a dense MLP with biases
+    b1, b2 = torch.randn(1, 2 * I), torch.randn(1, H)
+    sel, ones = torch.zeros(T, 1, dtype=torch.long), torch.ones(T, 1)
+    yb = O.moe_experts(x, ones, sel, w1, w2, O.swiglu_packed, b1, b2)
+    hb = x @ w1[0].T + b1[0]
+    assert torch.allclose(yb, (hb[:, :I] * F.silu(hb[:, I:])) @ w2[0].T + b2[0], atol=1e-5)
+    # every expert adds its own bias: with zero weights the output is the gate-weighted sum of the chosen biases
+    E, k = 5, 2
+    sel2, gates = O.make_routing(T, E, k, "uniform", seed=3)
+    bias_out = torch.randn(E, H)
+    y0 = O.moe_experts(x, gates, sel2, torch.zeros(E, 2 * I, H), torch.zeros(E, H, I), O.swiglu_packed, None, bias_out)
+    assert torch.allclose(y0, (gates.unsqueeze(-1) * bias_out[sel2]).sum(1), atol=1e-6)
 
 
 def test_layer_against_per_token_loop():
