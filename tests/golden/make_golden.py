@@ -1,4 +1,4 @@
-"""Writes tests/golden/c1_moe_fp32.npz: BASELINE configuration 1 (T=512 tokens, hidden 256, SwiGLU intermediate 512,
+"""Writes tests/golden/c1_moe_fp32.npz: the small CPU-runnable configuration (T=512 tokens, hidden 256, SwiGLU intermediate 512,
 E=8, top-k 2, fp32; activations ~N(0,1), expert weights ~N(0,0.02), softmax top-k routing, seed 42) evaluated by the
 CPU oracle (oracle/moe_oracle.py). The reference's own tests hold no stored vectors for this path, and its Python
 is never imported: the oracle is pinned by tests/test_oracle.py instead.

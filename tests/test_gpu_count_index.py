@@ -37,7 +37,7 @@ def test_count_reference_generator(dtype):
 @pytest.mark.parametrize("kind", ["uniform", "zipf"])
 @pytest.mark.parametrize("np_dtype,dtype", [(np.int32, torch.int32), (np.int64, torch.int64)])
 def test_count_16m_ids(kind, np_dtype, dtype):
-    # BASELINE configuration: 16 Mi ids in [0, 64), uniform and Zipf(1.2)
+    # the histogram benchmark configuration: 16 Mi ids in [0, 64), uniform and Zipf(1.2)
     n, E = 16 << 20, 64
     ids = O.make_ids(n, E, kind, seed=11, dtype=np_dtype)
     x = torch.from_numpy(ids).to(DEV)

@@ -122,7 +122,7 @@ def test_moe_fp16(act_name):
 
 
 def test_moe_plumbing_config_against_golden_fixture():
-    # BASELINE configuration 1 (T=512, H=256, I=512, E=8, k=2): expected values were written by the fp32 oracle
+    # the small CPU-runnable configuration (T=512, H=256, I=512, E=8, k=2): expected values were written by the fp32 oracle
     # (tests/golden/make_golden.py); the HIP path runs it in bf16
     from golden.make_golden import c1_inputs
 
