@@ -22,6 +22,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
+PEAK_F32_TFLOPS = 157.3  # MI355X dense fp32 MFMA
 
 WORKLOADS = {
     # name: T, H, I, E, k, routing kind, experts forced empty
@@ -208,13 +209,13 @@ def main():
         def want(name):
             return not only or any(w in name for w in only)
 
-        def mfma(name, flops, fn, n=iters, nbytes=None):
+        def mfma(name, flops, fn, n=iters, nbytes=None, peak=PEAK_BF16_TFLOPS):
             if not want(name):
                 return
             t = time_gpu(fn, n, blocker=blocker)
             tf = flops / (t[0] * 1e-3) / 1e12
-            kernels[name] = {"ms": t[0], "ms_mean": t[1], "bound": "mfma", "achieved": tf, "peak": PEAK_BF16_TFLOPS,
-                             "unit": "TFLOP/s", "frac": tf / PEAK_BF16_TFLOPS, "flop": flops}
+            kernels[name] = {"ms": t[0], "ms_mean": t[1], "bound": "mfma", "achieved": tf, "peak": peak,
+                             "unit": "TFLOP/s", "frac": tf / peak, "flop": flops}
             if nbytes is not None:  # the second roof: operands read once, output written once
                 kernels[name]["hbm_bytes"] = nbytes
                 kernels[name]["hbm_frac"] = nbytes / (t[0] * 1e-3) / 1e9 / PEAK_HBM_GBS
@@ -245,6 +246,17 @@ def main():
              nbytes=R * 2 * I * s + w1_b + R * H * s)
         mfma("up_projection_wgrad(TN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, xg, dw1, N_fc, K_fc, counts, 1, 0),
              nbytes=R * 2 * I * s + R * H * s + w1_b)
+
+        # the fp32 grouped GEMM (fp32 matrix instruction, 157.3 TFLOP/s peak) on the down-projection's forward shape;
+        # only on request (--only fp32): it is not part of the bf16 layer and takes 40 ms per launch
+        if only and want("down_projection_fwd_fp32(NT)"):
+            a32, w32 = a.float().normal_(), w2.float()
+            o32 = torch.empty(R, H, dtype=torch.float32, device=dev)
+            mfma("down_projection_fwd_fp32(NT)", 2.0 * R * I * H,
+                 lambda i: ok(lib.fma_grouped_gemm(a32.data_ptr(), w32.data_ptr(), o32.data_ptr(), counts.data_ptr(),
+                                                   N_pj.data_ptr(), K_pj.data_ptr(), E, 0, 1, 1.0, fma._lib.FMA_F32,
+                                                   stream)), n=3, peak=PEAK_F32_TFLOPS)
+            del a32, w32, o32
 
         # calibration for the profiler's FETCH_SIZE / WRITE_SIZE counters: a plain device copy of known size (ATen's
         # elementwise copy kernel): reads 1 GiB, writes 1 GiB

@@ -26,6 +26,7 @@
 //    columns of one output row. The epilogue transposes the wavefront's sub-tile through LDS (stage 1) and stores
 //    whole 128-byte row segments; the next tile's first loads are already on their way into stage 0 by then.
 #include "common.h"
+#include "grouped_gemm_f32.h"
 
 namespace fmahip {
 namespace gemm {
@@ -903,8 +904,7 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
                      void* stream) {
     using namespace fmahip;
     using namespace fmahip::gemm;
-    FMA_REQUIRE(dtype == FMA_BF16 || dtype == FMA_F16, dtype_bytes(dtype) ? FMA_ERR_UNSUPPORTED : FMA_ERR_BAD_DTYPE,
-                "grouped_gemm: bf16 and fp16 operands are implemented (dtype code %d)", dtype);
+    FMA_REQUIRE(dtype_bytes(dtype) != 0, FMA_ERR_BAD_DTYPE, "grouped_gemm: unknown dtype code %d", dtype);
     FMA_REQUIRE(E >= 0, FMA_ERR_BAD_SIZE, "grouped_gemm: negative group count %lld", (long long)E);
     FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "grouped_gemm: E=%lld exceeds the limit %d",
                 (long long)E, FMA_MAX_GROUPS);
@@ -912,6 +912,10 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
     FMA_REQUIRE(A && B && D && M_arr && N_arr && K_arr, FMA_ERR_NULL_POINTER, "grouped_gemm: NULL pointer");
     FMA_REQUIRE(aligned16(A) && aligned16(B) && aligned16(D), FMA_ERR_MISALIGNED,
                 "grouped_gemm: A, B and D must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const bool a_kc = trans_a == 0;  // A stored [M, K]: reduction dim contiguous
+    const bool b_kc = trans_b != 0;  // B stored [N, K]: reduction dim contiguous
+    if (dtype == FMA_F32) return gemm_f32::launch(A, B, D, M_arr, N_arr, K_arr, E, a_kc, b_kc, alpha, st);
     GemmArgs args{};
     args.A = (const uint16_t*)A;
     args.B = (const uint16_t*)B;
@@ -922,9 +926,6 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
     args.K_arr = K_arr;
     args.E = (uint32_t)E;
     args.alpha = alpha;
-    hipStream_t st = (hipStream_t)stream;
-    const bool a_kc = trans_a == 0;  // A stored [M, K]: reduction dim contiguous
-    const bool b_kc = trans_b != 0;  // B stored [N, K]: reduction dim contiguous
     return dtype == FMA_BF16 ? launch_plain<ElemBf16>(args, a_kc, b_kc, st) : launch_plain<ElemF16>(args, a_kc, b_kc, st);
 }
 

@@ -187,7 +187,7 @@ class MoE(nn.Module):
         # rows of every expert back to back: x[slot // top_k]
         hidden_states = gather_rows(hidden_states, sorted_scattered_idxs, inverse, self.top_k)
 
-        if self.fuse_swiglu:
+        if self.fuse_swiglu and hidden_states.dtype in (torch.bfloat16, torch.float16):
             hidden_states = self.c_fc.cuda_forward_swiglu(input=hidden_states, expert_frequency=expert_frequency)
         else:
             hidden_states = self.c_fc.cuda_forward(input=hidden_states, expert_frequency=expert_frequency)

@@ -150,9 +150,10 @@ int fma_swiglu_backward(const void* gate, const void* up, const void* dy, void* 
  *   trans_a == 0: A_e stored [M_e, K_e] row-major;  trans_a != 0: stored [K_e, M_e].
  *   trans_b != 0: B_e stored [N_e, K_e] row-major;  trans_b == 0: stored [K_e, N_e].
  * M_arr / N_arr / K_arr: E uint32 each, DEVICE memory (never read on the host). A group with K_e == 0
- * gets zeros; a group with M_e == 0 or N_e == 0 produces nothing. dtype: FMA_BF16 or FMA_F16.
- * Each group's contiguous dimension should be a multiple of 8 elements (16 bytes); other groups are
- * computed by a slow scalar path. E <= FMA_MAX_GROUPS.
+ * gets zeros; a group with M_e == 0 or N_e == 0 produces nothing. dtype: FMA_BF16, FMA_F16 or FMA_F32
+ * (fp32 runs on the fp32 matrix instruction, one sixteenth of the 16-bit rate, with no restriction on sizes).
+ * For the 16-bit types each group's contiguous dimension should be a multiple of 8 elements (16 bytes); other
+ * groups are computed by a slow scalar path. E <= FMA_MAX_GROUPS.
  * Replaces grouped_gemm_cuda(A, B, C, output, M_array, N_array, K_array, is_A_transposed,
  * is_B_transposed, alpha, beta, benchmark) (fma/ops/grouped_gemm/cuda_implementation/ops.cpp,
  * kernel.cu:354-388); beta must be 0 and C absent there, so neither exists here. */
