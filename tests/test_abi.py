@@ -85,7 +85,8 @@ def test_swiglu_and_gemm_validation(lib):
     assert lib.fma_swiglu_forward(p, p, p, 0, 8, 8, 8, 8, 2, None) == 0
     assert lib.fma_swiglu_backward(p, p, p, p, None, 4, 8, 8, 8, 8, 8, 8, 2, None) == -1
     assert lib.fma_grouped_gemm(p, p, p, p, p, p, 1025, 0, 1, 1.0, 2, None) == -4 and "1024" in _err(lib)
-    assert lib.fma_grouped_gemm(p, p, p, p, p, p, 4, 0, 1, 1.0, 0, None) == -8  # fp32 operands: not implemented
+    assert lib.fma_grouped_gemm(p + 4, p, p, p, p, p, 4, 0, 1, 1.0, 0, None) == -6  # fp32 operands: same alignment rule
+    assert lib.fma_grouped_gemm_swiglu(p, p, p, p, p, 4, 16, 64, 0, None) == -8  # the fused epilogue is 16-bit only
     assert lib.fma_grouped_gemm(p, p, p, p, p, p, 4, 0, 1, 1.0, 5, None) == -2
     assert lib.fma_grouped_gemm(p, p, p, None, p, p, 4, 0, 1, 1.0, 2, None) == -1
     assert lib.fma_grouped_gemm(p, p, p, p, p, p, 0, 0, 1, 1.0, 2, None) == 0
@@ -93,6 +94,39 @@ def test_swiglu_and_gemm_validation(lib):
     assert lib.fma_grouped_gemm_swiglu(p, p, p, p, p, 4, 16, 60, 2, None) == -3  # K % 8 != 0
     assert lib.fma_grouped_gemm_swiglu(p, p, p, p, p, 4, 1 << 22, 64, 2, None) == -3  # beyond the 32-bit tile offsets
     assert lib.fma_grouped_gemm_swiglu(p, p, p, p, p, 4, 16, 1 << 21, 2, None) == -3
+
+
+def test_router_norm_and_bias_validation(lib):
+    buf = ctypes.create_string_buffer(4096 + 16)
+    p = (ctypes.addressof(buf) + 15) & ~15
+    # router: T, H, E, top_k
+    assert lib.fma_router_topk(p, p, 4, 64, 8, 9, p, p, p, None, 2, None) == -3 and "top_k" in _err(lib)
+    assert lib.fma_router_topk(p, p, 4, 64, 8, 65, p, p, p, None, 2, None) == -3
+    assert lib.fma_router_topk(p, p, 4, 60, 8, 2, p, p, p, None, 2, None) == -3 and "multiple of 8" in _err(lib)
+    assert lib.fma_router_topk(p, p, 4, 64, 1025, 2, p, p, p, None, 2, None) == -4
+    assert lib.fma_router_topk(p, p, 4, 64, 8, 2, p, p, p, None, 0, None) == -2  # 16-bit dtypes only
+    assert lib.fma_router_topk(p, p, 4, 64, 8, 2, None, p, p, None, 2, None) == -1
+    assert lib.fma_router_topk(p + 2, p, 4, 64, 8, 2, p, p, p, None, 2, None) == -6
+    assert lib.fma_router_topk(p, p, 0, 64, 8, 2, p, p, p, None, 2, None) == 0
+    assert lib.fma_router_topk_bwd(p, p, None, None, 4, 8, 9, p, 2, None) == -3
+    assert lib.fma_router_topk_bwd(p, None, None, None, 4, 8, 2, p, 2, None) == -1
+    # residual add + RMSNorm: B, H
+    assert lib.fma_fused_residual_add_rmsnorm_fwd(p, p, None, p, p, None, 4, 0, 1e-5, 1.0, 0, None) == -3
+    assert lib.fma_fused_residual_add_rmsnorm_fwd(p, p, None, p, p, None, 4, 65537, 1e-5, 1.0, 0, None) == -3
+    assert lib.fma_fused_residual_add_rmsnorm_fwd(p, p, None, p, p, None, 4, 64, 1e-5, 1.0, 3, None) == -2
+    assert lib.fma_fused_residual_add_rmsnorm_fwd(p, None, None, p, p, None, 4, 64, 1e-5, 1.0, 0, None) == -1
+    assert lib.fma_fused_residual_add_rmsnorm_fwd(p, p, None, p, p, None, 0, 64, 1e-5, 1.0, 0, None) == 0
+    assert lib.fma_fused_residual_add_rmsnorm_bwd_workspace_bytes(16384, 4096) % (4096 * 4) == 0
+    assert lib.fma_fused_residual_add_rmsnorm_bwd_workspace_bytes(0, 4096) == 0
+    # weight without weight_grad
+    assert lib.fma_fused_residual_add_rmsnorm_bwd(p, p, p, None, None, p, p, None, 4, 64, 1e-5, 1.0, p, 4096, 0, None) == -1
+    # expert bias: E, R, N
+    assert lib.fma_expert_bias_add(p, p, p, 2, 4, 12, 2, None) == -3 and "16 bytes" in _err(lib)
+    assert lib.fma_expert_bias_add(p, p, p, 1025, 4, 16, 2, None) == -4
+    assert lib.fma_expert_bias_add(p, None, p, 2, 4, 16, 2, None) == -1
+    assert lib.fma_expert_bias_add(p, p, p, 2, 0, 16, 2, None) == 0
+    assert lib.fma_expert_bias_grad_workspace_bytes(8, 32768, 4096) == (32768 // 256 + 8) * 4096 * 4
+    assert lib.fma_expert_bias_grad(p, p, 2, 1000, 16, p, p, 8, 2, None) == -7 and "workspace" in _err(lib)
 
 
 def test_check_raises_runtime_error(lib):
