@@ -176,10 +176,10 @@ __device__ __forceinline__ void topk_softmax_tokens(uint32_t* const (&keys)[NR],
     }
 }
 
-__device__ __forceinline__ void flush_histogram(const RouterArgs& a, const uint32_t* s_hist, int tid) {
+__device__ __forceinline__ void flush_histogram(const RouterArgs& a, const uint32_t* s_hist, int tid, int nthreads) {
     if (!a.counts) return;
     __syncthreads();
-    for (int n = tid; n < a.E; n += kRouterThreads) {
+    for (int n = tid; n < a.E; n += nthreads) {
         const uint32_t h = s_hist[n];
         if (h) atomicAdd(a.counts + n, h);
     }
@@ -323,7 +323,7 @@ __global__ __launch_bounds__(kRouterThreads) void router_topk_kernel(const Route
         }
         topk_softmax_tokens<EL, RB>(rows, tid & 15, tokens, a, s_hist);
     }
-    flush_histogram(a, s_hist, tid);
+    flush_histogram(a, s_hist, tid, kRouterThreads);
 }
 
 // ---- the same for more than 16 experts -------------------------------------------------------------------------------
@@ -337,10 +337,13 @@ constexpr int kRing = 4;                        // operands are requested kRing 
                                                 // LDS tile index step % 2 is taken from the ring index)
 constexpr int kTileRowBytes = kStepK * 2 + 16;  // 16 bytes of padding: consecutive expert rows start 4 banks apart
 
-template <typename EL, int NBLK, int EMAX>
-__global__ __launch_bounds__(kRouterThreads) void router_topk_wide_kernel(const RouterArgs a) {
+// W: wavefronts (of 16 tokens each) per workgroup: 4, or 2 when the token count would otherwise leave compute units idle
+template <typename EL, int NBLK, int EMAX, int W>
+__global__ __launch_bounds__(W * kWave) void router_topk_wide_kernel(const RouterArgs a) {
     using frag = typename EL::frag;
-    constexpr int kCols = NBLK * 16, kToks = kRouterWaves * kTok;
+    constexpr int kThreadsW = W * kWave;
+    constexpr int kUnits = NBLK * 256 / kThreadsW;  // 16-byte units of a weight tile per thread
+    constexpr int kCols = NBLK * 16, kToks = W * kTok;
     __shared__ __attribute__((aligned(16))) uint8_t s_tile[2][kCols * kTileRowBytes];
     __shared__ uint32_t s_key[kToks][EMAX + kRowPad];
     __shared__ uint32_t s_hist[EMAX];
@@ -351,7 +354,7 @@ __global__ __launch_bounds__(kRouterThreads) void router_topk_wide_kernel(const 
     const int64_t tok0 = (int64_t)blockIdx.x * kToks;
 
     if (a.counts)
-        for (int n = tid; n < E; n += kRouterThreads) s_hist[n] = 0;
+        for (int n = tid; n < E; n += kThreadsW) s_hist[n] = 0;
 
     const int64_t t_mine = tok0 + wave * kTok + r;
     const uint16_t* xa = a.x + (t_mine < a.T ? t_mine : a.T - 1) * H + q * 32;  // past the end: the last token again
@@ -363,28 +366,28 @@ __global__ __launch_bounds__(kRouterThreads) void router_topk_wide_kernel(const 
     // The unchecked forms are for whole steps of the pipelined loop (nothing may consume a loaded register right after
     // the load there, or the wavefront waits for it on the spot); the checked forms zero what lies past the end of the
     // row (H is a multiple of 8: a 16-byte unit is inside the row or outside).
-    auto fetch_tile = [&](u32x4 (&regs)[NBLK], int col0, int step) {
+    auto fetch_tile = [&](u32x4 (&regs)[kUnits], int col0, int step) {
 #pragma unroll
-        for (int i = 0; i < NBLK; ++i) {
-            const int u = tid + i * kRouterThreads;
+        for (int i = 0; i < kUnits; ++i) {
+            const int u = tid + i * kThreadsW;
             const int n = col0 + (u >> 4);
             regs[i] = *reinterpret_cast<const u32x4*>(a.w + (int64_t)(n < E ? n : E - 1) * H + step * kStepK + (u & 15) * 8);
         }
     };
-    auto fetch_tile_checked = [&](u32x4 (&regs)[NBLK], int col0, int step) {
+    auto fetch_tile_checked = [&](u32x4 (&regs)[kUnits], int col0, int step) {
 #pragma unroll
-        for (int i = 0; i < NBLK; ++i) {
-            const int u = tid + i * kRouterThreads;
+        for (int i = 0; i < kUnits; ++i) {
+            const int u = tid + i * kThreadsW;
             const int n = col0 + (u >> 4), kk = step * kStepK + (u & 15) * 8;
             const bool in = kk < H;
             regs[i] = *reinterpret_cast<const u32x4*>(a.w + (int64_t)(n < E ? n : E - 1) * H + (in ? kk : 0));
             if (!in) regs[i] = u32x4{0u, 0u, 0u, 0u};
         }
     };
-    auto store_tile = [&](const u32x4 (&regs)[NBLK], int buf) {
+    auto store_tile = [&](const u32x4 (&regs)[kUnits], int buf) {
 #pragma unroll
-        for (int i = 0; i < NBLK; ++i) {
-            const int u = tid + i * kRouterThreads;
+        for (int i = 0; i < kUnits; ++i) {
+            const int u = tid + i * kThreadsW;
             *reinterpret_cast<u32x4*>(&s_tile[buf][(u >> 4) * kTileRowBytes + (u & 15) * 16]) = regs[i];
         }
     };
@@ -430,7 +433,7 @@ __global__ __launch_bounds__(kRouterThreads) void router_topk_wide_kernel(const 
             // wavefront per SIMD is the usual occupancy here (a wavefront per 16 tokens), so the latency of the L2 and
             // of HBM is covered by this distance, not by other wavefronts.
             frag xq[kRing][4];
-            u32x4 staged[kRing][NBLK];
+            u32x4 staged[kRing][kUnits];
 #pragma unroll
             for (int d = 0; d < kRing - 1; ++d) {
                 fetch_tile(staged[d], col0, d);
@@ -451,7 +454,7 @@ __global__ __launch_bounds__(kRouterThreads) void router_topk_wide_kernel(const 
             }
         }
         for (int step = npipe; step < nsteps; ++step) {
-            u32x4 staged[NBLK];
+            u32x4 staged[kUnits];
             frag xf[4];
             fetch_tile_checked(staged, col0, step);
             fetch_x_checked(xf, step);
@@ -480,23 +483,31 @@ __global__ __launch_bounds__(kRouterThreads) void router_topk_wide_kernel(const 
 
     // ---- top-k and softmax over the kept logits ----------------------------------------------------------------------
     {
-        uint32_t* rows[kRouterWaves];
-        int64_t tokens[kRouterWaves];
+        // 16 lanes per token: W * 4 tokens at a time, four rounds
+        uint32_t* rows[4];
+        int64_t tokens[4];
 #pragma unroll
-        for (int round = 0; round < kRouterWaves; ++round) {
-            rows[round] = s_key[round * kTok + (tid >> 4)];
-            tokens[round] = tok0 + round * kTok + (tid >> 4);
+        for (int round = 0; round < 4; ++round) {
+            rows[round] = s_key[round * (W * 4) + (tid >> 4)];
+            tokens[round] = tok0 + round * (W * 4) + (tid >> 4);
         }
-        topk_softmax_tokens<EL, kRouterWaves>(rows, tid & 15, tokens, a, s_hist);
+        topk_softmax_tokens<EL, 4>(rows, tid & 15, tokens, a, s_hist);
     }
-    flush_histogram(a, s_hist, tid);
+    flush_histogram(a, s_hist, tid, kThreadsW);
 }
 
 template <typename EL, int NBLK, int EMAX>
 int launch_router_wide(const RouterArgs& a, hipStream_t st) {
-    const int64_t toks = (int64_t)kRouterWaves * kTok;
-    const uint32_t blocks = (uint32_t)((a.T + toks - 1) / toks);
-    hipLaunchKernelGGL((router_topk_wide_kernel<EL, NBLK, EMAX>), dim3(blocks), dim3(kRouterThreads), 0, st, a);
+    // 64 tokens per workgroup share each weight tile four ways; with too few tokens to give every compute unit such a
+    // workgroup, 32 tokens per workgroup keep twice as many units busy
+    const int64_t cus = num_compute_units() > 0 ? num_compute_units() : 256;
+    if ((a.T + 63) / 64 >= cus) {
+        const uint32_t blocks = (uint32_t)((a.T + 63) / 64);
+        hipLaunchKernelGGL((router_topk_wide_kernel<EL, NBLK, EMAX, 4>), dim3(blocks), dim3(256), 0, st, a);
+    } else {
+        const uint32_t blocks = (uint32_t)((a.T + 31) / 32);
+        hipLaunchKernelGGL((router_topk_wide_kernel<EL, NBLK, EMAX, 2>), dim3(blocks), dim3(128), 0, st, a);
+    }
     return launch_status("router_topk");
 }
 
