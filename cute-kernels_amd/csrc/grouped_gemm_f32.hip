@@ -2,9 +2,12 @@
 // 157 TFLOP/s peak: one sixteenth of the bf16 rate, so this kernel is bound by the matrix pipe long before memory and is
 // kept simple). 128 x 128 output tiles, 16-wide K steps, four wavefronts of 64 x 64 each. Operands are fetched element
 // by element with bounds checks (any M, N, K and either storage order; rows past a group's edge and K past its end read as
-// zero), staged in LDS reduction-major ([k][row], rows padded to 160 floats so the two half-wavefronts of a fragment read
-// hit different banks), double-buffered with one barrier per K step. Workgroups are persistent and find their tiles in a
-// per-workgroup prefix table of the groups' tile counts, like the 16-bit kernel.
+// zero) two K steps ahead into registers, staged in LDS as [row][16 k] with rows padded to 20 floats, double-buffered
+// with one barrier per K step. The instruction multiplies two k values at a time (lane half h supplies one of them);
+// since the order of a sum's terms is free, half h takes k = 8 h .. 8 h + 7 of the step, so a lane's eight values of a
+// fragment are contiguous in LDS and come with two 16-byte reads (the padded rows make those conflict-free).
+// Workgroups are persistent and find their tiles in a per-workgroup prefix table of the groups' tile counts, like the
+// 16-bit kernel.
 #include "common.h"
 #include "grouped_gemm_f32.h"
 
@@ -16,7 +19,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 constexpr int BM = 128, BN = 128, BK = 16;
 constexpr int kThreads = 256;
-constexpr int kPitch = 160;                          // floats per LDS row: 128 + 32 of padding
+constexpr int kPitch = 20;                           // floats per LDS row: 16 k + 4 of padding
 constexpr int kPerThread = BM * BK / kThreads;       // operand elements per thread and K step (8)
 static_assert(BM == BN, "one staging routine serves both operands");
 
@@ -45,6 +48,9 @@ __device__ __forceinline__ void element_of(int i, int tid, int& row, int& k) {
     }
 }
 
+// Requests the thread's elements of the operand tile at (row0, k0). Elements outside the operand are requested from
+// its first element instead (a valid address: a tile exists only if M, N >= 1, a K step only if K >= 1) and replaced by
+// zeros in stage(): nothing here consumes a loaded value, so the loads stay in flight until the data is needed.
 template <bool K_CONTIG>
 __device__ __forceinline__ void fetch(float (&regs)[kPerThread], const float* __restrict__ base, uint32_t rows,
                                       uint32_t K, uint32_t row0, uint32_t k0, int tid) {
@@ -55,24 +61,26 @@ __device__ __forceinline__ void fetch(float (&regs)[kPerThread], const float* __
         const uint32_t row = row0 + r, kk = k0 + k;
         const bool in = row < rows && kk < K;
         const uint64_t idx = K_CONTIG ? (uint64_t)row * K + kk : (uint64_t)kk * rows + row;
-        regs[i] = in ? base[in ? idx : 0] : 0.0f;
+        regs[i] = base[in ? idx : 0];
     }
 }
 
 template <bool K_CONTIG>
-__device__ __forceinline__ void stage(const float (&regs)[kPerThread], float* __restrict__ tile, int tid) {
+__device__ __forceinline__ void stage(const float (&regs)[kPerThread], float* __restrict__ tile, uint32_t rows,
+                                      uint32_t K, uint32_t row0, uint32_t k0, int tid) {
 #pragma unroll
     for (int i = 0; i < kPerThread; ++i) {
         int r, k;
         element_of<K_CONTIG>(i, tid, r, k);
-        tile[k * kPitch + r] = regs[i];
+        const bool in = row0 + r < rows && k0 + k < K;
+        tile[r * kPitch + k] = in ? regs[i] : 0.0f;
     }
 }
 
 template <bool A_KC, bool B_KC>
 __global__ __launch_bounds__(kThreads) void grouped_gemm_f32_kernel(const Args args) {
-    __shared__ float s_a[2][BK * kPitch];
-    __shared__ float s_b[2][BK * kPitch];
+    __shared__ __attribute__((aligned(16))) float s_a[2][BM * kPitch];
+    __shared__ __attribute__((aligned(16))) float s_b[2][BN * kPitch];
     __shared__ uint32_t s_tile_start[FMA_MAX_GROUPS + 1];
     __shared__ uint64_t s_off_a[FMA_MAX_GROUPS], s_off_b[FMA_MAX_GROUPS], s_off_d[FMA_MAX_GROUPS];
 
@@ -125,44 +133,55 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_f32_kernel(const Args a
                 for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.0f;
 
         const uint32_t KT = (Ke + BK - 1) / BK;
-        float ra[kPerThread], rb[kPerThread];
-        if (KT > 0) {
-            fetch<A_KC>(ra, Ae, Me, Ke, m0, 0, tid);
-            fetch<B_KC>(rb, Be, Ne, Ke, n0, 0, tid);
-            __syncthreads();  // the previous tile is done with the LDS stages
-            stage<A_KC>(ra, s_a[0], tid);
-            stage<B_KC>(rb, s_b[0], tid);
-            __syncthreads();
-        }
-        for (uint32_t kt = 0; kt < KT; ++kt) {
-            const int buf = kt & 1;
-            if (kt + 1 < KT) {
-                fetch<A_KC>(ra, Ae, Me, Ke, m0, (kt + 1) * BK, tid);
-                fetch<B_KC>(rb, Be, Ne, Ke, n0, (kt + 1) * BK, tid);
-            }
-            // a fragment of the 32x32x2 instruction: lane l holds row (l % 32) of the operand at k = l / 32
-            const float* ta = s_a[buf] + (lane >> 5) * kPitch + wm * 64 + (lane & 31);
-            const float* tb = s_b[buf] + (lane >> 5) * kPitch + wn * 64 + (lane & 31);
+        // two register sets: set s holds the operands of the steps with kt % 2 == s, fetched two steps before their use
+        float ra[2][kPerThread], rb[2][kPerThread];
+        auto compute = [&](int buf) {
+            // lane l: row (l % 32) of a 32-row block, k values 8 (l / 32) .. + 7 of the step
+            const float* ta = s_a[buf] + (wm * 64 + (lane & 31)) * kPitch + (lane >> 5) * 8;
+            const float* tb = s_b[buf] + (wn * 64 + (lane & 31)) * kPitch + (lane >> 5) * 8;
+            float4 fa[2][2], fb[2][2];
 #pragma unroll
-            for (int kk = 0; kk < BK; kk += 2) {
-                float fa[2], fb[2];
+            for (int i = 0; i < 2; ++i)
 #pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    fa[i] = ta[kk * kPitch + i * 32];
-                    fb[i] = tb[kk * kPitch + i * 32];
+                for (int hh = 0; hh < 2; ++hh) {
+                    fa[i][hh] = *reinterpret_cast<const float4*>(ta + i * 32 * kPitch + hh * 4);
+                    fb[i][hh] = *reinterpret_cast<const float4*>(tb + i * 32 * kPitch + hh * 4);
                 }
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
                 // B first: a lane then owns one output row and four consecutive output columns per register quad
 #pragma unroll
                 for (int i = 0; i < 2; ++i)
 #pragma unroll
-                    for (int j = 0; j < 2; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j], fa[i], acc[i][j], 0, 0, 0);
+                    for (int j = 0; j < 2; ++j) {
+                        const float av = reinterpret_cast<const float*>(&fa[i][kk >> 2])[kk & 3];
+                        const float bv = reinterpret_cast<const float*>(&fb[j][kk >> 2])[kk & 3];
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv, av, acc[i][j], 0, 0, 0);
+                    }
             }
-            if (kt + 1 < KT) {
-                stage<A_KC>(ra, s_a[buf ^ 1], tid);
-                stage<B_KC>(rb, s_b[buf ^ 1], tid);
+        };
+        if (KT > 0) {
+            fetch<A_KC>(ra[0], Ae, Me, Ke, m0, 0, tid);
+            fetch<B_KC>(rb[0], Be, Ne, Ke, n0, 0, tid);
+            fetch<A_KC>(ra[1], Ae, Me, Ke, m0, BK, tid);  // past the end of K: zeros
+            fetch<B_KC>(rb[1], Be, Ne, Ke, n0, BK, tid);
+            __syncthreads();  // the previous tile is done with the LDS stages
+            stage<A_KC>(ra[0], s_a[0], Me, Ke, m0, 0, tid);
+            stage<B_KC>(rb[0], s_b[0], Ne, Ke, n0, 0, tid);
+            __syncthreads();
+        }
+        for (uint32_t kt = 0; kt < KT; kt += 2) {
+#pragma unroll
+            for (int ph = 0; ph < 2; ++ph) {
+                // step kt + ph (a step past the last one multiplies zeros): request step + 2 into the set this step's
+                // operands came from, multiply from stage ph, move step + 1 from its registers to the other stage
+                fetch<A_KC>(ra[ph], Ae, Me, Ke, m0, (kt + ph + 2) * BK, tid);
+                fetch<B_KC>(rb[ph], Be, Ne, Ke, n0, (kt + ph + 2) * BK, tid);
+                compute(ph);
+                stage<A_KC>(ra[ph ^ 1], s_a[ph ^ 1], Me, Ke, m0, (kt + ph + 1) * BK, tid);
+                stage<B_KC>(rb[ph ^ 1], s_b[ph ^ 1], Ne, Ke, n0, (kt + ph + 1) * BK, tid);
+                __syncthreads();  // stage ph^1 is complete; stage ph may be overwritten in the next step
             }
-            __syncthreads();  // stage buf^1 is complete; stage buf may be overwritten in the next step
         }
 
         // accumulator register 4 q + j of block (i, j'): row m = ... + (lane % 32), column n = ... + 8 q + 4 (lane / 32) + j
