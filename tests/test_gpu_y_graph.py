@@ -51,3 +51,38 @@ def test_expert_path_replays_from_a_captured_graph():
             graph.replay()
             torch.cuda.synchronize()
             assert torch.equal(y_static, expect), f"replay with batch {seed} differs from the eager result"
+
+
+def test_whole_layer_with_the_fused_router_replays_from_a_captured_graph():
+    # the same with the router inside the captured region: gate product, top-k and softmax are one kernel that clears
+    # nothing (the optional histogram, which a fill kernel would clear, is not requested by the module)
+    torch.manual_seed(8)
+    T, H, I, E, k = 200, 512, 256, 64, 8
+    moe = MoE(E, k, H, I, swiglu_packed, True, False, 0.02).to(torch.bfloat16).to(DEV)
+    assert moe._router_is_fusable(torch.zeros(1, H, dtype=torch.bfloat16, device=DEV))
+    x_static = torch.zeros(T, H, dtype=torch.bfloat16, device=DEV)
+
+    def draw(seed):
+        return torch.randn(T, H, generator=torch.Generator().manual_seed(seed)).bfloat16().to(DEV)
+
+    with torch.no_grad():
+        x_static.copy_(draw(0))
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                moe(x_static, kernel_backend=KernelBackend.cuda)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y_static, logits_static = moe(x_static, kernel_backend=KernelBackend.cuda)
+
+        for seed in (1, 2, 3, 4):
+            x = draw(seed)
+            expect, expect_logits = moe(x, kernel_backend=KernelBackend.cuda)  # eager, between the replays
+            torch.cuda.synchronize()
+            x_static.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(logits_static, expect_logits), f"router logits of replay {seed} differ"
+            assert torch.equal(y_static, expect), f"replay with batch {seed} differs from the eager result"
