@@ -107,3 +107,40 @@ def test_package_has_no_oracle_dependency():
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.replace("moe_oracle", "oracle") or "import oracle" not in text
                 assert "from oracle" not in text and "import oracle" not in text
+
+
+def test_fused_residual_add_rmsnorm_signature_and_errors():
+    from fma import fused_residual_add_rmsnorm
+
+    sig = inspect.signature(fused_residual_add_rmsnorm)
+    assert list(sig.parameters) == ["x", "residual", "weight", "eps", "multiplier", "memory_efficient", "kernel_backend"]
+    assert sig.parameters["multiplier"].default is None and sig.parameters["memory_efficient"].default is False
+    assert sig.parameters["kernel_backend"].default is KernelBackend.triton
+    x = torch.randn(4, 8)
+    with pytest.raises(ValueError):
+        fused_residual_add_rmsnorm(x, x, None, 1e-5, kernel_backend=KernelBackend.torch)
+    with pytest.raises(RuntimeError, match="GPU only"):  # no eager implementation to fall back to
+        fused_residual_add_rmsnorm(x, x, None, 1e-5)
+    with pytest.raises(AssertionError, match="weight should be 1D"):
+        fused_residual_add_rmsnorm(x, x, torch.randn(2, 8), 1e-5)
+    with pytest.raises(AssertionError, match="hidden size"):
+        fused_residual_add_rmsnorm(x, x, torch.randn(4), 1e-5)
+
+
+def test_router_and_bias_host_logic():
+    moe = MoE(8, 2, 64, 128, swiglu_packed, True, False, 0.02)
+    assert moe.fuse_router and moe.fuse_swiglu and moe.c_fc.bias is None
+    # the fused router serves 16-bit activations on the GPU only: everything else takes the reference's ATen formulation
+    assert not moe._router_is_fusable(torch.randn(4, 64))
+    assert not moe._router_is_fusable(torch.randn(4, 64).bfloat16())  # a CPU tensor
+    logits, weights, selected = moe._compute_routing_weights(torch.randn(5, 64))
+    assert logits.shape == (5, 8) and weights.shape == selected.shape == (5, 2) and selected.dtype == torch.int64
+    assert torch.allclose(weights.sum(-1), torch.ones(5), atol=1e-6)
+    assert bool((logits.gather(1, selected)[:, 0] >= logits.gather(1, selected)[:, 1]).all())
+    # a layer with biases keeps them as parameters of the reference's shapes and runs the up-projection unfused
+    biased = MoE(8, 2, 64, 128, swiglu_packed, True, True, 0.02)
+    assert biased.c_fc.bias.shape == (8, 256) and biased.c_proj.bias.shape == (8, 64) and not biased.fuse_swiglu
+    assert float(biased.c_fc.bias.abs().max()) == 0.0  # reset_parameters zeroes them (fma/modules/moe/__init__.py:121-122)
+    top1 = MoE(4, 1, 64, 128, swiglu_packed, True, False, 0.02)
+    _, w1, s1 = top1._compute_routing_weights(torch.randn(5, 64))
+    assert torch.equal(w1, torch.ones(5, 1)) and s1.shape == (5, 1)
