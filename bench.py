@@ -266,17 +266,39 @@ def main():
             hbm("hbm_copy_1GiB", 2 * src.numel() * s, lambda i: dst.copy_(src), n=10)
             del src, dst
 
-        # row kernels: algorithmic bytes = each distinct input row once + each output row once + index / gate words
-        hbm("gather_rows", T * H * s + R * H * s + R * 4,
-            lambda i: ok(lib.fma_gather_rows(x.data_ptr(), perm.data_ptr(), R, H, k, xg.data_ptr(), BF16, stream)))
-        hbm("dispatch_rows", T * H * s + R * H * s + R * 4,
-            lambda i: ok(lib.fma_dispatch_rows(x.data_ptr(), inv.data_ptr(), T, k, H, xg.data_ptr(), BF16, stream)))
-        hbm("combine", R * H * s + R * (4 + s) + T * H * s,
-            lambda i: ok(lib.fma_combine(o.data_ptr(), inv.data_ptr(), weights_d.data_ptr(), T, k, H, y.data_ptr(), BF16,
-                                         stream)))
-        hbm("combine_backward", T * H * s + 2 * R * H * s + R * (4 + 2 * s),
-            lambda i: ok(lib.fma_combine_bwd(dy.data_ptr(), o.data_ptr(), inv.data_ptr(), weights_d.data_ptr(), T, k, H,
-                                             d_o.data_ptr(), dgates.data_ptr(), BF16, stream)))
+        # Row kernels: algorithmic bytes = each distinct input row once + each output row once + index / gate words.
+        # Inputs and outputs rotate over several buffer sets whose footprint together exceeds 1 GiB (four times the
+        # 256 MiB last-level cache), so that a launch finds neither its inputs nor the lines it writes in that cache.
+        def copies(t, set_bytes):
+            n = max(2, -(-(1 << 30) // set_bytes))
+            return [t] + [t.clone() for _ in range(n - 1)]
+
+        gather_b = T * H * s + R * H * s + R * 4
+        combine_b = R * H * s + R * (4 + s) + T * H * s
+        combine_bwd_b = T * H * s + 2 * R * H * s + R * (4 + 2 * s)
+        if want("gather_rows") or want("dispatch_rows"):
+            xs_r, xg_r = copies(x, gather_b), copies(xg, gather_b)
+            nr = len(xs_r)
+            hbm("gather_rows", gather_b,
+                lambda i: ok(lib.fma_gather_rows(xs_r[i % nr].data_ptr(), perm.data_ptr(), R, H, k, xg_r[i % nr].data_ptr(),
+                                                 BF16, stream)))
+            hbm("dispatch_rows", gather_b,
+                lambda i: ok(lib.fma_dispatch_rows(xs_r[i % nr].data_ptr(), inv.data_ptr(), T, k, H,
+                                                   xg_r[i % nr].data_ptr(), BF16, stream)))
+            del xs_r, xg_r
+        if want("combine"):
+            o_r, y_r = copies(o, combine_b), copies(y, combine_b)
+            nc = len(o_r)
+            hbm("combine", combine_b,
+                lambda i: ok(lib.fma_combine(o_r[i % nc].data_ptr(), inv.data_ptr(), weights_d.data_ptr(), T, k, H,
+                                             y_r[i % nc].data_ptr(), BF16, stream)))
+            dy_r, do_r = copies(dy, combine_bwd_b), copies(d_o, combine_bwd_b)
+            nb = len(dy_r)
+            hbm("combine_backward", combine_bwd_b,
+                lambda i: ok(lib.fma_combine_bwd(dy_r[i % nb].data_ptr(), o_r[i % nc].data_ptr(), inv.data_ptr(),
+                                                 weights_d.data_ptr(), T, k, H, do_r[i % nb].data_ptr(), dgates.data_ptr(),
+                                                 BF16, stream)))
+            del o_r, y_r, dy_r, do_r
         es = 2 * I  # row stride of the packed pre-activation and of its gradient
         hbm("swiglu_forward", 3 * R * I * s,
             lambda i: ok(lib.fma_swiglu_forward(h.data_ptr() + I * s, h.data_ptr(), a.data_ptr(), R, I, es, es, I, BF16,
@@ -319,24 +341,31 @@ def main():
         # normalised activations and the new residual; backward reads the saved residual and both incoming gradients and
         # writes the two input gradients (plus the per-workgroup partial weight gradients and their sum)
         if want("rmsnorm"):
-            res_in = torch.randn(T, H, device=dev).bfloat16()
+            fwd_b, bwd_b = 4 * T * H * s + H * s + T * 4, 5 * T * H * s + H * (s + 4) + T * 4
             nw = (1 + 0.1 * torch.randn(H, device=dev)).bfloat16()
-            n_out, n_added = torch.empty(T, H, **bf), torch.empty(T, H, **bf)
+            nn_ = max(2, -(-(1 << 30) // fwd_b))  # buffer sets, rotated like the row kernels' above
+            x_n = [x] + [x.clone() for _ in range(nn_ - 1)]
+            res_in = [torch.randn(T, H, device=dev).bfloat16() for _ in range(nn_)]
+            n_out = [torch.empty(T, H, **bf) for _ in range(nn_)]
+            n_added = [torch.empty(T, H, **bf) for _ in range(nn_)]
             n_inv = torch.empty(T, dtype=torch.float32, device=dev)
-            hbm("fused_residual_add_rmsnorm_fwd", 4 * T * H * s + H * s + T * 4,
-                lambda i: ok(lib.fma_fused_residual_add_rmsnorm_fwd(x.data_ptr(), res_in.data_ptr(), nw.data_ptr(),
-                                                                    n_out.data_ptr(), n_added.data_ptr(), n_inv.data_ptr(),
-                                                                    T, H, 1e-5, 1.0, BF16, stream)))
+            hbm("fused_residual_add_rmsnorm_fwd", fwd_b,
+                lambda i: ok(lib.fma_fused_residual_add_rmsnorm_fwd(x_n[i % nn_].data_ptr(), res_in[i % nn_].data_ptr(),
+                                                                    nw.data_ptr(), n_out[i % nn_].data_ptr(),
+                                                                    n_added[i % nn_].data_ptr(), n_inv.data_ptr(), T, H,
+                                                                    1e-5, 1.0, BF16, stream)))
             ws_n = torch.empty(max(lib.fma_fused_residual_add_rmsnorm_bwd_workspace_bytes(T, H), 4), dtype=torch.uint8,
                                device=dev)
-            n_dx, n_dres = torch.empty(T, H, **bf), torch.empty(T, H, **bf)
             n_dw = torch.empty(H, dtype=torch.float32, device=dev)
-            hbm("fused_residual_add_rmsnorm_bwd(2 launches)", 5 * T * H * s + H * (s + 4) + T * 4,
-                lambda i: ok(lib.fma_fused_residual_add_rmsnorm_bwd(n_added.data_ptr(), nw.data_ptr(), dy.data_ptr(),
-                                                                    d_o.data_ptr(), n_inv.data_ptr(), n_dx.data_ptr(),
-                                                                    n_dres.data_ptr(), n_dw.data_ptr(), T, H, 1e-5, 1.0,
-                                                                    ws_n.data_ptr(), ws_n.numel(), BF16, stream)))
-            del res_in, n_out, n_added, n_dx, n_dres, ws_n
+            # the forward's buffers serve as the backward's: saved residual, two incoming gradients, two outputs
+            hbm("fused_residual_add_rmsnorm_bwd(2 launches)", bwd_b,
+                lambda i: ok(lib.fma_fused_residual_add_rmsnorm_bwd(n_added[i % nn_].data_ptr(), nw.data_ptr(),
+                                                                    x_n[i % nn_].data_ptr(), res_in[i % nn_].data_ptr(),
+                                                                    n_inv.data_ptr(), n_out[(i + 1) % nn_].data_ptr(),
+                                                                    n_added[(i + 1) % nn_].data_ptr(), n_dw.data_ptr(), T,
+                                                                    H, 1e-5, 1.0, ws_n.data_ptr(), ws_n.numel(), BF16,
+                                                                    stream)))
+            del x_n, res_in, n_out, n_added, ws_n
         # per-expert bias on the up-projection's output [R, 2I] (layers built with add_bias=True)
         if want("expert_bias"):
             b1 = torch.randn(E, 2 * I, device=dev).bfloat16()
