@@ -142,6 +142,25 @@ def main():
     tokens_per_s = T * args.steps / elapsed
     gemm_flops_step = 3 * 2.0 * R * (2 * I * H + I * H)  # fwd + dgrad + wgrad of both projections
 
+    # the same step with the router inside (gate product, top-k, softmax by the fused kernel, and their backward): the
+    # expert choice then comes from the randomly initialised gate (close to uniform), not from the workload's routing
+    def step_with_router():
+        moe.zero_grad(set_to_none=True)
+        xs = x.detach().requires_grad_()
+        y, _ = moe(xs, kernel_backend=KernelBackend.cuda)
+        y.backward(dy)
+
+    ms_with_router = None
+    if args.steps:
+        for _ in range(max(1, args.warmup)):
+            step_with_router()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            step_with_router()
+        torch.cuda.synchronize()
+        ms_with_router = (time.perf_counter() - t1) * 1e3 / args.steps
+
     result = {
         "metric": "MoE layer fwd+bwd tokens/s",
         "value": tokens_per_s,
@@ -158,8 +177,10 @@ def main():
         "config": {
             "workload": f"{args.workload}: MoE layer fwd+bwd, T={T} tokens, hidden={H}, SwiGLU intermediate={I}, "
             f"E={E}, top-k={k}, {c['kind']} routing" + (f", {c['empty']} experts empty" if c["empty"] else ""),
-            "router": "excluded (routing computed once, outside the timed region)",
+            "router": "excluded (routing computed once, outside the timed region); ms_per_step_with_router includes it",
         },
+        "ms_per_step_with_router": ms_with_router,
+        "tokens_per_s_with_router": None if ms_with_router is None else T / (ms_with_router * 1e-3),
         "layer_gemm_tflops": gemm_flops_step / (ms_per_step * 1e-3) / 1e12,
         "layer_gemm_frac_of_peak": gemm_flops_step / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
     }
