@@ -25,7 +25,11 @@ SHAPES = [
     (7, 2048, 8, 2),
     (16384, 4096, 8, 2),  # the Mixtral-like benchmark layer
     (4099, 2048, 64, 8),  # fine-grained shape, a ragged last workgroup
-    (2050, 4096, 128, 8),  # large-E shape: two passes over the expert columns
+    (32768, 2048, 64, 8),  # the fine-grained benchmark layer at full size
+    (2050, 4096, 128, 8),  # large-E shape with few tokens: 32-token workgroups
+    (8192, 4096, 128, 8),  # the large-E benchmark layer at full size
+    (16400, 1024, 128, 8),  # enough tokens for 64-token workgroups, ragged end
+    (300, 640, 200, 5),  # 128 < E <= 256: two passes over the activations
     (33, 200, 6, 4),  # H not a multiple of the 128-element step
     (100, 8, 3, 1),  # H smaller than one step, top-1
     (64, 512, 24, 3),
