@@ -354,9 +354,11 @@ def main():
             dlg = torch.randn(T, E, device=dev).bfloat16()
             drw = torch.randn(T, k, device=dev).bfloat16()
             dlg_out = torch.empty(T, E, **bf)
-            hbm("router_topk_backward", 3 * T * E * s + T * k * (s + 4),
-                lambda i: ok(lib.fma_router_topk_bwd(lg.data_ptr(), sel32.data_ptr(), drw.data_ptr(), dlg.data_ptr(), T,
-                                                     E, k, dlg_out.data_ptr(), BF16, stream)))
+            # a few MB at most: bound by launch latency, so only the time is reported
+            t = time_gpu(lambda i: ok(lib.fma_router_topk_bwd(lg.data_ptr(), sel32.data_ptr(), drw.data_ptr(),
+                                                              dlg.data_ptr(), T, E, k, dlg_out.data_ptr(), BF16, stream)),
+                         20, blocker=blocker)
+            kernels["router_topk_backward"] = {"ms": t[0], "ms_mean": t[1], "bytes": 3 * T * E * s + T * k * (s + 4)}
             del xs3
         # residual add + RMSNorm on the layer's residual stream [T, H]: forward reads x and the residual and writes the
         # normalised activations and the new residual; backward reads the saved residual and both incoming gradients and
