@@ -10,9 +10,15 @@ from ...constants import LIBRARY_NAME
 
 def _launch(A, B, output, M_array, N_array, K_array, is_A_transposed, is_B_transposed, alpha) -> None:
     lib = _lib.load()
+    if output.numel() == 0:
+        return
+    # An operand without elements (every group has M_e * K_e == 0, resp. K_e * N_e == 0) is never read, but the entry point
+    # rejects NULL: any valid device address stands in for it.
+    a_ptr = A.data_ptr() if A.numel() else output.data_ptr()
+    b_ptr = B.data_ptr() if B.numel() else output.data_ptr()
     with torch.cuda.device(A.device):
         rc = lib.fma_grouped_gemm(
-            A.data_ptr(), B.data_ptr(), output.data_ptr(), M_array.data_ptr(), N_array.data_ptr(), K_array.data_ptr(),
+            a_ptr, b_ptr, output.data_ptr(), M_array.data_ptr(), N_array.data_ptr(), K_array.data_ptr(),
             M_array.numel(), int(is_A_transposed), int(is_B_transposed), float(alpha), _lib.dtype_code(A.dtype),
             _lib.current_stream(A.device),
         )

@@ -210,7 +210,26 @@ def test_maximum_group_count(tA, tB):
     assert float((got.cpu().float() - expect.float()).abs().max()) == 0
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_groups_without_a_reduction_dimension_and_empty_outputs(dtype):
+    # K_e == 0 for every group: both operands are empty tensors, the output is all zeros (found by a wider run of the
+    # seeded random problems below: the wrapper used to hand the empty operand's NULL address to the entry point)
+    M_list, N_list, K_list = [5, 0, 300], [16, 16, 16], [0, 0, 0]
+    empty = torch.empty(0, dtype=dtype, device=DEV)
+    got = grouped_gemm(
+        A=empty, B=empty, C=None, M_array=_u32(M_list), N_array=_u32(N_list), K_array=_u32(K_list),
+        output_shape=(305 * 16,), is_A_transposed=False, is_B_transposed=True,
+    )
+    assert got.shape == (305 * 16,) and float(got.float().abs().max()) == 0.0
+    # no output at all (every group has M_e == 0): nothing to do
+    none = grouped_gemm(
+        A=empty, B=torch.ones(3 * 16 * 8, dtype=dtype, device=DEV), C=None, M_array=_u32([0, 0, 0]),
+        N_array=_u32(N_list), K_array=_u32([8, 8, 8]), output_shape=(0,), is_A_transposed=False, is_B_transposed=True,
+    )
+    assert none.numel() == 0
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3, 4, 5, 103])
 def test_random_problem_shapes(seed):
     # seeded random problems: every layout, group counts 1..40, ragged / empty / one-row groups, reduction lengths from 0
     # to 17 K steps (even and odd step counts, partial last step), sizes off the 8-element grid now and then (scalar
