@@ -108,7 +108,9 @@ def test_router_with_exact_logits_and_many_ties(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("T,E,k", [(7, 8, 2), (1000, 8, 2), (513, 64, 8), (300, 128, 8), (100, 3, 1), (77, 300, 16), (20, 1024, 64)])
+@pytest.mark.parametrize(
+    "T,E,k", [(7, 8, 2), (1000, 8, 2), (513, 64, 8), (300, 128, 8), (100, 3, 1), (77, 300, 16), (20, 1024, 64), (31, 65, 36)]
+)
 @pytest.mark.parametrize("which", ["both", "weights", "logits"])
 def test_router_backward(dtype, T, E, k, which):
     torch.manual_seed(E + k)
@@ -142,10 +144,14 @@ def test_router_backward(dtype, T, E, k, which):
     direct = torch.zeros(T, E, dtype=torch.float64) if dl is None else dl.double()
     assert torch.equal(got[untouched], direct[untouched])
 
-    # and the oracle's autograd in the same dtype (same rounding points; fp32 exp may differ in the last place, which
-    # can move a 16-bit rounding by one unit)
+    # and the oracle's autograd in the same dtype. Same rounding points, but the two fp32 evaluations of
+    # s * (dw - <s, dw>) differ in the last places, which can move the 16-bit rounding of that intermediate by one of ITS
+    # units (larger than a unit of the final sum where the direct term cancels it) and the rounding of the sum by one more.
     auto = O.router_logits_grad(logits, selected, dw, dl).double()
-    assert bool(((got - auto).abs() <= EPS[dtype] * auto.abs() + 1e-7).all())
+    slack = torch.full((T, E), 2e-6, dtype=torch.float64)
+    if dw is not None:
+        slack = slack.scatter_add(1, selected, EPS[dtype] * ds.abs() + 2e-6 * float(dw.abs().max()))
+    assert bool(((got - auto).abs() <= EPS[dtype] * auto.abs() + slack).all())
 
 
 def test_router_autograd_matches_unfused_router():
