@@ -105,9 +105,9 @@ __device__ __forceinline__ float sigmoid_clamped(float x) {
 // The same sigmoid from the hardware's exp2 and reciprocal instructions (about 2 ulp in fp32): used wherever the result
 // is rounded to a 16-bit type, where the difference is far below half an ulp of the output.
 __device__ __forceinline__ float sigmoid_clamped_fast(float x) {
-    x = fmaxf(-88.3762626647949f, x);
-    x = fminf(88.3762626647949f, x);
-    return __frcp_rn(1.0f + __expf(-x));
+    x = __builtin_amdgcn_fmed3f(x, -88.3762626647949f, 88.3762626647949f);  // the clamp as one instruction
+    // v_rcp_f32 (1 ulp); a correctly rounded reciprocal would expand to the ten-instruction division sequence
+    return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
 }
 
 // sigmoid for an op whose output type is T
