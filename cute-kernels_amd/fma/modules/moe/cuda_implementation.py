@@ -138,6 +138,8 @@ def grouped_gemm_swiglu_cuda(
     assert M_array.dtype == torch.uint32 and M_array.numel() == E
     for t in (x, weight, M_array, h, act):
         assert t is None or t.is_contiguous()
+    if act.numel() == 0:
+        return  # no rows routed anywhere (or no output columns): nothing to compute, and empty tensors have no address
     with torch.cuda.device(x.device):
         rc = _lib.load().fma_grouped_gemm_swiglu(
             x.data_ptr(), weight.data_ptr(), _lib.ptr(h), act.data_ptr(), M_array.data_ptr(), E, inter, K,
