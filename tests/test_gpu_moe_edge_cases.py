@@ -1,0 +1,116 @@
+"""The layer as callers hand it things: views that are not contiguous, inputs with a batch dimension, every expert
+selected (top_k == E) or a single expert, parameters that are frozen, and calls under no_grad / inference_mode. The
+reference makes operands contiguous at the autograd boundary (fma/utils/contiguous.py), flattens the leading dimensions
+(fma/modules/moe/__init__.py:167-189) and lets autograd skip what needs no gradient."""
+
+import pytest
+import torch
+
+from fma import KernelBackend, MoE, swiglu_packed
+
+from gpu_util import DEV
+
+pytestmark = pytest.mark.gpu
+
+
+def _step(moe, x):
+    x = x.detach().requires_grad_()
+    moe.zero_grad(set_to_none=True)
+    y, logits = moe(x, kernel_backend=KernelBackend.cuda)
+    (y.float().pow(2).sum() + logits.float().sum()).backward()
+    return y.detach(), logits.detach(), x.grad, {n: p.grad.clone() for n, p in moe.named_parameters() if p.grad is not None}
+
+
+def _assert_same(a, b, what):
+    assert a.shape == b.shape and torch.equal(a, b), f"{what}: max diff {float((a.float() - b.float()).abs().max())}"
+
+
+def test_views_that_are_not_contiguous():
+    # bf16: the router is this library's kernel too, so the whole step has to be bit-identical to the contiguous call
+    torch.manual_seed(1)
+    moe = MoE(8, 2, 64, 128, swiglu_packed, True, False, 0.02).to(DEV).to(torch.bfloat16)
+    for view in (torch.randn(33, 128, device=DEV).bfloat16()[:, ::2], torch.randn(64, 33, device=DEV).bfloat16().t()):
+        assert not view.is_contiguous()
+        ref, got = _step(moe, view.contiguous()), _step(moe, view)
+        for a, b, what in zip(ref[:3], got[:3], ("output", "router logits", "input gradient")):
+            _assert_same(a, b, what)
+        for name in ref[3]:
+            _assert_same(ref[3][name], got[3][name], name)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_input_with_batch_dimensions(dtype):
+    torch.manual_seed(2)
+    moe = MoE(8, 2, 64, 128, swiglu_packed, True, True, 0.02).to(DEV).to(dtype)
+    x = torch.randn(3, 5, 64, device=DEV).to(dtype)
+    ref, got = _step(moe, x.reshape(15, 64)), _step(moe, x)
+    assert got[0].shape == (3, 5, 64) and got[2].shape == (3, 5, 64) and got[1].shape == (15, 8)
+    _assert_same(ref[0], got[0].reshape(15, 64), "output")
+    _assert_same(ref[2], got[2].reshape(15, 64), "input gradient")
+    for name in ref[3]:
+        _assert_same(ref[3][name], got[3][name], name)
+
+
+@pytest.mark.parametrize("dtype,rtol", [(torch.bfloat16, 2e-2), (torch.float32, 1e-5)])
+@pytest.mark.parametrize("E,k", [(4, 4), (8, 1), (1, 1), (16, 16), (17, 17), (64, 64)])
+def test_every_expert_selected_or_only_one(E, k, dtype, rtol):
+    # against the layer's definition (fma/modules/moe/__init__.py:267-286) evaluated token by token in fp64 from the
+    # routing the layer itself chose
+    torch.manual_seed(3)
+    T, H, I = 19, 64, 64
+    moe = MoE(E, k, H, I, swiglu_packed, True, False, 0.02).to(DEV).to(dtype)
+    x = torch.randn(T, H, device=DEV).to(dtype)
+    with torch.no_grad():
+        y, _ = moe(x, kernel_backend=KernelBackend.cuda)
+        _, weights, selected = moe._compute_routing_weights(x)
+    assert sorted(selected[0].tolist()) == list(range(E)) if k == E else selected.shape == (T, k)
+    weights, selected = weights.double().cpu(), selected.long().cpu()
+    xd, W1, W2 = x.double().cpu(), moe.c_fc.weight.detach().double().cpu(), moe.c_proj.weight.detach().double().cpu()
+    expect = torch.zeros(T, H, dtype=torch.float64)
+    for t in range(T):
+        for j in range(k):
+            e = int(selected[t, j])
+            h = W1[e] @ xd[t]
+            up, gate = h[:I], h[I:]
+            expect[t] += weights[t, j] * (W2[e] @ (up * gate * torch.sigmoid(gate)))
+    err = float((y.double().cpu() - expect).abs().max())
+    assert err <= rtol * float(expect.abs().max()), f"max error {err} against scale {float(expect.abs().max())}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_frozen_parameters_and_inference(dtype):
+    torch.manual_seed(4)
+    moe = MoE(8, 2, 64, 128, swiglu_packed, True, True, 0.02).to(DEV).to(dtype)
+    x = torch.randn(21, 64, device=DEV).to(dtype)
+    y_full, _, dx_full, grads_full = _step(moe, x)
+
+    def backward_of(inp):
+        moe.zero_grad(set_to_none=True)
+        y, logits = moe(inp, kernel_backend=KernelBackend.cuda)
+        (y.float().pow(2).sum() + logits.float().sum()).backward()
+
+    # an input that needs no gradient: the parameters get the same gradients
+    backward_of(x)
+    for name, p in moe.named_parameters():
+        _assert_same(grads_full[name], p.grad, f"{name} (input without gradient)")
+    # experts frozen: the input and the gate still get theirs, the experts get none
+    for name, p in moe.named_parameters():
+        p.requires_grad_(name.startswith("gate"))
+    xg = x.clone().requires_grad_()
+    backward_of(xg)
+    _assert_same(dx_full, xg.grad, "input gradient (experts frozen)")
+    _assert_same(grads_full["gate.weight"], moe.gate.weight.grad, "gate gradient (experts frozen)")
+    assert all(p.grad is None for name, p in moe.named_parameters() if not name.startswith("gate"))
+    # gate frozen, input without gradient: only the experts
+    for name, p in moe.named_parameters():
+        p.requires_grad_(not name.startswith("gate"))
+    backward_of(x)
+    assert moe.gate.weight.grad is None
+    for name, p in moe.named_parameters():
+        if not name.startswith("gate"):
+            _assert_same(grads_full[name], p.grad, f"{name} (gate frozen)")
+    # no graph at all
+    with torch.no_grad():
+        _assert_same(y_full, moe(x, kernel_backend=KernelBackend.cuda)[0], "output under no_grad")
+    with torch.inference_mode():
+        _assert_same(y_full, moe(x, kernel_backend=KernelBackend.cuda)[0], "output under inference_mode")
