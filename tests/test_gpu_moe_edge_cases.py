@@ -114,3 +114,37 @@ def test_frozen_parameters_and_inference(dtype):
         _assert_same(y_full, moe(x, kernel_backend=KernelBackend.cuda)[0], "output under no_grad")
     with torch.inference_mode():
         _assert_same(y_full, moe(x, kernel_backend=KernelBackend.cuda)[0], "output under inference_mode")
+
+
+@pytest.mark.parametrize("add_bias", [False, True])
+def test_training_step_is_bit_reproducible(add_bias):
+    # nothing on the path accumulates with floating-point atomics (the reference's grouped rows, weight gradients and
+    # norm weight gradient do): two runs of one step on skewed routing over many experts give the same bits everywhere
+    from fma import fused_residual_add_rmsnorm
+
+    torch.manual_seed(5)
+    T, H, I, E, k = 4096, 256, 192, 64, 8
+    moe = MoE(E, k, H, I, swiglu_packed, True, add_bias, 0.02).to(DEV).to(torch.bfloat16)
+    with torch.no_grad():  # skew the routing: logits of the first experts spread wider, so they win the top-k more often
+        moe.gate.weight.mul_(torch.linspace(3.0, 0.2, E, device=DEV).bfloat16()[:, None])
+    norm_weight = torch.ones(H, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    x0 = torch.randn(T, H, device=DEV).bfloat16()
+    r0 = torch.randn(T, H, device=DEV).bfloat16()
+
+    def step():
+        moe.zero_grad(set_to_none=True)
+        norm_weight.grad = None
+        x, r = x0.clone().requires_grad_(), r0.clone().requires_grad_()
+        normed, residual = fused_residual_add_rmsnorm(x, r, norm_weight, 1e-5)
+        y, logits = moe(normed, kernel_backend=KernelBackend.cuda)
+        out = y + residual
+        (out.float().pow(2).mean() + 1e-2 * logits.float().pow(2).mean()).backward()
+        grads = {n: p.grad.clone() for n, p in moe.named_parameters()}
+        grads.update(x=x.grad, r=r.grad, norm_weight=norm_weight.grad.clone(), out=out.detach(), logits=logits.detach())
+        return grads
+
+    first, second = step(), step()
+    for name in first:
+        assert torch.equal(first[name], second[name]), name
+    counts = torch.bincount(moe._compute_routing_weights(x0)[2].flatten().long(), minlength=E)
+    assert int(counts.max()) > 4 * max(int(counts.min()), 1), "the routing of this test is meant to be skewed"
