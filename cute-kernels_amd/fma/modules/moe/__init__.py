@@ -117,8 +117,15 @@ class MoE(nn.Module):
         )
 
         self.act = activation_function
-        # swiglu_packed as the activation of a GLU layer is computed inside the up-projection's epilogue
-        self.fuse_swiglu = is_glu and _is_swiglu_packed(activation_function) and not add_bias
+        # swiglu_packed as the activation of a GLU layer is computed inside the up-projection's epilogue (a kernel for
+        # rows of whole 16-byte pieces; other sizes run the GEMM's element-wise path and the activation after it)
+        self.fuse_swiglu = (
+            is_glu
+            and _is_swiglu_packed(activation_function)
+            and not add_bias
+            and self.hidden_size % 8 == 0
+            and self.intermediate_size % 8 == 0
+        )
 
         self.c_proj = Experts(
             num_experts=num_experts,

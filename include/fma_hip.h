@@ -96,7 +96,8 @@ int fma_moe_build_index(const void* ids, int id_bytes, int64_t R, int64_t E, uin
 
 /* ---- row movement ------------------------------------------------------------------------- */
 
-/* out[i, :] = x[idx[i] / divisor, :] for i < R (rows of H elements, H*elem_bytes a multiple of 16).
+/* out[i, :] = x[idx[i] / divisor, :] for i < R (rows of H elements; the four row kernels move 16 bytes per lane when
+ * H*elem_bytes is a multiple of 16 and the buffers are 16-byte aligned, single elements otherwise).
  * Replaces group_with_padding_triton(..., NEEDS_DUPLICATION=True) without padding
  * (fma/modules/moe/cuda_implementation/group_kernel.py:26-74) and `hidden_states[fan_in_index]`
  * (fma/modules/moe/__init__.py:269,275). divisor = top_k maps a slot to its token; divisor = 1 is a

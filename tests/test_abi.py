@@ -64,14 +64,14 @@ def test_build_index_validation(lib):
 def test_row_kernels_validation(lib):
     buf = ctypes.create_string_buffer(4096 + 16)
     p = (ctypes.addressof(buf) + 15) & ~15
-    assert lib.fma_gather_rows(p, p, 4, 12, 1, p, 2, None) == -3 and "16 bytes" in _err(lib)  # H*2 % 16 != 0
+    assert lib.fma_gather_rows(p, p, 4, 0, 1, p, 2, None) == -3 and "row length" in _err(lib)  # any H >= 1 is served
     assert lib.fma_gather_rows(p, p, 4, 16, 0, p, 2, None) == -3  # divisor < 1
     assert lib.fma_gather_rows(p, p, 4, 16, 1, p, 7, None) == -2  # dtype code
     assert lib.fma_dispatch_rows(p, p, 4, 0, 16, p, 2, None) == -3  # top_k < 1
     assert lib.fma_dispatch_rows(p, None, 4, 2, 16, p, 2, None) == -1
     assert lib.fma_dispatch_rows(p, p, 0, 2, 16, p, 2, None) == 0
     assert lib.fma_combine(p, p, p, 4, 0, 16, p, 2, None) == -3  # top_k < 1
-    assert lib.fma_combine(p + 2, p, p, 4, 2, 16, p, 2, None) == -6
+    assert lib.fma_combine(p + 1, p, p, 4, 2, 16, p, 2, None) == -6  # not even aligned to the element size
     assert lib.fma_combine_bwd(p, None, p, p, 4, 2, 16, p, p, 2, None) == -1  # d_gates needs o
     assert lib.fma_gather_rows(p, p, 0, 16, 1, p, 2, None) == 0  # empty input: nothing to do
     assert lib.fma_combine(p, p, p, 0, 2, 16, p, 2, None) == 0

@@ -16,10 +16,12 @@ DTYPES = [torch.float32, torch.float16, torch.bfloat16]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,H,E,k", [(7, 64, 4, 2), (300, 4096, 8, 2), (257, 2048, 64, 8), (100, 576, 128, 8), (33, 8, 3, 1)])
+@pytest.mark.parametrize(
+    "T,H,E,k",
+    [(7, 64, 4, 2), (300, 4096, 8, 2), (257, 2048, 64, 8), (100, 576, 128, 8), (33, 8, 3, 1),
+     (33, 4, 3, 1), (64, 13, 17, 1), (50, 1, 4, 2), (40, 1001, 8, 3)],  # rows that are not whole 16-byte pieces: element-wise kernels
+)
 def test_gather_is_bit_exact(dtype, T, H, E, k):
-    if H * torch.finfo(dtype).bits // 8 % 16:
-        pytest.skip("row is not a multiple of 16 bytes")
     torch.manual_seed(T)
     x = torch.randn(T, H).to(dtype)
     selected, _ = O.make_routing(T, E, k, "uniform", seed=1)
@@ -34,7 +36,11 @@ def test_gather_is_bit_exact(dtype, T, H, E, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,H,E,k", [(7, 64, 4, 2), (300, 4096, 8, 2), (257, 2048, 64, 8), (64, 576, 128, 8), (50, 128, 16, 5)])
+@pytest.mark.parametrize(
+    "T,H,E,k",
+    [(7, 64, 4, 2), (300, 4096, 8, 2), (257, 2048, 64, 8), (64, 576, 128, 8), (50, 128, 16, 5),
+     (64, 13, 17, 1), (50, 1, 4, 2), (40, 1001, 8, 3), (9, 700, 16, 6)],  # element-wise kernels, cached and re-read dy rows
+)
 def test_combine_forward_and_backward(dtype, T, H, E, k):
     torch.manual_seed(T + k)
     selected, gates = O.make_routing(T, E, k, "uniform", seed=2)
