@@ -5,7 +5,7 @@ custom ops must trace without graph breaks and give the eager results."""
 import pytest
 import torch
 
-from fma import KernelBackend, MoE, continuous_count, grouped_gemm, swiglu, swiglu_packed
+from fma import KernelBackend, MoE, continuous_count, fused_residual_add_rmsnorm, grouped_gemm, swiglu, swiglu_packed
 from oracle import moe_oracle as O
 
 from gpu_util import DEV, to_np
@@ -67,8 +67,51 @@ def test_moe_compiled_matches_eager():
     yc = torch.compile(moe, fullgraph=True)(xc, kernel_backend=KernelBackend.cuda)[0]
     yc.sum().backward()
     assert torch.equal(yc, ye)
-    # gradients that pass through the router (ATen linear / top-k / softmax) are re-fused by Inductor and round
-    # differently in bf16; the custom ops themselves see identical inputs
+    # Inductor fuses the ATen glue around the custom ops (the loss, dtype casts, the matrix products of the router's
+    # backward) and rounds it differently in bf16; the custom ops themselves see identical inputs
     torch.testing.assert_close(xc.grad, xe.grad, rtol=1.6e-2, atol=2e-3)
     for k, p in moe.named_parameters():
         torch.testing.assert_close(p.grad, grads_e[k], rtol=1.6e-2, atol=2e-3, msg=k)
+
+
+class _Block(torch.nn.Module):
+    def __init__(self, E, k, H, I, add_bias, activation, is_glu):
+        super().__init__()
+        self.norm_weight = torch.nn.Parameter(torch.ones(H))
+        self.moe = MoE(E, k, H, I, activation, is_glu, add_bias, 0.05)
+
+    def forward(self, x, residual):
+        normed, residual = fused_residual_add_rmsnorm(x, residual, self.norm_weight, 1e-5)
+        y, router_logits = self.moe(normed, kernel_backend=KernelBackend.cuda)
+        return y + residual, router_logits
+
+
+@pytest.mark.parametrize(
+    "dtype,add_bias,activation,is_glu",
+    [
+        (torch.bfloat16, False, swiglu_packed, True),  # fused router, fused SwiGLU epilogue
+        (torch.bfloat16, True, swiglu_packed, True),  # fused router, GEMM + in-place bias + activation
+        (torch.bfloat16, False, torch.nn.GELU(approximate="tanh"), False),
+        (torch.float32, True, swiglu_packed, True),  # ATen router, fp32 GEMM
+    ],
+)
+def test_block_compiled_matches_eager(dtype, add_bias, activation, is_glu):
+    # residual add + RMSNorm, the layer with its router, the residual connection: one graph without breaks, forward and
+    # backward, against the eager run of the same modules
+    torch.manual_seed(0)
+    block = _Block(8, 2, 64, 128, add_bias, activation, is_glu).to(DEV).to(dtype)
+    x = torch.randn(50, 64, device=DEV).to(dtype)
+    residual = torch.randn(50, 64, device=DEV).to(dtype)
+
+    def step(f):
+        block.zero_grad(set_to_none=True)
+        xa, ra = x.clone().requires_grad_(), residual.clone().requires_grad_()
+        out, logits = f(xa, ra)
+        (out.float().pow(2).mean() + logits.float().pow(2).mean()).backward()
+        return [out.detach(), logits.detach(), xa.grad, ra.grad] + [p.grad.clone() for p in block.parameters()]
+
+    eager = step(block)
+    compiled = step(torch.compile(block, fullgraph=True))
+    bar = 1.6e-2 if dtype == torch.bfloat16 else 1e-5  # two bf16 ulps of the largest value for the re-fused glue
+    for a, b in zip(eager, compiled):
+        assert float((a.float() - b.float()).abs().max()) <= bar * float(a.float().abs().max())
