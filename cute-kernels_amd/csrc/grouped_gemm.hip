@@ -25,6 +25,8 @@
 //  * The MFMA is issued with B as the first operand, so a lane ends up holding four consecutive output
 //    columns of one output row. The epilogue transposes the wavefront's sub-tile through LDS (stage 1) and stores
 //    whole 128-byte row segments; the next tile's first loads are already on their way into stage 0 by then.
+#include <type_traits>
+
 #include "common.h"
 #include "grouped_gemm_f32.h"
 
@@ -675,60 +677,76 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                 for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.0f;
 
         // MFMA operand fragments of one 16-wide k slice, double buffered in registers
+        // The K loop exists in four versions, for wavefronts whose first FA = 4, 2, 1 or 0 row blocks (of 32 rows) hold
+        // rows of the group: the other blocks would multiply rows that the loads zero-filled, so their LDS reads and
+        // MFMAs are left out (their accumulators stay zero and the stores mask them). The last row tile of a group, and
+        // every tile of a group with few rows, then costs what its loads cost instead of a full tile's matrix work.
+        // FA is passed as an integral_constant so that each version is straight-line code.
         typename EL::frag fa[2][FM], fb[2][FN];
-        auto load_frags = [&](int stage, int ks, int buf) {
-            const uint8_t* ta = stage ? s_a1 : s_a0;
-            const uint8_t* tb = stage ? s_b1 : s_b0;
+        auto load_frags = [&](auto fa_c, int stage, int ks, int buf) {
+            constexpr int FA = decltype(fa_c)::value;
+            if constexpr (FA > 0) {
+                const uint8_t* ta = stage ? s_a1 : s_a0;
+                const uint8_t* tb = stage ? s_b1 : s_b0;
 #pragma unroll
-            for (int i = 0; i < FM; ++i) {
-                if constexpr (A_KC) fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_kc_frag(ta + a_off[i] + kc_slice[ks]));
-                else fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_tr_frag(ta + a_off[i] + ks * 16 * kTRowBytes));
-            }
+                for (int i = 0; i < FA; ++i) {
+                    if constexpr (A_KC) fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_kc_frag(ta + a_off[i] + kc_slice[ks]));
+                    else fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_tr_frag(ta + a_off[i] + ks * 16 * kTRowBytes));
+                }
 #pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                if constexpr (B_KC) fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_kc_frag(tb + b_off[j] + kc_slice[ks]));
-                else fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_tr_frag(tb + b_off[j] + ks * 16 * kTRowBytes));
+                for (int j = 0; j < FN; ++j) {
+                    if constexpr (B_KC) fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_kc_frag(tb + b_off[j] + kc_slice[ks]));
+                    else fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_tr_frag(tb + b_off[j] + ks * 16 * kTRowBytes));
+                }
             }
         };
-        auto mma = [&](int buf) {
+        auto mma = [&](auto fa_c, int buf) {
+            constexpr int FA = decltype(fa_c)::value;
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
+            for (int i = 0; i < FA; ++i)
 #pragma unroll
                 for (int j = 0; j < FN; ++j)
                     acc[i][j] = EL::mfma(fb[buf][j], fa[buf][i], acc[i][j]);
         };
         // ask the scheduler to alternate the MFMAs of one slice with the LDS reads of the next
-        constexpr int kReads = (A_KC ? FM : 2 * FM) + (B_KC ? FN : 2 * FN);
-        auto interleave_reads = [&]() { interleave_mfma_lds<0, FM * FN, kReads>(); };
+        auto interleave_reads = [&](auto fa_c) {
+            constexpr int FA = decltype(fa_c)::value;
+            constexpr int kReads = (A_KC ? FA : 2 * FA) + (B_KC ? FN : 2 * FN);
+            if constexpr (FA > 0) interleave_mfma_lds<0, FA * FN, kReads>();
+        };
 
         // ---- main loop over K ----
         // Step kt computes from stage kt&1. The workgroup barrier of a step sits between the LDS reads of its last
         // k slice and the MFMAs of that slice: once it is passed, the stage just read is free (the loads of step kt+2
         // are issued into it) and the other stage is complete (its first fragments are fetched), and both overlap
         // with the MFMAs still to be issued, so the matrix pipe has work while the barrier's latencies play out.
-        auto step = [&](int stage, uint32_t kt) {
-            load_frags(stage, 1, 1);
-            mma(0);
-            interleave_reads();
-            load_frags(stage, 2, 0);
-            mma(1);
-            interleave_reads();
-            load_frags(stage, 3, 1);
-            mma(0);
-            interleave_reads();
+        auto step = [&](auto fa_c, int stage, uint32_t kt) {
+            constexpr int FA = decltype(fa_c)::value;
+            load_frags(fa_c, stage, 1, 1);
+            mma(fa_c, 0);
+            interleave_reads(fa_c);
+            load_frags(fa_c, stage, 2, 0);
+            mma(fa_c, 1);
+            interleave_reads(fa_c);
+            load_frags(fa_c, stage, 3, 1);
+            mma(fa_c, 0);
+            interleave_reads(fa_c);
             // every load of step kt+1 has landed and every LDS read of this stage has returned
             __builtin_amdgcn_s_waitcnt(0x0070);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             // unconditional (after the last step the fragments are simply not used): straight-line code lets the
             // compiler count outstanding LDS reads exactly, so the MFMAs below do not wait for these reads
-            load_frags(stage ^ 1, 0, 0);
+            load_frags(fa_c, stage ^ 1, 0, 0);
             // the loads of step kt+2 go out one per MFMA (a burst of loads stalls the wavefront's instruction issue);
             // past the end of K they are all out of range (zero-fill), which keeps the loop body free of branches
             issue(stage, (kt + 2) * BK);
-            mma(1);
-            __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
-            spread_mfma_vmem<0, FM * FN, 2 * (32 / NW)>();
+            mma(fa_c, 1);
+            if constexpr (FA > 0) {
+                constexpr int kReads = (A_KC ? FA : 2 * FA) + (B_KC ? FN : 2 * FN);
+                __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
+                spread_mfma_vmem<0, FA * FN, 2 * (32 / NW)>();
+            }
         };
         const uint32_t KT = (Ke + BK - 1) / BK;
         Tile nxt{};
@@ -741,15 +759,26 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             wait_outstanding((prefetched ? tile_stores : 0u) + (KT > 1 ? kStepLoads : 0u));
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            load_frags(0, 0, 0);
-            // two steps per iteration without a branch between them (a branch there makes the compiler wait for the
-            // loads in flight before every LDS read at the top of the loop); an odd last step is peeled
-            uint32_t kt = 0;
-            for (; kt + 1 < KT; kt += 2) {
-                step(0, kt);
-                step(1, kt + 1);
-            }
-            if (kt < KT) step(0, kt);
+            auto k_loop = [&](auto fa_c) {
+                load_frags(fa_c, 0, 0, 0);
+                // two steps per iteration without a branch between them (a branch there makes the compiler wait for
+                // the loads in flight before every LDS read at the top of the loop); an odd last step is peeled
+                uint32_t kt = 0;
+                for (; kt + 1 < KT; kt += 2) {
+                    step(fa_c, 0, kt);
+                    step(fa_c, 1, kt + 1);
+                }
+                if (kt < KT) step(fa_c, 0, kt);
+            };
+            // rows of the group inside this wavefront's WM rows of the tile, in blocks of 32
+            const uint32_t tile_rows = Me - m0 < (uint32_t)BM ? Me - m0 : (uint32_t)BM;
+            const uint32_t wave_rows = tile_rows > wm * WM ? tile_rows - wm * WM : 0u;
+            const uint32_t row_blocks = uniform((wave_rows + 31u) / 32u);
+            static_assert(FM == 4, "the versions below are for four row blocks per wavefront");
+            if (row_blocks > 2) k_loop(std::integral_constant<int, 4>{});
+            else if (row_blocks == 2) k_loop(std::integral_constant<int, 2>{});
+            else if (row_blocks == 1) k_loop(std::integral_constant<int, 1>{});
+            else k_loop(std::integral_constant<int, 0>{});
             // the zero-fill loads issued past the end of K must have landed before the stages are reused below
             __builtin_amdgcn_s_waitcnt(0x0f70);
             __builtin_amdgcn_s_barrier();
