@@ -93,3 +93,16 @@ def test_routing_index(T, E, k, kind, empty, dtype):
     assert np.array_equal(to_np(eid), sorted_ids.numpy().astype(np.int32))
     if empty:
         assert (to_np(counts)[-empty:] == 0).all()
+
+
+def test_routing_index_fixture():
+    # tests/golden/routing_index_4096.npz: 4096 skewed ids, three empty experts, answers from numpy
+    import os
+
+    fx = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "routing_index_4096.npz"))
+    for dtype in (torch.int32, torch.int64):
+        ids = torch.from_numpy(fx["ids"]).to(dtype).to(DEV)
+        assert np.array_equal(to_np(continuous_count(x=ids, size=64)), fx["counts"])
+        counts, offsets, perm, eid, inv = build_routing_index(ids.view(-1, 1), 64)
+        for got, key in ((counts, "counts"), (offsets, "offsets"), (perm, "perm"), (eid, "eid"), (inv, "inv")):
+            assert np.array_equal(to_np(got), fx[key]), f"{key} ({dtype})"

@@ -290,3 +290,24 @@ def test_random_problems_with_several_tiles_per_workgroup(tA, tB):
         output_shape=(sum(m * n for m, n in zip(M_list, N_list)),), is_A_transposed=tA, is_B_transposed=tB,
     )
     assert float((got.float() - torch.cat(Ds).float()).abs().max()) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("layout", ["NT", "NN", "TN", "TT"])
+def test_known_answer_fixture(layout, dtype):
+    # tests/golden/grouped_gemm_kat.npz: int64 products of integer operands in [-8, 8] (four ragged groups, one empty);
+    # every partial sum is an integer below 2^24, so the kernel's result is the stored product rounded once to the dtype
+    import os
+
+    import numpy as np
+    from golden.make_golden import kat_problem
+
+    fx = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "grouped_gemm_kat.npz"))
+    M, N, K, tA, tB, As, Bs = kat_problem(layout)
+    A = torch.from_numpy(np.concatenate([a.reshape(-1) for a in As])).to(dtype).to(DEV)
+    B = torch.from_numpy(np.concatenate([b.reshape(-1) for b in Bs])).to(dtype).to(DEV)
+    got = grouped_gemm(
+        A=A, B=B, C=None, M_array=_u32(M), N_array=_u32(N), K_array=_u32(K),
+        output_shape=(sum(m * n for m, n in zip(M, N)),), is_A_transposed=tA, is_B_transposed=tB,
+    )
+    assert got.dtype == dtype and torch.equal(got.cpu(), torch.from_numpy(fx[layout]).float().to(dtype))

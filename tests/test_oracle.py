@@ -2,6 +2,8 @@
 the reference's own known-answer constructions, chosen so that a dropped term, a wrong index or a transposed operand
 fails at least one of them."""
 
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -332,3 +334,32 @@ def test_golden_fixture_is_what_the_oracle_computes():
     assert np.allclose(y.numpy(), fx["y"], atol=1e-6)
     idx = O.routing_index(selected.numpy(), 8)
     assert np.array_equal(idx["perm"], fx["perm"]) and np.array_equal(idx["counts"], fx["counts"])
+
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.mark.parametrize("count,index", [(O.continuous_count, O.routing_index), (c_oracle.continuous_count, c_oracle.routing_index)])
+def test_routing_index_fixture(count, index):
+    # 4096 skewed ids with three empty experts; the stored answers come from numpy's bincount / cumsum / stable argsort
+    fx = np.load(os.path.join(GOLDEN, "routing_index_4096.npz"))
+    assert np.array_equal(count(fx["ids"], 64), fx["counts"])
+    assert np.array_equal(count(fx["ids"].astype(np.int64), 64), fx["counts"])
+    idx = index(fx["ids"], 64)
+    for key in ("counts", "offsets", "perm", "eid", "inv"):
+        assert np.array_equal(idx[key], fx[key]), key
+
+
+@pytest.mark.parametrize("layout", ["NT", "NN", "TN", "TT"])
+def test_grouped_gemm_known_answer_fixture(layout):
+    # the stored products are int64 matrix products of the regenerated integer operands
+    from tests.golden.make_golden import kat_problem
+
+    fx = np.load(os.path.join(GOLDEN, "grouped_gemm_kat.npz"))
+    M, N, K, tA, tB, As, Bs = kat_problem(layout)
+    A = torch.from_numpy(np.concatenate([a.reshape(-1) for a in As])).float()
+    B = torch.from_numpy(np.concatenate([b.reshape(-1) for b in Bs])).float()
+    got = O.grouped_gemm(A, B, M, N, K, tA, tB)
+    assert got.dtype == torch.float32 and np.array_equal(got.numpy().astype(np.int64), fx[layout])
+    got16 = O.grouped_gemm(A.bfloat16(), B.bfloat16(), M, N, K, tA, tB)  # operands exact in bf16, one rounding of the result
+    assert torch.equal(got16, torch.from_numpy(fx[layout]).float().bfloat16())
