@@ -57,7 +57,7 @@ def parse_args():
 
 
 def time_gpu(fn, iters, warmup=3, blocker=None):
-    """Median and mean milliseconds of one launch of fn(i). Every launch is bracketed by its own pair of events on the
+    """Median, mean and minimum milliseconds of one launch of fn(i). Every launch is bracketed by its own pair of events on the
     current stream (the stream the kernels are launched on). `blocker` first queues a few milliseconds of other GPU
     work, so that all launches are already in the queue when the GPU reaches them and no host latency is measured."""
     import torch
@@ -75,7 +75,7 @@ def time_gpu(fn, iters, warmup=3, blocker=None):
         stops[i].record()
     torch.cuda.synchronize()
     times = sorted(starts[i].elapsed_time(stops[i]) for i in range(iters))
-    return times[len(times) // 2], sum(times) / len(times)
+    return times[len(times) // 2], sum(times) / len(times), times[0]
 
 
 def main():
@@ -223,7 +223,7 @@ def main():
                                     E, ta, tb, 1.0, BF16, stream))
 
         ok(lib.fma_gather_rows(x.data_ptr(), perm.data_ptr(), R, H, k, xg.data_ptr(), BF16, stream))
-        iters = max(5, args.steps)
+        iters = max(20, args.steps)
 
         only = [w for w in args.only.split(",") if w]
 
@@ -233,20 +233,20 @@ def main():
         def mfma(name, flops, fn, n=iters, nbytes=None, peak=PEAK_BF16_TFLOPS):
             if not want(name):
                 return
-            t = time_gpu(fn, n, blocker=blocker)
+            t = time_gpu(fn, n, warmup=5, blocker=blocker)
             tf = flops / (t[0] * 1e-3) / 1e12
-            kernels[name] = {"ms": t[0], "ms_mean": t[1], "bound": "mfma", "achieved": tf, "peak": peak,
+            kernels[name] = {"ms": t[0], "ms_mean": t[1], "ms_min": t[2], "bound": "mfma", "achieved": tf, "peak": peak,
                              "unit": "TFLOP/s", "frac": tf / peak, "flop": flops}
             if nbytes is not None:  # the second roof: operands read once, output written once
                 kernels[name]["hbm_bytes"] = nbytes
                 kernels[name]["hbm_frac"] = nbytes / (t[0] * 1e-3) / 1e9 / PEAK_HBM_GBS
 
-        def hbm(name, nbytes, fn, n=20, warmup=3):
+        def hbm(name, nbytes, fn, n=50, warmup=10):
             if not want(name):
                 return
             t = time_gpu(fn, n, warmup=warmup, blocker=blocker)
             gbs = nbytes / (t[0] * 1e-3) / 1e9
-            kernels[name] = {"ms": t[0], "ms_mean": t[1], "bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS,
+            kernels[name] = {"ms": t[0], "ms_mean": t[1], "ms_min": t[2], "bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS,
                              "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "bytes": nbytes}
 
         w1_b, w2_b = E * 2 * I * H * s, E * H * I * s  # bytes of the two weight tensors
@@ -284,7 +284,7 @@ def main():
         if want("hbm_copy_1GiB"):
             src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()
             dst = torch.empty_like(src)
-            hbm("hbm_copy_1GiB", 2 * src.numel() * s, lambda i: dst.copy_(src), n=10)
+            hbm("hbm_copy_1GiB", 2 * src.numel() * s, lambda i: dst.copy_(src), n=30)
             del src, dst
 
         # Row kernels: algorithmic bytes = each distinct input row once + each output row once + index / gate words.
@@ -323,10 +323,10 @@ def main():
         es = 2 * I  # row stride of the packed pre-activation and of its gradient
         hbm("swiglu_forward", 3 * R * I * s,
             lambda i: ok(lib.fma_swiglu_forward(h.data_ptr() + I * s, h.data_ptr(), a.data_ptr(), R, I, es, es, I, BF16,
-                                                stream)), n=10)
+                                                stream)), n=30)
         hbm("swiglu_backward", 5 * R * I * s,
             lambda i: ok(lib.fma_swiglu_backward(h.data_ptr() + I * s, h.data_ptr(), da.data_ptr(), dh.data_ptr() + I * s,
-                                                 dh.data_ptr(), R, I, es, es, I, es, es, BF16, stream)), n=10)
+                                                 dh.data_ptr(), R, I, es, es, I, es, es, BF16, stream)), n=30)
         # router: x and the gate weight read once, logits / weights / choice / histogram written. Three copies of x
         # (together larger than the 256 MiB last-level cache) are rotated so that every launch reads from HBM.
         if want("router"):
@@ -397,10 +397,10 @@ def main():
                                device=dev)
             hbm("expert_bias_add", 2 * R * 2 * I * s + E * 2 * I * s,
                 lambda i: ok(lib.fma_expert_bias_add(h.data_ptr(), b1.data_ptr(), counts.data_ptr(), E, R, 2 * I, BF16,
-                                                     stream)), n=10)
+                                                     stream)), n=30)
             hbm("expert_bias_grad(2 launches)", R * 2 * I * s + E * 2 * I * s,
                 lambda i: ok(lib.fma_expert_bias_grad(dh.data_ptr(), counts.data_ptr(), E, R, 2 * I, db1.data_ptr(),
-                                                      ws_b.data_ptr(), ws_b.numel(), BF16, stream)), n=10)
+                                                      ws_b.data_ptr(), ws_b.numel(), BF16, stream)), n=30)
         if want("build_routing_index"):
             ws_idx = torch.empty(max(lib.fma_moe_build_index_workspace_bytes(R, E), 4) // 4, dtype=torch.int32, device=dev)
             t = time_gpu(lambda i: ok(lib.fma_moe_build_index(selected_d.data_ptr(), 8, R, E, counts.data_ptr(),
