@@ -254,6 +254,11 @@ def main():
              lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), h.data_ptr(), a.data_ptr(),
                                                       counts.data_ptr(), E, I, H, BF16, stream)),
              nbytes=R * H * s + w1_b + R * 3 * I * s)
+        # the same launch as a forward without a backward runs it: the pre-activation h is not stored
+        mfma("up_projection_swiglu_fwd_inference(NT, h not stored)", 2.0 * R * 2 * I * H,
+             lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), None, a.data_ptr(),
+                                                      counts.data_ptr(), E, I, H, BF16, stream)),
+             nbytes=R * H * s + w1_b + R * I * s)
         # the unfused pair the fused kernel above replaces (same bits): plain up-projection, then swiglu_forward below
         mfma("up_projection_plain_fwd(NT)", 2.0 * R * 2 * I * H, lambda i: gemm(xg, w1, h, counts, N_fc, K_fc, 0, 1),
              nbytes=R * H * s + w1_b + R * 2 * I * s)
