@@ -53,7 +53,8 @@ constexpr int kGroupM = 8;                  // m-tiles that share one column swe
 constexpr int kXcds = 8;
 
 constexpr int EPI_PLAIN = 0;
-constexpr int EPI_SWIGLU = 1;
+constexpr int EPI_SWIGLU = 1;      // stores the rounded pre-activation h and the activation
+constexpr int EPI_SWIGLU_ACT = 2;  // the activation only (a forward pass that no backward follows)
 
 struct GemmArgs {
     const uint16_t* A;
@@ -436,7 +437,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     // n-extent covered by the tile grid: for the SwiGLU epilogue a tile spans 128 up + 128 gate columns
     auto tiles_of = [&](uint32_t m, uint32_t n) -> uint32_t {
         if (m == 0 || n == 0) return 0;
-        const uint32_t tn = EPI == EPI_SWIGLU ? (n / 2 + BN / 2 - 1) / (BN / 2) : (n + BN - 1) / BN;
+        const uint32_t tn = EPI != EPI_PLAIN ? (n / 2 + BN / 2 - 1) / (BN / 2) : (n + BN - 1) / BN;
         return ((m + BM - 1) / BM) * tn;
     };
 
@@ -513,7 +514,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
 
     // first tile row of B fragment j of this wavefront
     auto b_frag_row = [&](int j) -> uint32_t {
-        if constexpr (EPI == EPI_SWIGLU) {
+        if constexpr (EPI != EPI_PLAIN) {
             return j < FN / 2 ? wn * (WN / 2) + j * 32 : BN / 2 + wn * (WN / 2) + (j - FN / 2) * 32;
         } else {
             return wn * WN + j * 32;
@@ -547,7 +548,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         uint32_t Me, Ne, Ke, n_span, m0, n0;
         uint64_t off_a, off_b, off_d;
     };
-    constexpr uint32_t TN = EPI == EPI_SWIGLU ? BN / 2 : BN;  // columns of the tile grid one tile covers
+    constexpr uint32_t TN = EPI != EPI_PLAIN ? BN / 2 : BN;  // columns of the tile grid one tile covers
     // Rounds of `grid` tiles are dealt in alternating directions (slot s takes tile s of even rounds and tile
     // grid-1-s of odd ones): when the tiles get cheaper along the tile order (groups with shrinking reduction length, as in
     // weight gradients under skewed routing) a workgroup that drew an expensive tile in one round draws a cheap one in the
@@ -568,7 +569,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         t.Me = group_m(e);
         t.Ne = group_n(e);
         t.Ke = group_k(e);
-        t.n_span = EPI == EPI_SWIGLU ? t.Ne / 2 : t.Ne;  // columns the tile grid runs over
+        t.n_span = EPI != EPI_PLAIN ? t.Ne / 2 : t.Ne;  // columns the tile grid runs over
         const uint32_t tiles_m = (t.Me + BM - 1) / BM;
         const uint32_t tiles_n = (t.n_span + TN - 1) / TN;
         const uint32_t local = v - uniform(s_tile_start[pos]);
@@ -590,14 +591,14 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                     (t.off_d % 8u == 0);
         if (A_KC || B_KC) fast = fast && (t.Ke % 8u == 0) && (t.Ke < (1u << 21));
         if (!A_KC) fast = fast && (t.Me % 8u == 0) && (t.Me < (1u << 23));
-        if (EPI == EPI_SWIGLU) fast = fast && (t.n_span % 8u == 0);
+        if (EPI != EPI_PLAIN) fast = fast && (t.n_span % 8u == 0);
         t.fast = fast;
         return t;
     };
 
     // ---- loaders (state of the tile whose operands are being loaded) ----
     LoaderK<NW, false> lk_a;
-    LoaderK<NW, EPI == EPI_SWIGLU> lk_b;
+    LoaderK<NW, EPI != EPI_PLAIN> lk_b;
     LoaderT<NW> lt_a, lt_b;
     auto setup_loaders = [&](const Tile& t) {
         const uint16_t* Ae = args.A + t.off_a;
@@ -609,7 +610,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             lt_a.setup(Ae, t.Me, t.Ke, t.m0, wave, lane);
         }
         if constexpr (B_KC) {
-            if constexpr (EPI == EPI_SWIGLU) {
+            if constexpr (EPI != EPI_PLAIN) {
                 // tile rows 0..127: "up" rows n0.. of the weight; rows 128..255: "gate" rows I + n0..
                 const uint32_t rows = t.n_span - t.n0 < (uint32_t)(BN / 2) ? t.n_span - t.n0 : (uint32_t)(BN / 2);
                 lk_b.setup(Be + (uint64_t)t.n0 * t.Ke, Be + (uint64_t)(t.n_span + t.n0) * t.Ke, rows, t.Ke, wave, lane);
@@ -637,7 +638,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     };
     constexpr uint32_t kStepLoads = 2 * (32 / NW);  // load instructions per wavefront and K step
     // store instructions per wavefront and tile (stage_flush issues a fixed number)
-    const uint32_t tile_stores = EPI == EPI_PLAIN ? WM * WN * 2 / 1024 : (args.D ? WM * WN * 2 / 1024 : 0) + WM * WN / 1024;
+    const uint32_t tile_stores = EPI == EPI_PLAIN ? WM * WN * 2 / 1024 : (EPI == EPI_SWIGLU ? WM * WN * 2 / 1024 : 0) + WM * WN / 1024;
     // waits until at most n of this wavefront's loads and stores are outstanding (they complete in issue order)
     auto wait_outstanding = [&](uint32_t n) {
         if (n >= 40) __builtin_amdgcn_s_waitcnt(0x8f78);       // vmcnt(40)
@@ -854,7 +855,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                             }
                             ypack[i][j][q][0] = EL::pack2(y[0], y[1]);
                             ypack[i][j][q][1] = EL::pack2(y[2], y[3]);
-                            if (args.D) {
+                            if constexpr (EPI == EPI_SWIGLU) {
                                 const uint32_t m = i * 32 + (el & 31u);
                                 const uint32_t c = j * 32 + q * 8 + (el >> 5) * 4;
                                 uint2 wu, wg;
@@ -866,7 +867,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                                 stage_put<HB>(img, m, WN / 2 + c, wg);
                             }
                         }
-                if (args.D)
+                if constexpr (EPI == EPI_SWIGLU)
                     stage_flush_split<HB, HM, WN / 2>(img, args.D + off_d + (uint64_t)row0 * Ne + col0, Ne, rows_valid,
                                                       cols_valid, n_span, el);
 #pragma unroll
@@ -901,7 +902,8 @@ constexpr int kWavesN = FMA_GEMM_WAVES_N;
     template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, true, false, EPI_PLAIN>(const GemmArgs); \
     template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, false, true, EPI_PLAIN>(const GemmArgs); \
     template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, false, false, EPI_PLAIN>(const GemmArgs); \
-    template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, true, true, EPI_SWIGLU>(const GemmArgs);
+    template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, true, true, EPI_SWIGLU>(const GemmArgs); \
+    template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, true, true, EPI_SWIGLU_ACT>(const GemmArgs);
 FMA_GEMM_INSTANTIATE(ElemBf16)
 FMA_GEMM_INSTANTIATE(ElemF16)
 #undef FMA_GEMM_INSTANTIATE
@@ -988,8 +990,12 @@ int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, co
     args.const_n = (uint32_t)(2 * I);
     args.const_k = (uint32_t)K;
     args.alpha = 1.0f;
-    return dtype == FMA_BF16 ? launch<ElemBf16, true, true, EPI_SWIGLU>(args, (hipStream_t)stream)
-                             : launch<ElemF16, true, true, EPI_SWIGLU>(args, (hipStream_t)stream);
+    // whether h is stored is a compile-time property of the kernel: the epilogue is then one straight-line block
+    if (h)
+        return dtype == FMA_BF16 ? launch<ElemBf16, true, true, EPI_SWIGLU>(args, (hipStream_t)stream)
+                                 : launch<ElemF16, true, true, EPI_SWIGLU>(args, (hipStream_t)stream);
+    return dtype == FMA_BF16 ? launch<ElemBf16, true, true, EPI_SWIGLU_ACT>(args, (hipStream_t)stream)
+                             : launch<ElemF16, true, true, EPI_SWIGLU_ACT>(args, (hipStream_t)stream);
 }
 
 }  // extern "C"
