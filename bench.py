@@ -88,9 +88,8 @@ def main():
     import torch
 
     import fma
-    from fma import KernelBackend, MoE, continuous_count, grouped_gemm, swiglu_packed
+    from fma import KernelBackend, MoE, swiglu_packed
     from fma.modules.moe import cuda_implementation as ci
-    from fma.ops.swiglu.cuda_implementation import swiglu_backward_cuda
     from oracle import moe_oracle as O
 
     if not torch.cuda.is_available():

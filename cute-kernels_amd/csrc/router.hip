@@ -197,7 +197,7 @@ __global__ __launch_bounds__(kRouterThreads) void router_topk_kernel(const Route
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
-    const int H = a.H, E = a.E, k = a.k;
+    const int H = a.H, E = a.E;
     const int64_t tok0 = (int64_t)blockIdx.x * kToks;
 
     if (a.counts)

@@ -1,7 +1,6 @@
 """GPU parity of the per-expert bias (fma_expert_bias_add / fma_expert_bias_grad) and of the MoE layer with
 add_bias=True against the oracle's per-expert F.linear(x_e, W[e], bias[e]) (fma/modules/moe/__init__.py:98-105)."""
 
-import numpy as np
 import pytest
 import torch
 import torch.nn as nn
