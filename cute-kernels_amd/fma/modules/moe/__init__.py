@@ -25,25 +25,19 @@ from .cuda_implementation import (
 
 
 class Experts(nn.Module):
+    """The weights (and optional biases) of all experts of one projection: `weight[e]` is expert e's [out, in] matrix."""
+
     def __init__(
         self, num_experts: int, in_features: int, out_features: int, add_bias: bool = True, std: float | None = None
     ) -> None:
         super().__init__()
+        self.num_experts, self.in_features, self.out_features, self.std = num_experts, in_features, out_features, std
 
         self.weight = nn.Parameter(torch.empty(num_experts, out_features, in_features))
-
-        self.bias = None
-        if add_bias:
-            self.bias = nn.Parameter(torch.empty(num_experts, out_features))
-
-        self.std = std
-
-        self.num_experts = num_experts
-        self.in_features = in_features
-        self.out_features = out_features
-
-        self.register_buffer("N_array", torch.empty((num_experts,), dtype=torch.uint32))
-        self.register_buffer("K_array", torch.empty((num_experts,), dtype=torch.uint32))
+        self.bias = nn.Parameter(torch.empty(num_experts, out_features)) if add_bias else None
+        # per-group N and K of the grouped GEMM, kept on the device next to the weights (buffers of the state_dict)
+        for name in ("N_array", "K_array"):
+            self.register_buffer(name, torch.empty((num_experts,), dtype=torch.uint32))
 
         self.reset_parameters()
 
@@ -64,17 +58,15 @@ class Experts(nn.Module):
             x=input, weight=self.weight, M_array=expert_frequency, N_array=self.N_array, K_array=self.K_array
         )
 
-    def extra_repr(self):
-        return "num_experts={}, in_features={}, out_features={}".format(
-            self.num_experts, self.in_features, self.out_features
-        )
+    def extra_repr(self) -> str:
+        return f"num_experts={self.num_experts}, in_features={self.in_features}, out_features={self.out_features}"
 
     @torch.no_grad()
     def reset_parameters(self) -> None:
+        # N(0, std) weights, zero biases (fma/modules/moe/__init__.py:112-121), and the two size buffers
         nn.init.normal_(self.weight, mean=0, std=self.std)
-        if hasattr(self, "bias") and self.bias is not None:
+        if getattr(self, "bias", None) is not None:
             self.bias.zero_()
-
         self.N_array.fill_(self.out_features)
         self.K_array.fill_(self.in_features)
 

@@ -1,3 +1,2 @@
 from .contiguous import ensure_contiguous
-from .random import set_seed
-from .tensor import get_num_elements_and_hidden_size
+from .misc import get_num_elements_and_hidden_size, set_seed
