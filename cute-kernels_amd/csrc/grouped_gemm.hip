@@ -216,6 +216,26 @@ struct LoaderK {
             buffer_load_lds_quiet(second ? r1 : r0, v, k0 * 2u + row * ldb, lds0 + (uint32_t)(i * NW) * 1024u);
         }
     }
+    // only the instruction that covers tile rows 0 .. NW*8-1, to the LDS address lds_base (a tile with few rows)
+    __device__ __forceinline__ void issue_quiet_first_rows(uint32_t lds_base, uint32_t k0) const {
+        uint32_t v = voff;
+        if (k0 + BK > kdim && k0 + chunk * 8u >= kdim) v = kOutOfRange;
+        buffer_load_lds_quiet(make_rsrc_words(base0, bytes), v, k0 * 2u, lds_base + wave * 1024u);
+    }
+    // the NI loads with the first half of the tile's 1 KB pieces going to lds_lo and the second half to lds_hi
+    __device__ __forceinline__ void issue_quiet_halves(uint32_t lds_lo, uint32_t lds_hi, uint32_t k0) const {
+        uint32_t v = voff;
+        if (k0 + BK > kdim && k0 + chunk * 8u >= kdim) v = kOutOfRange;
+        const u32x4 r0 = make_rsrc_words(base0, bytes);
+        const u32x4 r1 = make_rsrc_words(SPLIT ? base1 : base0, bytes);
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const bool second = SPLIT && i >= NI / 2;
+            const uint32_t row = (uint32_t)(second ? i - NI / 2 : i) * kRowsPerInst;
+            const uint32_t lds = (i < NI / 2 ? lds_lo + (uint32_t)(i * NW) * 1024u : lds_hi + (uint32_t)((i - NI / 2) * NW) * 1024u) + wave * 1024u;
+            buffer_load_lds_quiet(second ? r1 : r0, v, k0 * 2u + row * ldb, lds);
+        }
+    }
 };
 
 // Operand stored [reduction][out] (out contiguous): tile [64 k][256 out]. A wavefront instruction moves two k rows
@@ -260,6 +280,16 @@ struct LoaderT {
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             buffer_load_lds_quiet(r, voff, (uint32_t)(i * NW + wave) * 2u * ldb, lds0 + (uint32_t)(i * NW) * 1024u);
+        }
+    }
+    // the NI loads with k rows 0..31 of the step going to lds_lo and k rows 32..63 to lds_hi
+    __device__ __forceinline__ void issue_quiet_halves(uint32_t lds_lo, uint32_t lds_hi, uint32_t k0) const {
+        const uint32_t rows = k0 >= kdim ? 0u : (kdim - k0 < (uint32_t)BK ? kdim - k0 : (uint32_t)BK);
+        const u32x4 r = make_rsrc_words(base + (uint64_t)k0 * (ldb / 2u), rows ? rows * ldb - col_bytes : 0u);
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const uint32_t lds = (i < NI / 2 ? lds_lo + (uint32_t)(i * NW) * 1024u : lds_hi + (uint32_t)((i - NI / 2) * NW) * 1024u) + wave * 1024u;
+            buffer_load_lds_quiet(r, voff, (uint32_t)(i * NW + wave) * 2u * ldb, lds);
         }
     }
 };
@@ -646,6 +676,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         else if (n >= 24) __builtin_amdgcn_s_waitcnt(0x4f78);  // vmcnt(24)
         else if (n >= 16) __builtin_amdgcn_s_waitcnt(0x4f70);  // vmcnt(16)
         else if (n >= 8) __builtin_amdgcn_s_waitcnt(0x0f78);   // vmcnt(8)
+        else if (n >= 5) __builtin_amdgcn_s_waitcnt(0x0f75);   // vmcnt(5)
         else __builtin_amdgcn_s_waitcnt(0x0f70);               // vmcnt(0)
     };
 
@@ -752,7 +783,90 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         const uint32_t KT = (Ke + BK - 1) / BK;
         Tile nxt{};
         if (KT == 0) nxt = lookup(++round);
-        if (KT > 0) {
+        // rows of the group inside the tile, and inside this wavefront's WM rows of it in blocks of 32
+        const uint32_t tile_rows = Me - m0 < (uint32_t)BM ? Me - m0 : (uint32_t)BM;
+        const uint32_t wave_rows = tile_rows > wm * WM ? tile_rows - wm * WM : 0u;
+        const uint32_t row_blocks = uniform((wave_rows + 31u) / 32u);
+        // A tile with at most 64 rows leaves three quarters of the A stages unused, and its K steps cost what the latency
+        // of their loads costs. It runs a K loop of its own with a third LDS stage in that unused space (A rows 0..63 are
+        // 8 KB; the B tile of stage 2 lies in two halves behind the A tiles of stages 0 and 1), so that two steps of
+        // loads are in flight instead of one. All of its loads are the assembly-written ones, counted by hand.
+        // Only groups that consist of such a tile alone take it (batches of a few rows per group, where the kernel is a
+        // stream of the B operand): the short last tile of a larger group gains nothing from running ahead of the full
+        // tiles beside it, whose loads of the same B panel it otherwise shares in the L2 (measured: 3 % slower).
+        const bool thin = A_KC && Me <= 64u && KT >= 3u;
+        if (thin) {
+            constexpr uint32_t kThinLoads = 1 + 32 / NW;  // per wavefront and K step: one for A, the usual ones for B
+            static_assert(kThinLoads == 5, "the waits below are written for five loads per step");
+            const uint8_t* const a_at[3] = {s_a0, s_a1, s_a0 + 8192};
+            const uint8_t* const b_lo[3] = {s_b0, s_b1, s_a0 + 16384};
+            const uint8_t* const b_hi[3] = {s_b0 + 16384, s_b1 + 16384, s_a1 + 16384};
+            auto issue_thin = [&](int st, uint32_t k0) {
+                if constexpr (A_KC) lk_a.issue_quiet_first_rows(lds_address(a_at[st]), k0);
+                if constexpr (B_KC) lk_b.issue_quiet_halves(lds_address(b_lo[st]), lds_address(b_hi[st]), k0);
+                else lt_b.issue_quiet_halves(lds_address(b_lo[st]), lds_address(b_hi[st]), k0);
+            };
+            // stage 0 in the usual places (an earlier prefetch put it there; the zero rows it wrote behind A's first
+            // 8 KB are complete, for every wavefront, once the barrier below is passed), stage 1 likewise
+            if (!prefetched) issue_thin(0, 0);
+            issue_thin(1, BK);
+            nxt = lookup(++round);
+            wait_outstanding((prefetched ? tile_stores : 0u) + kThinLoads);
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            issue_thin(2, 2 * BK);
+            auto thin_loop = [&](auto fa_c) {
+                constexpr int FA = decltype(fa_c)::value;
+                auto thin_step = [&](int st, uint32_t kt) {
+                    if constexpr (FA > 0) {
+#pragma unroll
+                        for (int ks = 0; ks < 4; ++ks) {
+                            typename EL::frag ta[FA], tb[FN];
+#pragma unroll
+                            for (int i = 0; i < FA; ++i)
+                                ta[i] = __builtin_bit_cast(typename EL::frag, read_kc_frag(a_at[st] + a_off[i] + kc_slice[ks]));
+#pragma unroll
+                            for (int j = 0; j < FN; ++j) {
+                                if constexpr (B_KC) {
+                                    // tile rows 0..127 are the first half of the B tile, rows 128..255 the second
+                                    const uint8_t* half = b_frag_row(j) < 128u ? b_lo[st] + b_off[j] : b_hi[st] + (b_off[j] - 128u * kRowBytes);
+                                    tb[j] = __builtin_bit_cast(typename EL::frag, read_kc_frag(half + kc_slice[ks]));
+                                } else {
+                                    // k rows 0..31 of the step are the first half, 32..63 the second
+                                    const uint8_t* half = ks < 2 ? b_lo[st] + ks * 16 * kTRowBytes : b_hi[st] + (ks - 2) * 16 * kTRowBytes;
+                                    tb[j] = __builtin_bit_cast(typename EL::frag, read_tr_frag(half + b_off[j]));
+                                }
+                            }
+#pragma unroll
+                            for (int i = 0; i < FA; ++i)
+#pragma unroll
+                                for (int j = 0; j < FN; ++j) acc[i][j] = EL::mfma(tb[j], ta[i], acc[i][j]);
+                        }
+                    }
+                    // all but the newest five loads: step kt+1 has landed (step kt+2 may still be on its way); past the
+                    // barrier every wavefront has finished reading this stage, which then takes the loads of step kt+3
+                    // (zero-filling ones past the end of K, so that the count stays the same)
+                    __builtin_amdgcn_s_waitcnt(0x0f75);
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    issue_thin(st, (kt + 3) * BK);
+                };
+                uint32_t kt = 0;
+                for (; kt + 2 < KT; kt += 3) {
+                    thin_step(0, kt);
+                    thin_step(1, kt + 1);
+                    thin_step(2, kt + 2);
+                }
+                if (kt < KT) thin_step(0, kt);
+                if (kt + 1 < KT) thin_step(1, kt + 1);
+            };
+            if (row_blocks == 2) thin_loop(std::integral_constant<int, 2>{});
+            else if (row_blocks == 1) thin_loop(std::integral_constant<int, 1>{});
+            else thin_loop(std::integral_constant<int, 0>{});
+            __builtin_amdgcn_s_waitcnt(0x0f70);
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        } else if (KT > 0) {
             if (!prefetched) issue_quiet(0, 0);
             if (KT > 1) issue_quiet(1, BK);
             nxt = lookup(++round);  // in the shadow of the loads
@@ -771,10 +885,6 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                 }
                 if (kt < KT) step(fa_c, 0, kt);
             };
-            // rows of the group inside this wavefront's WM rows of the tile, in blocks of 32
-            const uint32_t tile_rows = Me - m0 < (uint32_t)BM ? Me - m0 : (uint32_t)BM;
-            const uint32_t wave_rows = tile_rows > wm * WM ? tile_rows - wm * WM : 0u;
-            const uint32_t row_blocks = uniform((wave_rows + 31u) / 32u);
             static_assert(FM == 4, "the versions below are for four row blocks per wavefront");
             if (row_blocks > 2) k_loop(std::integral_constant<int, 4>{});
             else if (row_blocks == 2) k_loop(std::integral_constant<int, 2>{});

@@ -311,3 +311,45 @@ def test_known_answer_fixture(layout, dtype):
         output_shape=(sum(m * n for m, n in zip(M, N)),), is_A_transposed=tA, is_B_transposed=tB,
     )
     assert got.dtype == dtype and torch.equal(got.cpu(), torch.from_numpy(fx[layout]).float().to(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tB", [True, False])
+@pytest.mark.parametrize("K", [192, 256, 320, 1000, 2112, 4096])  # 3, 4, 5, 16, 33, 64 K steps: every phase of the three-stage loop
+def test_groups_of_few_rows_with_long_reductions(K, tB, dtype):
+    # groups of at most 64 rows (batches of a few tokens per expert) run a K loop of their own with three LDS stages;
+    # groups of 65 and 300 rows beside them take the usual loop. Integer operands in [-2, 2]: every partial sum is an
+    # integer far below 2^24, so the kernel's result is the exact (int64) product rounded once to the dtype
+    M_list, N = [1, 8, 33, 64, 0, 65, 17, 300, 64, 5], 328
+    E = len(M_list)
+    g = torch.Generator().manual_seed(K)
+    As = [torch.randint(-2, 3, (m, K), generator=g) for m in M_list]
+    Bs = [torch.randint(-2, 3, (N, K) if tB else (K, N), generator=g) for _ in M_list]
+    A = torch.cat([a.reshape(-1) for a in As]).to(dtype).to(DEV)
+    B = torch.cat([b.reshape(-1) for b in Bs]).to(dtype).to(DEV)
+    got = grouped_gemm(
+        A=A, B=B, C=None, M_array=_u32(M_list), N_array=_u32([N] * E), K_array=_u32([K] * E),
+        output_shape=(sum(M_list) * N,), is_A_transposed=False, is_B_transposed=tB,
+    )
+    expect = torch.cat([(a @ (b.T if tB else b)).reshape(-1) for a, b in zip(As, Bs)]).float().to(dtype)  # int64 products
+    assert torch.equal(got.cpu(), expect)
+
+
+@pytest.mark.parametrize("K", [192, 1000, 4096])
+def test_fused_swiglu_on_groups_of_few_rows(K):
+    # the same for the fused epilogue: bit-identical to the plain GEMM followed by swiglu_packed
+    M_list, I = [3, 64, 0, 40, 200, 64, 1], 136
+    E, R = len(M_list), sum(M_list)
+    g = torch.Generator().manual_seed(K + 1)
+    x = (torch.randn(R, K, generator=g) * 0.5).bfloat16().to(DEV)
+    w = (torch.randn(E, 2 * I, K, generator=g) * 0.05).bfloat16().to(DEV)
+    h = torch.empty(R, 2 * I, dtype=torch.bfloat16, device=DEV)
+    act = torch.empty(R, I, dtype=torch.bfloat16, device=DEV)
+    grouped_gemm_swiglu_cuda(x, w, _u32(M_list), h, act)
+    h_plain = grouped_gemm(
+        A=x, B=w, C=None, M_array=_u32(M_list), N_array=_u32([2 * I] * E), K_array=_u32([K] * E),
+        output_shape=(R, 2 * I), is_A_transposed=False, is_B_transposed=True,
+    )
+    assert torch.equal(h, h_plain) and torch.equal(act, swiglu_packed(h_plain))
+    expect = torch.cat([xe.float() @ w[e].float().T for e, xe in enumerate(x.split(M_list))])
+    assert float((h.float() - expect).abs().max()) <= 2**-8 * float(expect.abs().max())
