@@ -283,6 +283,20 @@ def main():
                                                    stream)), n=3, peak=PEAK_F32_TFLOPS)
             del a32, w32, o32
 
+        # the same two forward GEMMs on a batch of a few rows per expert (16 each, e.g. 64 tokens at top-2 of 8): there
+        # the kernels are a stream of the expert weights, so the roof is the HBM one and the bytes are the weights' (plus
+        # the few activation rows)
+        M_dec = max(1, min(64, 128 // E))
+        R_dec = M_dec * E
+        counts_dec = torch.full((E,), M_dec, dtype=torch.int32, device=dev).view(torch.uint32)
+        if want("small_batch_up_fwd"):
+            hbm(f"small_batch_up_fwd(NT + SwiGLU, {M_dec} rows per expert, h not stored)", w1_b + R_dec * (H + I) * s,
+                lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), None, a.data_ptr(),
+                                                         counts_dec.data_ptr(), E, I, H, BF16, stream)), n=30)
+        if want("small_batch_down_fwd"):
+            hbm(f"small_batch_down_fwd(NT, {M_dec} rows per expert)", w2_b + R_dec * (H + I) * s,
+                lambda i: gemm(a, w2, o, counts_dec, N_pj, K_pj, 0, 1), n=30)
+
         # calibration for the profiler's FETCH_SIZE / WRITE_SIZE counters: a plain device copy of known size (ATen's
         # elementwise copy kernel): reads 1 GiB, writes 1 GiB
         if want("hbm_copy_1GiB"):
