@@ -464,10 +464,16 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     auto group_m = [&](uint32_t e) { return m_arr[e]; };
     auto group_n = [&](uint32_t e) { return n_arr ? n_arr[e] : args.const_n; };
     auto group_k = [&](uint32_t e) { return k_arr ? k_arr[e] : args.const_k; };
+    // Column tiles of half the width for groups of at most 64 rows, when the launch would otherwise have tiles for no more
+    // than half of the workgroups (a few rows per group and a short N: the kernel is then a stream of the B operand, and
+    // twice as many workgroups stream it). Decided once per launch, below, from the group sizes; plain NT only.
+    constexpr bool kCanNarrow = EPI == EPI_PLAIN && A_KC && B_KC;
+    bool narrow = false;
     // n-extent covered by the tile grid: for the SwiGLU epilogue a tile spans 128 up + 128 gate columns
     auto tiles_of = [&](uint32_t m, uint32_t n) -> uint32_t {
         if (m == 0 || n == 0) return 0;
-        const uint32_t tn = EPI != EPI_PLAIN ? (n / 2 + BN / 2 - 1) / (BN / 2) : (n + BN - 1) / BN;
+        uint32_t tn = EPI != EPI_PLAIN ? (n / 2 + BN / 2 - 1) / (BN / 2) : (n + BN - 1) / BN;
+        if (kCanNarrow && narrow && m <= 64u) tn = (n + BN / 2 - 1) / (BN / 2);
         return ((m + BM - 1) / BM) * tn;
     };
 
@@ -498,6 +504,19 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         } else {
             for (uint32_t e = tid; e < E; e += NT) s_order[e] = (uint16_t)e;
         }
+        __syncthreads();
+    }
+
+    if constexpr (kCanNarrow) {
+        // tiles of the launch at full width; every thread adds up its groups, the workgroup votes on the total
+        uint32_t mine = 0;
+        for (uint32_t e = tid; e < E; e += NT) mine += tiles_of(group_m(e), group_n(e));
+        uint32_t* const total = reinterpret_cast<uint32_t*>(s_a0);
+        if (tid == 0) *total = 0;
+        __syncthreads();
+        if (mine) atomicAdd(total, mine);
+        __syncthreads();
+        narrow = uniform(*total) * 2u <= gridDim.x;
         __syncthreads();
     }
 
@@ -575,7 +594,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     // Everything that identifies one output tile; the same in every lane.
     struct Tile {
         bool valid, fast;
-        uint32_t Me, Ne, Ke, n_span, m0, n0;
+        uint32_t Me, Ne, Ke, n_span, m0, n0, n_lim;  // n_lim: first column past the tile (its width is TN, or half)
         uint64_t off_a, off_b, off_d;
     };
     constexpr uint32_t TN = EPI != EPI_PLAIN ? BN / 2 : BN;  // columns of the tile grid one tile covers
@@ -601,7 +620,8 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         t.Ke = group_k(e);
         t.n_span = EPI != EPI_PLAIN ? t.Ne / 2 : t.Ne;  // columns the tile grid runs over
         const uint32_t tiles_m = (t.Me + BM - 1) / BM;
-        const uint32_t tiles_n = (t.n_span + TN - 1) / TN;
+        const uint32_t tile_n = (kCanNarrow && narrow && t.Me <= 64u) ? TN / 2 : TN;
+        const uint32_t tiles_n = (t.n_span + tile_n - 1) / tile_n;
         const uint32_t local = v - uniform(s_tile_start[pos]);
         const uint32_t band = kGroupM * tiles_n;
         const uint32_t first_m = (local / band) * kGroupM;
@@ -609,7 +629,8 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         const uint32_t mt = first_m + (local % band) % band_m;
         const uint32_t nt = (local % band) / band_m;
         t.m0 = mt * BM;
-        t.n0 = nt * TN;
+        t.n0 = nt * tile_n;
+        t.n_lim = t.n_span - t.n0 < tile_n ? t.n_span : t.n0 + tile_n;
         t.off_a = uniform(s_off_a[e]);
         t.off_b = uniform(s_off_b[e]);
         t.off_d = uniform(s_off_d[e]);
@@ -645,8 +666,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                 const uint32_t rows = t.n_span - t.n0 < (uint32_t)(BN / 2) ? t.n_span - t.n0 : (uint32_t)(BN / 2);
                 lk_b.setup(Be + (uint64_t)t.n0 * t.Ke, Be + (uint64_t)(t.n_span + t.n0) * t.Ke, rows, t.Ke, wave, lane);
             } else {
-                lk_b.setup(Be + (uint64_t)t.n0 * t.Ke, nullptr, t.Ne - t.n0 < (uint32_t)BN ? t.Ne - t.n0 : (uint32_t)BN,
-                           t.Ke, wave, lane);
+                lk_b.setup(Be + (uint64_t)t.n0 * t.Ke, nullptr, t.n_lim - t.n0, t.Ke, wave, lane);
             }
         } else {
             lt_b.setup(Be, t.Ne, t.Ke, t.n0, wave, lane);
@@ -686,7 +706,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     // epilogue of the previous tile, followed by exactly tile_stores stores
     bool prefetched = false;
     while (cur.valid) {
-        const uint32_t Me = cur.Me, Ne = cur.Ne, Ke = cur.Ke, n_span = cur.n_span, m0 = cur.m0, n0 = cur.n0;
+        const uint32_t Me = cur.Me, Ne = cur.Ne, Ke = cur.Ke, n_span = cur.n_span, m0 = cur.m0, n0 = cur.n0, n_lim = cur.n_lim;
         const uint64_t off_d = cur.off_d;
 
         if (!prefetched) {
@@ -786,7 +806,9 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         // rows of the group inside the tile, and inside this wavefront's WM rows of it in blocks of 32
         const uint32_t tile_rows = Me - m0 < (uint32_t)BM ? Me - m0 : (uint32_t)BM;
         const uint32_t wave_rows = tile_rows > wm * WM ? tile_rows - wm * WM : 0u;
-        const uint32_t row_blocks = uniform((wave_rows + 31u) / 32u);
+        // (a wavefront whose columns all lie past the end of the tile has nothing to compute either)
+        const bool has_columns = EPI != EPI_PLAIN || n0 + wn * WN < n_lim;
+        const uint32_t row_blocks = has_columns ? uniform((wave_rows + 31u) / 32u) : 0u;
         // A tile with at most 64 rows leaves three quarters of the A stages unused, and its K steps cost what the latency
         // of their loads costs. It runs a K loop of its own with a third LDS stage in that unused space (A rows 0..63 are
         // 8 KB; the B tile of stage 2 lies in two halves behind the A tiles of stages 0 and 1), so that two steps of
@@ -929,7 +951,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             const uint32_t rows_valid = row0 < Me ? (Me - row0 < (uint32_t)HM ? Me - row0 : (uint32_t)HM) : 0u;
             if constexpr (EPI == EPI_PLAIN) {
                 const uint32_t col0 = n0 + wn * WN;
-                const uint32_t cols_valid = col0 < Ne ? Ne - col0 : 0u;
+                const uint32_t cols_valid = col0 < n_lim ? n_lim - col0 : 0u;
 #pragma unroll
                 for (int i = 0; i < HF; ++i)
 #pragma unroll
