@@ -464,17 +464,19 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     auto group_m = [&](uint32_t e) { return m_arr[e]; };
     auto group_n = [&](uint32_t e) { return n_arr ? n_arr[e] : args.const_n; };
     auto group_k = [&](uint32_t e) { return k_arr ? k_arr[e] : args.const_k; };
-    // Column tiles of half the width for groups of at most 64 rows, when the launch would otherwise have tiles for no more
-    // than half of the workgroups (a few rows per group and a short N: the kernel is then a stream of the B operand, and
-    // twice as many workgroups stream it). Decided once per launch, below, from the group sizes; plain NT only.
-    constexpr bool kCanNarrow = EPI == EPI_PLAIN && A_KC && B_KC;
+    // Column tiles of half the width for groups of at most 64 rows (a few rows per group: the kernel is then a stream of
+    // the B operand), when that fills the workgroups better: a launch with tiles for at most half of them, or one made of
+    // such groups only whose last round of tiles would be at most half full. Decided once per launch, below, from the
+    // group sizes; NT only (a reduction-major B operand is loaded in rows of 256 columns whatever the tile's width).
+    constexpr bool kCanNarrow = A_KC && B_KC;
+    constexpr uint32_t kTileN = EPI != EPI_PLAIN ? BN / 2 : BN;  // columns of the tile grid one tile covers
     bool narrow = false;
     // n-extent covered by the tile grid: for the SwiGLU epilogue a tile spans 128 up + 128 gate columns
     auto tiles_of = [&](uint32_t m, uint32_t n) -> uint32_t {
         if (m == 0 || n == 0) return 0;
-        uint32_t tn = EPI != EPI_PLAIN ? (n / 2 + BN / 2 - 1) / (BN / 2) : (n + BN - 1) / BN;
-        if (kCanNarrow && narrow && m <= 64u) tn = (n + BN / 2 - 1) / (BN / 2);
-        return ((m + BM - 1) / BM) * tn;
+        const uint32_t span = EPI != EPI_PLAIN ? n / 2 : n;
+        const uint32_t width = (kCanNarrow && narrow && m <= 64u) ? kTileN / 2 : kTileN;
+        return ((m + BM - 1) / BM) * ((span + width - 1) / width);
     };
 
     // ---- order of the groups in the tile sequence: by K steps per tile, longest first ----
@@ -508,15 +510,23 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     }
 
     if constexpr (kCanNarrow) {
-        // tiles of the launch at full width; every thread adds up its groups, the workgroup votes on the total
-        uint32_t mine = 0;
-        for (uint32_t e = tid; e < E; e += NT) mine += tiles_of(group_m(e), group_n(e));
+        // tiles of the launch at full width, those of small groups apart; every thread adds up its groups
+        uint32_t mine_small = 0, mine_other = 0;
+        for (uint32_t e = tid; e < E; e += NT) {
+            const uint32_t m = group_m(e), t = tiles_of(m, group_n(e));
+            if (m <= 64u) mine_small += t;
+            else mine_other += t;
+        }
         uint32_t* const total = reinterpret_cast<uint32_t*>(s_a0);
-        if (tid == 0) *total = 0;
+        if (tid < 2) total[tid] = 0;
         __syncthreads();
-        if (mine) atomicAdd(total, mine);
+        if (mine_small) atomicAdd(total, mine_small);
+        if (mine_other) atomicAdd(total + 1, mine_other);
         __syncthreads();
-        narrow = uniform(*total) * 2u <= gridDim.x;
+        const uint32_t t_small = uniform(total[0]), t_other = uniform(total[1]), g = gridDim.x;
+        const uint32_t rounds = (t_small + t_other + g - 1) / g;  // as it is; at half width: half-cost rounds
+        const uint32_t half_rounds = (2 * t_small + g - 1) / g;
+        narrow = t_other == 0 ? half_rounds * 10u <= 2u * rounds * 9u : (t_small + t_other) * 2u <= g;
         __syncthreads();
     }
 
@@ -597,7 +607,6 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         uint32_t Me, Ne, Ke, n_span, m0, n0, n_lim;  // n_lim: first column past the tile (its width is TN, or half)
         uint64_t off_a, off_b, off_d;
     };
-    constexpr uint32_t TN = EPI != EPI_PLAIN ? BN / 2 : BN;  // columns of the tile grid one tile covers
     // Rounds of `grid` tiles are dealt in alternating directions (slot s takes tile s of even rounds and tile
     // grid-1-s of odd ones): when the tiles get cheaper along the tile order (groups with shrinking reduction length, as in
     // weight gradients under skewed routing) a workgroup that drew an expensive tile in one round draws a cheap one in the
@@ -620,7 +629,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         t.Ke = group_k(e);
         t.n_span = EPI != EPI_PLAIN ? t.Ne / 2 : t.Ne;  // columns the tile grid runs over
         const uint32_t tiles_m = (t.Me + BM - 1) / BM;
-        const uint32_t tile_n = (kCanNarrow && narrow && t.Me <= 64u) ? TN / 2 : TN;
+        const uint32_t tile_n = (kCanNarrow && narrow && t.Me <= 64u) ? kTileN / 2 : kTileN;
         const uint32_t tiles_n = (t.n_span + tile_n - 1) / tile_n;
         const uint32_t local = v - uniform(s_tile_start[pos]);
         const uint32_t band = kGroupM * tiles_n;
@@ -663,7 +672,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         if constexpr (B_KC) {
             if constexpr (EPI != EPI_PLAIN) {
                 // tile rows 0..127: "up" rows n0.. of the weight; rows 128..255: "gate" rows I + n0..
-                const uint32_t rows = t.n_span - t.n0 < (uint32_t)(BN / 2) ? t.n_span - t.n0 : (uint32_t)(BN / 2);
+                const uint32_t rows = t.n_lim - t.n0;
                 lk_b.setup(Be + (uint64_t)t.n0 * t.Ke, Be + (uint64_t)(t.n_span + t.n0) * t.Ke, rows, t.Ke, wave, lane);
             } else {
                 lk_b.setup(Be + (uint64_t)t.n0 * t.Ke, nullptr, t.n_lim - t.n0, t.Ke, wave, lane);
@@ -807,7 +816,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         const uint32_t tile_rows = Me - m0 < (uint32_t)BM ? Me - m0 : (uint32_t)BM;
         const uint32_t wave_rows = tile_rows > wm * WM ? tile_rows - wm * WM : 0u;
         // (a wavefront whose columns all lie past the end of the tile has nothing to compute either)
-        const bool has_columns = EPI != EPI_PLAIN || n0 + wn * WN < n_lim;
+        const bool has_columns = n0 + wn * (EPI != EPI_PLAIN ? WN / 2 : WN) < n_lim;
         const uint32_t row_blocks = has_columns ? uniform((wave_rows + 31u) / 32u) : 0u;
         // A tile with at most 64 rows leaves three quarters of the A stages unused, and its K steps cost what the latency
         // of their loads costs. It runs a K loop of its own with a third LDS stage in that unused space (A rows 0..63 are
@@ -970,7 +979,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                 constexpr int HB = WN * 2;  // bytes per staged row of h: 32 "up" columns | 32 "gate" columns
                 constexpr int YB = WN;      // bytes per staged row of the activation
                 const uint32_t col0 = n0 + wn * (WN / 2);
-                const uint32_t cols_valid = col0 < n_span ? n_span - col0 : 0u;
+                const uint32_t cols_valid = col0 < n_lim ? n_lim - col0 : 0u;
                 uint32_t ypack[HF][FN / 2][4][2];  // the packed activation waits here until h has left the staging slice
 #pragma unroll
                 for (int i = 0; i < HF; ++i)
