@@ -604,7 +604,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     // Everything that identifies one output tile; the same in every lane.
     struct Tile {
         bool valid, fast;
-        uint32_t Me, Ne, Ke, n_span, m0, n0, n_lim;  // n_lim: first column past the tile (its width is TN, or half)
+        uint32_t Me, Ne, Ke, n_span, m0, n0, n_lim;  // n_lim: first column past the tile (kTileN columns wide, or half of that)
         uint64_t off_a, off_b, off_d;
     };
     // Rounds of `grid` tiles are dealt in alternating directions (slot s takes tile s of even rounds and tile
