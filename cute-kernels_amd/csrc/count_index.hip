@@ -10,7 +10,15 @@
 //
 // index construction: three small launches (per-chunk histogram, scan, placement). Chunks are contiguous
 // ranges of slots, so "expert-major, chunk-minor, slot order inside the chunk" is exactly the stable order.
+#include <mutex>
+
 #include "common.h"
+
+// Device-resident scratch of fma_moe_build_index_static (the per-chunk histograms of the counting sort), for callers
+// that cannot hand over a workspace. One copy per GPU, held until the process ends; host code never uses this name as
+// an address: static_scratch() below asks the runtime for the array's address on the current device.
+#define FMA_STATIC_INDEX_WORDS (1 << 20)
+static __device__ __align__(256) uint32_t scratch[FMA_STATIC_INDEX_WORDS];
 
 namespace fmahip {
 namespace {
@@ -334,6 +342,79 @@ __global__ __launch_bounds__(kIdxThreads) void index_place_kernel(const id_t* __
 
 inline uint32_t index_nchunks(int64_t R) { return (uint32_t)((R + kIdxChunk - 1) / kIdxChunk); }
 
+int check_build_index(const void* ids, int id_bytes, int64_t R, int64_t E, uint32_t* counts, uint32_t* offsets,
+                      int32_t* perm, int32_t* eid, int32_t* inv) {
+    FMA_REQUIRE(id_bytes == 4 || id_bytes == 8, FMA_ERR_BAD_DTYPE,
+                "moe_build_index: ids must be int32 or int64 (id_bytes=%d)", id_bytes);
+    FMA_REQUIRE(E >= 1, FMA_ERR_BAD_SIZE, "moe_build_index: E must be >= 1 (got %lld)", (long long)E);
+    FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "moe_build_index: E=%lld exceeds the limit %d",
+                (long long)E, FMA_MAX_GROUPS);
+    FMA_REQUIRE(R >= 0, FMA_ERR_BAD_SIZE, "moe_build_index: negative slot count %lld", (long long)R);
+    FMA_REQUIRE(R <= 0x7fffffffll, FMA_ERR_TOO_MANY_ELEMENTS, "moe_build_index: R=%lld exceeds 2^31-1", (long long)R);
+    FMA_REQUIRE(counts && offsets, FMA_ERR_NULL_POINTER, "moe_build_index: counts/offsets is NULL");
+    FMA_REQUIRE(R == 0 || (ids && perm && eid && inv), FMA_ERR_NULL_POINTER,
+                "moe_build_index: ids/perm/eid/inv is NULL");
+    return FMA_OK;
+}
+
+// the three launches of the counting sort; hist: nchunks * E words of scratch (every word is written before it is read)
+int launch_build_index(const void* ids, int id_bytes, int64_t R, int64_t E, uint32_t* counts, uint32_t* offsets,
+                       int32_t* perm, int32_t* eid, int32_t* inv, uint32_t* hist, hipStream_t st) {
+    const uint32_t nchunks = index_nchunks(R);
+    const uint32_t blocks = (nchunks + kIdxWaves - 1) / kIdxWaves;
+    const size_t lds_bytes = (size_t)kIdxWaves * E * 4;
+    uint32_t nbits = 0;
+    while ((1ll << nbits) < E) ++nbits;
+
+    if (nchunks > 0) {
+        if (id_bytes == 4)
+            hipLaunchKernelGGL(index_hist_kernel<int32_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
+                               (const int32_t*)ids, R, (uint32_t)E, nchunks, hist);
+        else
+            hipLaunchKernelGGL(index_hist_kernel<int64_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
+                               (const int64_t*)ids, R, (uint32_t)E, nchunks, hist);
+        int rc = launch_status("moe_build_index(hist)");
+        if (rc) return rc;
+    }
+    hipLaunchKernelGGL(index_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, (uint32_t)E, nchunks, hist, counts,
+                       offsets);
+    int rc = launch_status("moe_build_index(scan)");
+    if (rc) return rc;
+    if (nchunks > 0) {
+        if (id_bytes == 4)
+            hipLaunchKernelGGL(index_place_kernel<int32_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
+                               (const int32_t*)ids, R, (uint32_t)E, nbits, nchunks, hist, perm, eid, inv);
+        else
+            hipLaunchKernelGGL(index_place_kernel<int64_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
+                               (const int64_t*)ids, R, (uint32_t)E, nbits, nchunks, hist, perm, eid, inv);
+        rc = launch_status("moe_build_index(place)");
+    }
+    return rc;
+}
+
+// Address of `scratch` on the current device, looked up once per device (each GPU holds its own copy of the array at
+// its own address). Only this pointer is ever handed to kernels.
+constexpr int kMaxDevices = 64;
+int static_scratch(uint32_t** out) {
+    static std::mutex mu;
+    static uint32_t* ptrs[kMaxDevices] = {};
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return fail((int)err, "moe_build_index_static: hipGetDevice: %s", hipGetErrorString(err));
+    FMA_REQUIRE(dev >= 0 && dev < kMaxDevices, FMA_ERR_UNSUPPORTED, "moe_build_index_static: device index %d", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || !p)
+            return fail(err != hipSuccess ? (int)err : FMA_ERR_NULL_POINTER,
+                        "moe_build_index_static: hipGetSymbolAddress(scratch): %s", hipGetErrorString(err));
+        ptrs[dev] = (uint32_t*)p;
+    }
+    *out = ptrs[dev];
+    return FMA_OK;
+}
+
 }  // namespace
 }  // namespace fmahip
 
@@ -401,54 +482,33 @@ int fma_moe_build_index(const void* ids, int id_bytes, int64_t R, int64_t E, uin
                         int32_t* perm, int32_t* eid, int32_t* inv, void* workspace, int64_t workspace_bytes,
                         void* stream) {
     using namespace fmahip;
-    FMA_REQUIRE(id_bytes == 4 || id_bytes == 8, FMA_ERR_BAD_DTYPE,
-                "moe_build_index: ids must be int32 or int64 (id_bytes=%d)", id_bytes);
-    FMA_REQUIRE(E >= 1, FMA_ERR_BAD_SIZE, "moe_build_index: E must be >= 1 (got %lld)", (long long)E);
-    FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "moe_build_index: E=%lld exceeds the limit %d",
-                (long long)E, FMA_MAX_GROUPS);
-    FMA_REQUIRE(R >= 0, FMA_ERR_BAD_SIZE, "moe_build_index: negative slot count %lld", (long long)R);
-    FMA_REQUIRE(R <= 0x7fffffffll, FMA_ERR_TOO_MANY_ELEMENTS, "moe_build_index: R=%lld exceeds 2^31-1", (long long)R);
-    FMA_REQUIRE(counts && offsets, FMA_ERR_NULL_POINTER, "moe_build_index: counts/offsets is NULL");
-    FMA_REQUIRE(R == 0 || (ids && perm && eid && inv), FMA_ERR_NULL_POINTER,
-                "moe_build_index: ids/perm/eid/inv is NULL");
+    int rc = check_build_index(ids, id_bytes, R, E, counts, offsets, perm, eid, inv);
+    if (rc) return rc;
     FMA_REQUIRE(workspace != nullptr, FMA_ERR_NULL_POINTER, "moe_build_index: workspace is NULL");
     const int64_t need = fma_moe_build_index_workspace_bytes(R, E);
     FMA_REQUIRE(workspace_bytes >= need, FMA_ERR_WORKSPACE_TOO_SMALL,
                 "moe_build_index: workspace of %lld bytes is smaller than the %lld needed", (long long)workspace_bytes,
                 (long long)need);
+    return launch_build_index(ids, id_bytes, R, E, counts, offsets, perm, eid, inv, (uint32_t*)workspace,
+                              (hipStream_t)stream);
+}
 
-    hipStream_t st = (hipStream_t)stream;
-    const uint32_t nchunks = index_nchunks(R);
-    uint32_t* hist = (uint32_t*)workspace;
-    const uint32_t blocks = (nchunks + kIdxWaves - 1) / kIdxWaves;
-    const size_t lds_bytes = (size_t)kIdxWaves * E * 4;
-    uint32_t nbits = 0;
-    while ((1ll << nbits) < E) ++nbits;
+int64_t fma_moe_build_index_static_max_words(void) { return FMA_STATIC_INDEX_WORDS; }
 
-    if (nchunks > 0) {
-        if (id_bytes == 4)
-            hipLaunchKernelGGL(index_hist_kernel<int32_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
-                               (const int32_t*)ids, R, (uint32_t)E, nchunks, hist);
-        else
-            hipLaunchKernelGGL(index_hist_kernel<int64_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
-                               (const int64_t*)ids, R, (uint32_t)E, nchunks, hist);
-        int rc = launch_status("moe_build_index(hist)");
-        if (rc) return rc;
-    }
-    hipLaunchKernelGGL(index_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, (uint32_t)E, nchunks, hist, counts,
-                       offsets);
-    int rc = launch_status("moe_build_index(scan)");
+int fma_moe_build_index_static(const void* ids, int id_bytes, int64_t R, int64_t E, uint32_t* counts, uint32_t* offsets,
+                               int32_t* perm, int32_t* eid, int32_t* inv, void* stream) {
+    using namespace fmahip;
+    int rc = check_build_index(ids, id_bytes, R, E, counts, offsets, perm, eid, inv);
     if (rc) return rc;
-    if (nchunks > 0) {
-        if (id_bytes == 4)
-            hipLaunchKernelGGL(index_place_kernel<int32_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
-                               (const int32_t*)ids, R, (uint32_t)E, nbits, nchunks, hist, perm, eid, inv);
-        else
-            hipLaunchKernelGGL(index_place_kernel<int64_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
-                               (const int64_t*)ids, R, (uint32_t)E, nbits, nchunks, hist, perm, eid, inv);
-        rc = launch_status("moe_build_index(place)");
-    }
-    return rc;
+    const int64_t need = fma_moe_build_index_workspace_bytes(R, E);
+    FMA_REQUIRE(need <= (int64_t)FMA_STATIC_INDEX_WORDS * 4, FMA_ERR_WORKSPACE_TOO_SMALL,
+                "moe_build_index_static: R=%lld slots with E=%lld experts need %lld bytes of scratch, the built-in "
+                "array holds %lld (use fma_moe_build_index with a workspace)",
+                (long long)R, (long long)E, (long long)need, (long long)FMA_STATIC_INDEX_WORDS * 4);
+    uint32_t* hist = nullptr;
+    rc = static_scratch(&hist);
+    if (rc) return rc;
+    return launch_build_index(ids, id_bytes, R, E, counts, offsets, perm, eid, inv, hist, (hipStream_t)stream);
 }
 
 }  // extern "C"

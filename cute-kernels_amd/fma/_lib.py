@@ -35,6 +35,8 @@ SIGNATURES = {
     "fma_continuous_count": (_i32, [_p, _i32, _i64, _p, _i64, _p, _i64, _p]),
     "fma_moe_build_index_workspace_bytes": (_i64, [_i64, _i64]),
     "fma_moe_build_index": (_i32, [_p, _i32, _i64, _i64, _p, _p, _p, _p, _p, _p, _i64, _p]),
+    "fma_moe_build_index_static_max_words": (_i64, []),
+    "fma_moe_build_index_static": (_i32, [_p, _i32, _i64, _i64, _p, _p, _p, _p, _p, _p]),
     "fma_gather_rows": (_i32, [_p, _p, _i64, _i64, _i32, _p, _i32, _p]),
     "fma_dispatch_rows": (_i32, [_p, _p, _i64, _i64, _i64, _p, _i32, _p]),
     "fma_combine": (_i32, [_p, _p, _p, _i64, _i64, _i64, _p, _i32, _p]),

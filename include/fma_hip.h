@@ -94,6 +94,19 @@ int fma_moe_build_index(const void* ids, int id_bytes, int64_t R, int64_t E, uin
                         uint32_t* offsets, int32_t* perm, int32_t* eid, int32_t* inv, void* workspace,
                         int64_t workspace_bytes, void* stream);
 
+/* Words (uint32) of the built-in scratch array of fma_moe_build_index_static: it serves calls with
+ * fma_moe_build_index_workspace_bytes(R, E) <= 4 * this value. */
+int64_t fma_moe_build_index_static_max_words(void);
+
+/* fma_moe_build_index without a workspace argument and without any allocation: the per-chunk histograms live in a
+ * fixed array in device memory that is part of the library image (4 MiB per GPU, held until the process ends), whose
+ * address is looked up once per device. Same outputs, bit for bit. No counterpart in the reference: it is for callers
+ * that cannot allocate or size a workspace (code under HIP graph capture, serving loops, harnesses that forbid
+ * hipMalloc). Rejects sizes whose scratch exceeds the array (FMA_ERR_WORKSPACE_TOO_SMALL; R * E up to about 5e8).
+ * All calls on one GPU share the array: calls that overlap in time on one GPU (different streams) race. */
+int fma_moe_build_index_static(const void* ids, int id_bytes, int64_t R, int64_t E, uint32_t* counts,
+                               uint32_t* offsets, int32_t* perm, int32_t* eid, int32_t* inv, void* stream);
+
 /* ---- row movement ------------------------------------------------------------------------- */
 
 /* out[i, :] = x[idx[i] / divisor, :] for i < R (rows of H elements; the four row kernels move 16 bytes per lane when
