@@ -25,23 +25,11 @@
 //  * The MFMA is issued with B as the first operand, so a lane ends up holding four consecutive output
 //    columns of one output row. The epilogue transposes the wavefront's sub-tile through LDS (stage 1) and stores
 //    whole 128-byte row segments; the next tile's first loads are already on their way into stage 0 by then.
-#include <type_traits>
-
-#include "common.h"
+#include "gemm_parts.h"
 #include "grouped_gemm_f32.h"
 
 namespace fmahip {
 namespace gemm {
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-typedef __attribute__((ext_vector_type(2))) float f32x2;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-typedef __attribute__((ext_vector_type(4))) short s16x4;
-typedef __attribute__((ext_vector_type(8))) short s16x8;
-typedef __attribute__((address_space(3))) void lds_void;
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
-typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
 constexpr int BM = 256;
 constexpr int BN = 256;
@@ -51,20 +39,36 @@ constexpr int kTRowBytes = BM * 2;          // 512: row of a [64 k][256 out] til
 constexpr int kTileBytes = BM * kRowBytes;  // 32 KB per operand per stage, either layout
 constexpr int kGroupM = 8;                  // m-tiles that share one column sweep of the tile order
 constexpr int kXcds = 8;
+// how the load instructions of a K step are spread over the slices after the barrier that frees their stage
+#ifndef FMA_PF_DIST
+#define FMA_PF_DIST 4
+#endif
+constexpr uint32_t kPfDist = FMA_PF_DIST;  // K steps between a line's prefetch and the step that loads it
+#ifndef FMA_LD_S3
+#define FMA_LD_S3 8
+#define FMA_LD_S0 0
+#define FMA_LD_S1 0
+#define FMA_LD_S2 0
+#endif
 
-constexpr int EPI_PLAIN = 0;
-constexpr int EPI_SWIGLU = 1;      // stores the rounded pre-activation h and the activation
-constexpr int EPI_SWIGLU_ACT = 2;  // the activation only (a forward pass that no backward follows)
+
+#ifdef FMA_PROF
+// timing instrumentation of a diagnostic build: per (workgroup, wavefront): cycles waiting for loads, cycles in the
+// barrier, K steps, cycles in the kernel, cycles at the tile boundary (epilogue + next tile's set-up)
+__device__ unsigned long long fma_prof[2 * 1024 * 8 * 8];
+#define PROF_STAMP(t) asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t))
+#endif
 
 struct GemmArgs {
     const uint16_t* A;
     const uint16_t* B;
     uint16_t* D;    // plain: output; swiglu: pre-activation h (may be NULL)
     uint16_t* ACT;  // swiglu only: activation output
-    const uint32_t* M_arr;
+    const uint32_t* M_arr;  // NULL: every group uses const_m
     const uint32_t* N_arr;  // NULL: every group uses const_n
     const uint32_t* K_arr;  // NULL: every group uses const_k
     uint32_t E;
+    uint32_t const_m;
     uint32_t const_n;
     uint32_t const_k;
     float alpha;
@@ -86,77 +90,6 @@ __device__ __forceinline__ uint32_t mc_frag_off(uint32_t r0, uint32_t lane) {
     const uint32_t chunk = (r0 >> 3) + 2u * (g & 1u) + (q >> 1);
     return (8u * (g >> 1) + kr) * kTRowBytes + ((chunk ^ (4u * kr)) << 4) + (q & 1u) * 8u;
 }
-
-// ---- the two 16-bit element types: conversions and the matrix instruction ------------------------------------------
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
-typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
-
-struct ElemBf16 {
-    using frag = bf16x8;
-    using act_t = bf16_t;  // selects the activation's arithmetic (the one swiglu_forward uses for this dtype)
-    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {  // round to nearest even, lo in the low half
-        f32x2 f = {lo, hi};
-        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
-    }
-    static __device__ __forceinline__ float round(float x) { return (float)(__bf16)x; }
-    static __device__ __forceinline__ float from_bits(uint16_t b) { return bf16_bits_to_float(b); }
-    static __device__ __forceinline__ f32x16 mfma(frag a, frag b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-    }
-};
-
-struct ElemF16 {
-    using frag = f16x8;
-    using act_t = f16_t;
-    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-        f32x2 f = {lo, hi};
-        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
-    }
-    static __device__ __forceinline__ float round(float x) { return (float)(_Float16)x; }
-    static __device__ __forceinline__ float from_bits(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
-    static __device__ __forceinline__ f32x16 mfma(frag a, frag b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-    }
-};
-
-// ---- direct global -> LDS loaders ---------------------------------------------------------------------------------
-// Every load is a buffer load to LDS (buffer_load_dwordx4 ... lds): the address is a 128-bit buffer descriptor held in
-// scalar registers plus one per-lane byte offset that stays the same for the whole tile plus a scalar offset per
-// instruction, so the K loop spends no vector instructions or registers on addresses. The descriptor's size field does
-// the edge handling: a dword whose offset (lane + scalar part) is not below it is not read and lands in LDS as zero.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const uint16_t* p, uint32_t bytes) {
-    // stride 0 (raw buffer), 32-bit data format
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, (int)bytes, 0x00020000);
-}
-// The same load written in assembly, with its M0 set-up (M0 holds the LDS address the wavefront's 1 KB goes to). The
-// compiler does not see that it writes LDS, so it places no waits of its own for it: the first loads of a tile are
-// issued this way, partly while the previous tile's epilogue is still running, and waited for with an exact count.
-__device__ __forceinline__ void buffer_load_lds_quiet(u32x4 rsrc, uint32_t voff, uint32_t soff, uint32_t lds_addr) {
-    // M0 is put back afterwards: the compiler keeps its own values in it and does not honour a clobber of it
-    uint32_t saved_m0;
-    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
-                 "s_mov_b32 m0, %0"
-                 : "=&s"(saved_m0)
-                 : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr));
-}
-__device__ __forceinline__ uint32_t lds_address(const uint8_t* p) {
-    return (uint32_t)(uintptr_t)(lds_void*)const_cast<uint8_t*>(p);
-}
-// the descriptor make_rsrc() builds, as four plain words in scalar registers (p and bytes are the same in every lane)
-__device__ __forceinline__ u32x4 make_rsrc_words(const uint16_t* p, uint32_t bytes) {
-    const uint64_t a = (uint64_t)(uintptr_t)p;
-    u32x4 r;
-    r.x = (uint32_t)a;
-    r.y = (uint32_t)(a >> 32) & 0xffffu;
-    r.z = bytes;
-    r.w = 0x00020000u;
-    return r;
-}
-__device__ __forceinline__ uint32_t uniform(uint32_t x) { return __builtin_amdgcn_readfirstlane(x); }
-__device__ __forceinline__ uint64_t uniform(uint64_t x) {
-    return ((uint64_t)uniform((uint32_t)(x >> 32)) << 32) | uniform((uint32_t)x);
-}
-constexpr uint32_t kOutOfRange = 0x80000000u;  // lane offset no descriptor of this kernel reaches (sizes stay < 2^31)
 
 // Operand with the reduction dimension contiguous: tile [256 rows][64 k]. A wavefront instruction moves 8 physical rows
 // (1 KB); NI instructions per wavefront and K step. SPLIT: tile rows 128..255 come from a second row range (base1).
@@ -188,14 +121,17 @@ struct LoaderK {
         voff = r * ldb + chunk * 16u;
     }
 
-    __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0) const {
+    __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0) const { issue_range<0, NI>(tile, k0); }
+    // instructions I0 .. I1-1 of the K step at k0
+    template <int I0, int I1>
+    __device__ __forceinline__ void issue_range(uint8_t* tile, uint32_t k0) const {
         uint32_t v = voff;
         // last, partial K step: chunks past the end of K are pushed out of range, which zero-fills them
         if (k0 + BK > kdim && k0 + chunk * 8u >= kdim) v = kOutOfRange;
         const __amdgpu_buffer_rsrc_t r0 = make_rsrc(base0, bytes);
         const __amdgpu_buffer_rsrc_t r1 = make_rsrc(SPLIT ? base1 : base0, bytes);
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
+        for (int i = I0; i < I1; ++i) {
             const bool second = SPLIT && i >= NI / 2;
             const uint32_t row = (uint32_t)(second ? i - NI / 2 : i) * kRowsPerInst;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(second ? r1 : r0, (lds_void*)(tile + (i * NW + wave) * 1024), 16, v,
@@ -263,12 +199,14 @@ struct LoaderT {
         voff = khalf * ldb + (((lane & 31u) ^ (4u * (krow & 3u))) << 4);
     }
 
-    __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0) const {
+    __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0) const { issue_range<0, NI>(tile, k0); }
+    template <int I0, int I1>
+    __device__ __forceinline__ void issue_range(uint8_t* tile, uint32_t k0) const {
         // rows of this K step that exist (none at all when the step lies past the end: everything is zero-filled)
         const uint32_t rows = k0 >= kdim ? 0u : (kdim - k0 < (uint32_t)BK ? kdim - k0 : (uint32_t)BK);
         const __amdgpu_buffer_rsrc_t r = make_rsrc(base + (uint64_t)k0 * (ldb / 2u), rows ? rows * ldb - col_bytes : 0u);
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
+        for (int i = I0; i < I1; ++i) {
             __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(tile + (i * NW + wave) * 1024), 16, voff,
                                                      (uint32_t)(i * NW + wave) * 2u * ldb, 0, 0);
         }
@@ -294,139 +232,12 @@ struct LoaderT {
     }
 };
 
-__device__ __forceinline__ s16x8 read_kc_frag(const uint8_t* p) { return *reinterpret_cast<const s16x8*>(p); }
-
 __device__ __forceinline__ s16x8 read_tr_frag(const uint8_t* p) {
     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p);
     const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p + 4 * kTRowBytes));
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-// ---- epilogue staging: a wavefront transposes its accumulator sub-tile, half at a time, through 8 KB of LDS ----
-// The MFMA leaves a lane with 4 consecutive columns of one row per 32x32 block, so storing straight from registers
-// writes 8-byte pieces of 32 different rows per instruction. Staged through LDS as rows of ROWB bytes, every store
-// instruction writes 16 bytes per lane and whole 64- or 128-byte row segments.
-// Row m, 16-byte chunk c of the image sits at m*ROWB + ((c ^ key(m)) << 4), key(m) = (m / rows-per-256-B) mod chunks:
-// the 8-byte writes of 32 consecutive rows conflict at most two ways, the 16-byte reads not at all.
-
-// 16-byte buffer store of a staged piece. A lane whose offset is not below the descriptor's size stores nothing, so
-// every lane always executes the instruction: the number of stores a wavefront issues per tile is a compile-time
-// constant, which the wait for the next tile's first loads relies on.
-// NT = the non-temporal hint: the output tile is not read again by this kernel, and a workgroup's 128 KB of results
-// should not push operand panels out of the L2 (measured: +0.5 to +1.5 points of peak over plain stores). Only where a
-// store instruction covers whole 128-byte lines: streamed 64-byte pieces are not merged in the L2 and cost a
-// read-modify-write each (measured on the SwiGLU epilogue: +35 % fetched and +28 % written bytes).
-template <bool NT>
-__device__ __forceinline__ void store_tile16(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint4 v) {
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc, (int)voff, 0, NT ? 2 : 0);
-}
-template <int ROWB>
-__device__ __forceinline__ uint32_t stage_off(uint32_t m, uint32_t chunk16) {
-    constexpr uint32_t kChunks = ROWB / 16;
-    constexpr uint32_t kRowsPer256 = 256 / ROWB;
-    return m * ROWB + ((chunk16 ^ ((m / kRowsPer256) & (kChunks - 1))) << 4);
-}
-// A wavefront's staging slice is made of the 1 KB pieces of LDS stage 1 that the wavefront itself fills when it loads
-// operands (pieces wave, wave + NW, ... of the A array, then of the B array), so only its own loads ever overwrite its
-// image and no workgroup barrier is needed between an epilogue and the next tile's loads into stage 1.
-template <int NW>
-struct StagingSlice {
-    uint8_t* a;  // LDS stage 1, A array, this wavefront's first piece
-    uint8_t* b;  // the same of the B array
-    __device__ __forceinline__ uint8_t* at(uint32_t off) const {  // byte `off` of the image
-        constexpr uint32_t kPieces = 32 / NW;                    // pieces per array
-        const uint32_t piece = off >> 10;
-        return (piece < kPieces ? a : b) + (piece % kPieces) * (uint32_t)(NW * 1024) + (off & 1023u);
-    }
-};
-// lane's 4 columns [col, col+4) of image row m
-template <int ROWB, typename Slice>
-__device__ __forceinline__ void stage_put(const Slice& img, uint32_t m, uint32_t col, uint2 v) {
-    *reinterpret_cast<uint2*>(img.at(stage_off<ROWB>(m, col >> 3) + ((col >> 2) & 1u) * 8u)) = v;
-}
-// Stores the image (ROWS rows of ROWB/2 columns) to origin[r * ld + c]; only the first rows_valid rows and cols_valid
-// columns exist in the output (both may be 0). ld and cols_valid are multiples of 8 elements, so every 16-byte piece
-// is wholly inside or outside. Issues exactly ROWS * ROWB / 1024 store instructions.
-template <int ROWB, int ROWS, typename Slice>
-__device__ __forceinline__ void stage_flush(const Slice& img, uint16_t* origin, uint32_t ld, uint32_t rows_valid,
-                                            uint32_t cols_valid, uint32_t lane) {
-    constexpr uint32_t kChunks = ROWB / 16;  // 16-byte pieces per image row
-    constexpr uint32_t kRowsPerInst = 64 / kChunks;
-    const uint32_t c16 = lane % kChunks;
-    const uint32_t ldb = ld * 2u;
-    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(origin, rows_valid * ldb);
-    const bool col_ok = c16 * 8u < cols_valid;
-#pragma unroll
-    for (uint32_t it = 0; it < ROWS / kRowsPerInst; ++it) {
-        const uint32_t r = it * kRowsPerInst + lane / kChunks;
-        const uint4 v = *reinterpret_cast<const uint4*>(img.at(stage_off<ROWB>(r, c16)));
-        store_tile16<(ROWB >= 128)>(rsrc, col_ok ? r * ldb + c16 * 16u : kOutOfRange, v);
-    }
-}
-
-// Like stage_flush for an image whose row holds two windows of HALF columns each: window 0 goes to columns 0.. of the
-// origin's row, window 1 to columns second0.. of the same row (the "up" and "gate" halves of h).
-template <int ROWB, int ROWS, int HALF, typename Slice>
-__device__ __forceinline__ void stage_flush_split(const Slice& img, uint16_t* origin, uint32_t ld, uint32_t rows_valid,
-                                                  uint32_t cols_valid, uint32_t second0, uint32_t lane) {
-    constexpr uint32_t kChunks = ROWB / 16;
-    constexpr uint32_t kRowsPerInst = 64 / kChunks;
-    const uint32_t c16 = lane % kChunks;
-    const uint32_t in_window = (c16 * 8u) % HALF;
-    const uint32_t window = (c16 * 8u) / HALF;
-    const uint32_t ldb = ld * 2u;
-    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(origin, rows_valid * ldb);
-    const bool col_ok = in_window < cols_valid;
-#pragma unroll
-    for (uint32_t it = 0; it < ROWS / kRowsPerInst; ++it) {
-        const uint32_t r = it * kRowsPerInst + lane / kChunks;
-        const uint4 v = *reinterpret_cast<const uint4*>(img.at(stage_off<ROWB>(r, c16)));
-        store_tile16<(HALF * 2 >= 128)>(rsrc, col_ok ? r * ldb + (window * second0 + in_window) * 2u : kOutOfRange, v);
-    }
-}
-
-// Scheduling hint for one k slice: MFMAS matrix instructions with READS LDS reads spread evenly between them.
-template <int R, int MFMAS, int READS>
-__device__ __forceinline__ void interleave_mfma_lds() {
-    constexpr int kPairs = READS < MFMAS ? READS : MFMAS;
-    constexpr int kPer = READS / kPairs;           // LDS reads after each of the first kPairs MFMAs
-    constexpr int kExtra = READS - kPairs * kPer;  // the first kExtra of them get one more
-    if constexpr (R < kPairs) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, kPer + (R < kExtra ? 1 : 0), 0);
-        interleave_mfma_lds<R + 1, MFMAS, READS>();
-    } else if constexpr (MFMAS - kPairs > 0) {
-        __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - kPairs, 0);
-    }
-}
-
-// Scheduling hint: MFMAS matrix instructions with LOADS buffer loads placed one after each of the first MFMAs.
-template <int R, int MFMAS, int LOADS>
-__device__ __forceinline__ void spread_mfma_vmem() {
-    if constexpr (R < MFMAS) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        if constexpr (R < LOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        spread_mfma_vmem<R + 1, MFMAS, LOADS>();
-    }
-}
-
-// Slow, layout-agnostic path for a group whose contiguous dimensions are not multiples of 8 elements.
-template <typename EL, bool A_KC, bool B_KC>
-__device__ void scalar_tile(const uint16_t* Ae, const uint16_t* Be, uint16_t* De, uint32_t Me, uint32_t Ne,
-                            uint32_t Ke, uint32_t m0, uint32_t n0, float alpha, uint32_t nthreads) {
-    for (uint32_t idx = threadIdx.x; idx < (uint32_t)(BM * BN); idx += nthreads) {
-        const uint32_t m = m0 + idx / BN;
-        const uint32_t n = n0 + idx % BN;
-        if (m >= Me || n >= Ne) continue;
-        float acc = 0.0f;
-        for (uint32_t k = 0; k < Ke; ++k) {
-            const uint16_t a = A_KC ? Ae[(uint64_t)m * Ke + k] : Ae[(uint64_t)k * Me + m];
-            const uint16_t b = B_KC ? Be[(uint64_t)n * Ke + k] : Be[(uint64_t)k * Ne + n];
-            acc = fmaf(EL::from_bits(a), EL::from_bits(b), acc);
-        }
-        De[(uint64_t)m * Ne + n] = (uint16_t)(EL::pack2(alpha * acc, 0.0f) & 0xffffu);
-    }
-}
 
 template <typename EL, int NWM, int NWN, bool A_KC, bool B_KC, int EPI>
 __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmArgs args) {
@@ -444,6 +255,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     __shared__ __attribute__((aligned(1024))) uint8_t s_b0[kTileBytes];
     __shared__ __attribute__((aligned(1024))) uint8_t s_a1[kTileBytes];
     __shared__ __attribute__((aligned(1024))) uint8_t s_b1[kTileBytes];
+    __shared__ uint32_t s_pf[64];  // where the dwords fetched by the L2 prefetch end up (never read)
     __shared__ uint32_t s_tile_start[FMA_MAX_GROUPS + 1];  // first tile of the group at position p of the tile sequence
     __shared__ uint16_t s_order[FMA_MAX_GROUPS];           // which group that is
     __shared__ uint64_t s_off_a[FMA_MAX_GROUPS + 1];
@@ -461,7 +273,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     // load (nothing writes the arrays while the kernel runs), not a vector load that every tile would wait for.
     typedef const __attribute__((address_space(4))) uint32_t* const_u32_ptr;
     const const_u32_ptr m_arr = (const_u32_ptr)args.M_arr, n_arr = (const_u32_ptr)args.N_arr, k_arr = (const_u32_ptr)args.K_arr;
-    auto group_m = [&](uint32_t e) { return m_arr[e]; };
+    auto group_m = [&](uint32_t e) { return m_arr ? m_arr[e] : args.const_m; };
     auto group_n = [&](uint32_t e) { return n_arr ? n_arr[e] : args.const_n; };
     auto group_k = [&](uint32_t e) { return k_arr ? k_arr[e] : args.const_k; };
     // Column tiles of half the width for groups of at most 64 rows (a few rows per group: the kernel is then a stream of
@@ -606,6 +418,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         bool valid, fast;
         uint32_t Me, Ne, Ke, n_span, m0, n0, n_lim;  // n_lim: first column past the tile (kTileN columns wide, or half of that)
         uint64_t off_a, off_b, off_d;
+        uint32_t pf_r, pf_c;  // position of the tile in its XCD's 8 x 4 block of tiles (row, column)
     };
     // Rounds of `grid` tiles are dealt in alternating directions (slot s takes tile s of even rounds and tile
     // grid-1-s of odd ones): when the tiles get cheaper along the tile order (groups with shrinking reduction length, as in
@@ -637,6 +450,8 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         const uint32_t band_m = tiles_m - first_m < (uint32_t)kGroupM ? tiles_m - first_m : (uint32_t)kGroupM;
         const uint32_t mt = first_m + (local % band) % band_m;
         const uint32_t nt = (local % band) / band_m;
+        t.pf_r = (local % band) % band_m;
+        t.pf_c = nt & 3u;
         t.m0 = mt * BM;
         t.n0 = nt * tile_n;
         t.n_lim = t.n_span - t.n0 < tile_n ? t.n_span : t.n0 + tile_n;
@@ -681,19 +496,98 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             lt_b.setup(Be, t.Ne, t.Ke, t.n0, wave, lane);
         }
     };
+    // ---- L2 prefetch by designated workgroups ----
+    // The 32 workgroups of an XCD work on an 8 x 4 block of tiles: an A panel is shared by the 4 tiles of a block row, a
+    // B panel by the 8 tiles of a block column, and whichever workgroup asks for a 128-byte line first waits for it to
+    // come from beyond the L2 while the K step's window is one step long. Every workgroup therefore requests, kPfDist K
+    // steps ahead, its share of the lines its block neighbours will load (a quarter of its A tile's lines, an eighth of
+    // its B tile's): one 4-byte load per line and one instruction per wavefront and K step (even wavefronts: A, 16
+    // lanes each; odd ones: B, 8 lanes each; the other lanes are out of the descriptor's range and fetch nothing).
+    uint32_t pf_voff = kOutOfRange;
+    const uint16_t* pf_base = nullptr;
+    uint32_t pf_bytes = 0, pf_ldb = 0, pf_col_bytes = 0, pf_kdim = 0;
+    const bool pf_is_b = (wave & 1u) != 0;
+    const bool pf_t = pf_is_b ? !B_KC : !A_KC;  // reduction-major operand: the descriptor moves with the K step
+    auto setup_prefetch = [&](const Tile& t) {
+        const uint32_t p = wave >> 1;  // 0..3 among the wavefronts that serve the same operand
+        if (!pf_is_b) {
+            const uint32_t i = p * 16u + lane;  // 64 lines of the A tile's 256
+            if constexpr (A_KC) {
+                pf_base = lk_a.base0; pf_bytes = lk_a.bytes;
+                pf_voff = lane < 16u ? (4u * i + t.pf_c) * lk_a.ldb : kOutOfRange;
+            } else {
+                pf_base = lt_a.base; pf_ldb = lt_a.ldb; pf_col_bytes = lt_a.col_bytes; pf_kdim = lt_a.kdim;
+                pf_voff = lane < 16u ? i * lt_a.ldb + t.pf_c * 128u : kOutOfRange;
+            }
+        } else {
+            if constexpr (B_KC) {
+                pf_bytes = lk_b.bytes;
+                if constexpr (EPI != EPI_PLAIN) {
+                    pf_base = (p >> 1) ? lk_b.base1 : lk_b.base0;  // "up" rows, "gate" rows
+                    pf_voff = lane < 8u ? (8u * ((p & 1u) * 8u + lane) + t.pf_r) * lk_b.ldb : kOutOfRange;
+                } else {
+                    pf_base = lk_b.base0;
+                    pf_voff = lane < 8u ? (8u * (p * 8u + lane) + t.pf_r) * lk_b.ldb : kOutOfRange;
+                }
+            } else {
+                pf_base = lt_b.base; pf_ldb = lt_b.ldb; pf_col_bytes = lt_b.col_bytes; pf_kdim = lt_b.kdim;
+                pf_voff = lane < 8u ? (2u * (p * 8u + lane) + (t.pf_r >> 2)) * lt_b.ldb + (t.pf_r & 3u) * 128u : kOutOfRange;
+            }
+        }
+    };
+    // requests this wavefront's lines of K step `kstep` (any value: past the end of K it fetches nothing or a line of a
+    // later row, which is valid memory inside the descriptor's range)
+    // (measured on the Mixtral shapes: +1 point of peak where both operands have the same storage order; with one of
+    // each, where the two halves of the workgroup build different descriptors per step, -1.5: switched off there)
+    constexpr bool kPrefetch = A_KC == B_KC;
+    auto issue_prefetch = [&](uint32_t kstep) {
+        if constexpr (!kPrefetch) return;
+        const uint32_t k0 = kstep * (uint32_t)BK;
+        const uint32_t rows = k0 >= pf_kdim ? 0u : (pf_kdim - k0 < (uint32_t)BK ? pf_kdim - k0 : (uint32_t)BK);
+        const uint16_t* base = pf_t ? pf_base + (uint64_t)k0 * (pf_ldb / 2u) : pf_base;
+        const uint32_t bytes = pf_t ? (rows ? rows * pf_ldb - pf_col_bytes : 0u) : pf_bytes;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(make_rsrc(base, bytes), (lds_void*)s_pf, 4, pf_voff, pf_t ? 0u : k0 * 2u, 0, 0);
+    };
     // loads of the K step at k0 into `stage`: inside the K loop (compiler-visible, placed by the scheduling hints) ...
     auto issue = [&](int stage, uint32_t k0) {
+#if defined(FMA_DIAG) && FMA_DIAG == 4
+        return;
+#endif
         if constexpr (A_KC) lk_a.issue(stage ? s_a1 : s_a0, k0);
         else lt_a.issue(stage ? s_a1 : s_a0, k0);
+#if defined(FMA_DIAG) && FMA_DIAG == 3
+        return;
+#endif
         if constexpr (B_KC) lk_b.issue(stage ? s_b1 : s_b0, k0);
         else lt_b.issue(stage ? s_b1 : s_b0, k0);
     };
+    // load instructions FIRST .. FIRST+COUNT-1 of a K step (the A operand's come first)
+    auto issue_some = [&](auto first_c, auto count_c, int stage, uint32_t k0) {
+        constexpr int FIRST = decltype(first_c)::value, COUNT = decltype(count_c)::value;
+        constexpr int NI = 32 / NW;
+        constexpr int A0 = FIRST < NI ? FIRST : NI, A1 = FIRST + COUNT < NI ? FIRST + COUNT : NI;
+        constexpr int B0 = FIRST > NI ? FIRST - NI : 0, B1 = FIRST + COUNT > NI ? FIRST + COUNT - NI : 0;
+        if constexpr (A1 > A0) {
+            if constexpr (A_KC) lk_a.template issue_range<A0, A1>(stage ? s_a1 : s_a0, k0);
+            else lt_a.template issue_range<A0, A1>(stage ? s_a1 : s_a0, k0);
+        }
+        if constexpr (B1 > B0) {
+            if constexpr (B_KC) lk_b.template issue_range<B0, B1>(stage ? s_b1 : s_b0, k0);
+            else lt_b.template issue_range<B0, B1>(stage ? s_b1 : s_b0, k0);
+        }
+    };
     // ... and at the head of a tile
-    auto issue_quiet = [&](int stage, uint32_t k0) {
+    auto issue_quiet_a = [&](int stage, uint32_t k0) {
         if constexpr (A_KC) lk_a.issue_quiet(stage ? s_a1 : s_a0, k0);
         else lt_a.issue_quiet(stage ? s_a1 : s_a0, k0);
+    };
+    auto issue_quiet_b = [&](int stage, uint32_t k0) {
         if constexpr (B_KC) lk_b.issue_quiet(stage ? s_b1 : s_b0, k0);
         else lt_b.issue_quiet(stage ? s_b1 : s_b0, k0);
+    };
+    auto issue_quiet = [&](int stage, uint32_t k0) {
+        issue_quiet_a(stage, k0);
+        issue_quiet_b(stage, k0);
     };
     constexpr uint32_t kStepLoads = 2 * (32 / NW);  // load instructions per wavefront and K step
     // store instructions per wavefront and tile (stage_flush issues a fixed number)
@@ -709,11 +603,20 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         else __builtin_amdgcn_s_waitcnt(0x0f70);               // vmcnt(0)
     };
 
+#ifdef FMA_PROF
+    uint64_t prof_wait = 0, prof_bar = 0, prof_steps = 0, prof_start, prof_edge = 0, prof_e0 = 0;
+    uint64_t prof_seg[6] = {0, 0, 0, 0, 0, 0}, prof_t = 0;
+#define PROF_SEG(i) do { uint64_t t_; PROF_STAMP(t_); if (prof_e0) prof_seg[i] += t_ - prof_t; prof_t = t_; } while (0)
+    PROF_STAMP(prof_start);
+#endif
     uint32_t round = 0;
     Tile cur = lookup(0);
     // prefetched: the loaders are set up for `cur` and the loads of its first K step went out (into stage 0) before the
     // epilogue of the previous tile, followed by exactly tile_stores stores
     bool prefetched = false;
+    // prefetched_b1: the B operand of its second K step is on its way into stage 1 as well (the A half of stage 1 is the
+    // epilogue's staging space, so A's second step follows the epilogue)
+    bool prefetched_b1 = false;
     while (cur.valid) {
         const uint32_t Me = cur.Me, Ne = cur.Ne, Ke = cur.Ke, n_span = cur.n_span, m0 = cur.m0, n0 = cur.n0, n_lim = cur.n_lim;
         const uint64_t off_d = cur.off_d;
@@ -721,13 +624,14 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         if (!prefetched) {
             if (!cur.fast) {
                 if constexpr (EPI == EPI_PLAIN) {
-                    scalar_tile<EL, A_KC, B_KC>(args.A + cur.off_a, args.B + cur.off_b, args.D + off_d, Me, Ne, Ke, m0, n0,
+                    scalar_tile<EL, A_KC, B_KC, BM, BN>(args.A + cur.off_a, args.B + cur.off_b, args.D + off_d, Me, Ne, Ke, m0, n0,
                                                 args.alpha, NT);
                 }
                 cur = lookup(++round);
                 continue;
             }
             setup_loaders(cur);
+            setup_prefetch(cur);
         }
         f32x16 acc[FM][FN];
 #pragma unroll
@@ -751,11 +655,17 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                 const uint8_t* tb = stage ? s_b1 : s_b0;
 #pragma unroll
                 for (int i = 0; i < FA; ++i) {
+#if defined(FMA_DIAG) && (FMA_DIAG == 1 || FMA_DIAG == 2)
+                    if (ks & (FMA_DIAG == 1 ? 1 : 3)) { fa[buf][i] = fa[buf ^ 1][i]; continue; }
+#endif
                     if constexpr (A_KC) fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_kc_frag(ta + a_off[i] + kc_slice[ks]));
                     else fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_tr_frag(ta + a_off[i] + ks * 16 * kTRowBytes));
                 }
 #pragma unroll
                 for (int j = 0; j < FN; ++j) {
+#if defined(FMA_DIAG) && FMA_DIAG == 2
+                    if (ks & 3) { fb[buf][j] = fb[buf ^ 1][j]; continue; }
+#endif
                     if constexpr (B_KC) fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_kc_frag(tb + b_off[j] + kc_slice[ks]));
                     else fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_tr_frag(tb + b_off[j] + ks * 16 * kTRowBytes));
                 }
@@ -781,32 +691,74 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         // k slice and the MFMAs of that slice: once it is passed, the stage just read is free (the loads of step kt+2
         // are issued into it) and the other stage is complete (its first fragments are fetched), and both overlap
         // with the MFMAs still to be issued, so the matrix pipe has work while the barrier's latencies play out.
+        // The 2*(32/NW) loads of a K step are spread over the four slices that follow the barrier which frees their stage:
+        // kLd3 of them in the last slice of the step that frees it, kLd0 / kLd1 / kLd2 in slices 0 / 1 / 2 of the next step.
+        // A burst right after the barrier fills the address unit's queue; the wavefronts then block at a load with their
+        // matrix instructions behind it.
         auto step = [&](auto fa_c, int stage, uint32_t kt) {
             constexpr int FA = decltype(fa_c)::value;
+            constexpr int kReads = (A_KC ? FA : 2 * FA) + (B_KC ? FN : 2 * FN);
+            using L3 = std::integral_constant<int, FMA_LD_S3>;
+            using L0 = std::integral_constant<int, FMA_LD_S0>;
+            using L1 = std::integral_constant<int, FMA_LD_S1>;
+            using L2 = std::integral_constant<int, FMA_LD_S2>;
+            static_assert(FMA_LD_S3 + FMA_LD_S0 + FMA_LD_S1 + FMA_LD_S2 == 2 * (32 / NW), "every load of a step is issued once");
             load_frags(fa_c, stage, 1, 1);
+            issue_some(L3{}, L0{}, stage ^ 1, (kt + 1) * BK);
             mma(fa_c, 0);
-            interleave_reads(fa_c);
+            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, FMA_LD_S0>();
             load_frags(fa_c, stage, 2, 0);
+            issue_some(std::integral_constant<int, FMA_LD_S3 + FMA_LD_S0>{}, L1{}, stage ^ 1, (kt + 1) * BK);
             mma(fa_c, 1);
-            interleave_reads(fa_c);
+            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, FMA_LD_S1>();
             load_frags(fa_c, stage, 3, 1);
+            issue_some(std::integral_constant<int, FMA_LD_S3 + FMA_LD_S0 + FMA_LD_S1>{}, L2{}, stage ^ 1, (kt + 1) * BK);
             mma(fa_c, 0);
-            interleave_reads(fa_c);
+            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, FMA_LD_S2>();
             // every load of step kt+1 has landed and every LDS read of this stage has returned
-            __builtin_amdgcn_s_waitcnt(0x0070);
+#ifdef FMA_PROF
+            uint64_t pt0, pt1, pt2;
+            asm volatile("s_memtime %0" : "=s"(pt0));
+#endif
+#if defined(FMA_DIAG) && FMA_DIAG >= 5
+            __builtin_amdgcn_s_waitcnt(0x0070 + (FMA_DIAG - 3));  // all but the newest 2 / 3 / 4 loads
+#else
+            // all but the newest load when that is the previous step's prefetch, else all
+            if constexpr (kPrefetch) __builtin_amdgcn_s_waitcnt(0x0071);
+            else __builtin_amdgcn_s_waitcnt(0x0070);
+#endif
+#ifdef FMA_PROF
+            PROF_STAMP(pt1);
+#endif
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
+#ifdef FMA_PROF
+            PROF_STAMP(pt2);
+            prof_wait += pt1 - pt0;
+            prof_bar += pt2 - pt1;
+            prof_steps += 1;
+#endif
             // unconditional (after the last step the fragments are simply not used): straight-line code lets the
             // compiler count outstanding LDS reads exactly, so the MFMAs below do not wait for these reads
             load_frags(fa_c, stage ^ 1, 0, 0);
-            // the loads of step kt+2 go out one per MFMA (a burst of loads stalls the wavefront's instruction issue);
-            // past the end of K they are all out of range (zero-fill), which keeps the loop body free of branches
-            issue(stage, (kt + 2) * BK);
+            // past the end of K the loads are all out of range (zero-fill), which keeps the loop body free of branches
+#if defined(FMA_DIAG) && FMA_DIAG >= 5
+            // timing only (wrong results): the last loads of the burst belong to step kt+3, so that they are not waited
+            // for at the next barrier; what a partial third stage would allow
+            issue_some(std::integral_constant<int, 0>{}, std::integral_constant<int, 8 - (FMA_DIAG - 3)>{}, stage, (kt + 2) * BK);
+            issue_some(std::integral_constant<int, 8 - (FMA_DIAG - 3)>{}, std::integral_constant<int, FMA_DIAG - 3>{}, stage, (kt + 3) * BK);
+#else
+            issue_some(std::integral_constant<int, 0>{}, L3{}, stage, (kt + 2) * BK);
+#endif
+            // the prefetch goes out behind this step's loads (the empty statement orders it: the wait of the next step
+            // counts on it being the newest load) and has until the wait of the step after next to complete
+            if constexpr (kPrefetch) asm volatile("" : "+v"(pf_voff));
+            issue_prefetch(kt + kPfDist);
             mma(fa_c, 1);
             if constexpr (FA > 0) {
-                constexpr int kReads = (A_KC ? FA : 2 * FA) + (B_KC ? FN : 2 * FN);
                 __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
-                spread_mfma_vmem<0, FA * FN, 2 * (32 / NW)>();
+                spread_mfma_vmem<0, FA * FN, FMA_LD_S3>();
+                if constexpr (kPrefetch) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
             }
         };
         const uint32_t KT = (Ke + BK - 1) / BK;
@@ -899,12 +851,31 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             asm volatile("" ::: "memory");
         } else if (KT > 0) {
             if (!prefetched) issue_quiet(0, 0);
-            if (KT > 1) issue_quiet(1, BK);
+            if (KT > 1) {
+                issue_quiet_a(1, BK);
+                if (!prefetched_b1) issue_quiet_b(1, BK);
+            }
+#ifdef FMA_PROF
+            PROF_SEG(2);  // rest of the first loads issued
+#endif
             nxt = lookup(++round);  // in the shadow of the loads
+#ifdef FMA_PROF
+            PROF_SEG(3);  // look-up of the tile after
+#endif
             // the first K step's loads have landed; the second step's, and the previous tile's stores, may still be out
             wait_outstanding((prefetched ? tile_stores : 0u) + (KT > 1 ? kStepLoads : 0u));
+#ifdef FMA_PROF
+            PROF_SEG(4);  // wait for the first K step's operands
+#endif
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
+#ifdef FMA_PROF
+            PROF_SEG(5);  // barrier
+#endif
+#ifdef FMA_PROF
+            if (prof_e0) { uint64_t t; PROF_STAMP(t); prof_edge += t - prof_e0; }
+#endif
+            issue_prefetch(kPfDist - 1);
             auto k_loop = [&](auto fa_c) {
                 load_frags(fa_c, 0, 0, 0);
                 // two steps per iteration without a branch between them (a branch there makes the compiler wait for
@@ -925,25 +896,41 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             __builtin_amdgcn_s_waitcnt(0x0f70);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
+#ifdef FMA_PROF
+            PROF_STAMP(prof_e0);
+            prof_t = prof_e0;
+#endif
         }
 
         // ---- next tile: its first loads go out now, into stage 0, and fly while this tile's results are stored ----
         prefetched = nxt.valid && nxt.fast && nxt.Ke > 0;
+        prefetched_b1 = false;
         if (prefetched) {
             setup_loaders(nxt);
+            setup_prefetch(nxt);
             issue_quiet(0, 0);
+            const uint32_t next_kt = (nxt.Ke + BK - 1) / BK;
+            const bool next_thin = A_KC && nxt.Me <= 64u && next_kt >= 3u;  // (has its own LDS layout and loads)
+            if (next_kt > 1 && !next_thin) {
+                issue_quiet_b(1, BK);
+                prefetched_b1 = true;
+            }
         }
+#ifdef FMA_PROF
+        PROF_SEG(0);  // next tile's loaders set up and first loads issued
+#endif
 
         // ---- epilogue ----
-        // Past the last barrier of the K loop nobody reads the LDS stages any more. Stage 1 is the staging space: each
-        // wavefront takes a private slice of it for half of its sub-tile at a time.
+        // Past the last barrier of the K loop nobody reads the LDS stages any more. The A half of stage 1 is the staging
+        // space: each wavefront takes the four 1 KB pieces of it that it itself loads, for one 32-row block of its
+        // sub-tile at a time (stage 0 and the B half of stage 1 already receive the next tile's operands).
         // A lane holds row (lane & 31), columns q*8 + (lane >> 5)*4 + 0..3 of each 32x32 accumulator block.
-        static_assert(FM % 2 == 0 && WM * WN == 2 * (32 / NW) * 1024, "two passes over the slices of one LDS stage");
+        static_assert(32 * WN * 2 == (32 / NW) * 1024, "one 32-row block of a wavefront's sub-tile fills its pieces of one operand array");
         // the lane id is made opaque here so that the epilogue's per-lane address arithmetic is redone per tile instead
         // of being hoisted out of the tile loop, where it would occupy registers throughout the K loop
         uint32_t el = lane;
         asm volatile("" : "+v"(el));
-        const StagingSlice<NW> img{s_a1 + wave * 1024u, s_b1 + wave * 1024u};
+        const StagingSlice<NW> img{s_a1 + wave * 1024u, s_a1 + wave * 1024u};
         // alpha is applied up front, and only when it is not 1 (the usual case, and always so for the SwiGLU epilogue)
         if (EPI == EPI_PLAIN && args.alpha != 1.0f) {
             const float alpha = args.alpha;
@@ -952,82 +939,84 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
 #pragma unroll
                 for (int j = 0; j < FN; ++j) acc[i][j] *= alpha;
         }
-        constexpr int HM = WM / 2;  // rows per pass
-        constexpr int HF = FM / 2;  // accumulator row blocks per pass
 #pragma unroll
-        for (int pass = 0; pass < 2; ++pass) {
-            const uint32_t row0 = m0 + wm * WM + pass * HM;  // first output row of this pass
-            const uint32_t rows_valid = row0 < Me ? (Me - row0 < (uint32_t)HM ? Me - row0 : (uint32_t)HM) : 0u;
+        for (int i = 0; i < FM; ++i) {
+            const uint32_t row0 = m0 + wm * WM + i * 32;  // first output row of this pass
+            const uint32_t rows_valid = row0 < Me ? (Me - row0 < 32u ? Me - row0 : 32u) : 0u;
             if constexpr (EPI == EPI_PLAIN) {
                 const uint32_t col0 = n0 + wn * WN;
                 const uint32_t cols_valid = col0 < n_lim ? n_lim - col0 : 0u;
 #pragma unroll
-                for (int i = 0; i < HF; ++i)
+                for (int j = 0; j < FN; ++j)
 #pragma unroll
-                    for (int j = 0; j < FN; ++j)
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            const f32x16& c = acc[pass * HF + i][j];
-                            uint2 w;
-                            w.x = EL::pack2(c[q * 4 + 0], c[q * 4 + 1]);
-                            w.y = EL::pack2(c[q * 4 + 2], c[q * 4 + 3]);
-                            stage_put<WN * 2>(img, i * 32 + (el & 31u), j * 32 + q * 8 + (el >> 5) * 4, w);
-                        }
-                stage_flush<WN * 2, HM>(img, args.D + off_d + (uint64_t)row0 * Ne + col0, Ne, rows_valid, cols_valid, el);
+                    for (int q = 0; q < 4; ++q) {
+                        const f32x16& c = acc[i][j];
+                        uint2 w;
+                        w.x = EL::pack2(c[q * 4 + 0], c[q * 4 + 1]);
+                        w.y = EL::pack2(c[q * 4 + 2], c[q * 4 + 3]);
+                        stage_put<WN * 2>(img, el & 31u, j * 32 + q * 8 + (el >> 5) * 4, w);
+                    }
+                stage_flush<WN * 2, 32>(img, args.D + off_d + (uint64_t)row0 * Ne + col0, Ne, rows_valid, cols_valid, el);
             } else {
                 // first the rounded pre-activation (32 "up" columns | 32 "gate" columns per row), then the activation
                 constexpr int HB = WN * 2;  // bytes per staged row of h: 32 "up" columns | 32 "gate" columns
                 constexpr int YB = WN;      // bytes per staged row of the activation
+                static_assert(FN == 2, "one up block and one gate block per wavefront and row block");
                 const uint32_t col0 = n0 + wn * (WN / 2);
                 const uint32_t cols_valid = col0 < n_lim ? n_lim - col0 : 0u;
-                uint32_t ypack[HF][FN / 2][4][2];  // the packed activation waits here until h has left the staging slice
+                uint32_t ypack[4][2];  // the packed activation waits here until h has left the staging slice
 #pragma unroll
-                for (int i = 0; i < HF; ++i)
+                for (int q = 0; q < 4; ++q) {
+                    float u[4], g[4], y[4];
 #pragma unroll
-                    for (int j = 0; j < FN / 2; ++j)
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            float u[4], g[4], y[4];
-#pragma unroll
-                            for (int x = 0; x < 4; ++x) {
-                                u[x] = EL::round(acc[pass * HF + i][j][q * 4 + x]);
-                                g[x] = EL::round(acc[pass * HF + i][j + FN / 2][q * 4 + x]);
-                                y[x] = u[x] * g[x] * sigmoid_for<typename EL::act_t>(g[x]);
-                            }
-                            ypack[i][j][q][0] = EL::pack2(y[0], y[1]);
-                            ypack[i][j][q][1] = EL::pack2(y[2], y[3]);
-                            if constexpr (EPI == EPI_SWIGLU) {
-                                const uint32_t m = i * 32 + (el & 31u);
-                                const uint32_t c = j * 32 + q * 8 + (el >> 5) * 4;
-                                uint2 wu, wg;
-                                wu.x = EL::pack2(u[0], u[1]);
-                                wu.y = EL::pack2(u[2], u[3]);
-                                wg.x = EL::pack2(g[0], g[1]);
-                                wg.y = EL::pack2(g[2], g[3]);
-                                stage_put<HB>(img, m, c, wu);
-                                stage_put<HB>(img, m, WN / 2 + c, wg);
-                            }
-                        }
+                    for (int x = 0; x < 4; ++x) {
+                        u[x] = EL::round(acc[i][0][q * 4 + x]);
+                        g[x] = EL::round(acc[i][1][q * 4 + x]);
+                        y[x] = u[x] * g[x] * sigmoid_for<typename EL::act_t>(g[x]);
+                    }
+                    ypack[q][0] = EL::pack2(y[0], y[1]);
+                    ypack[q][1] = EL::pack2(y[2], y[3]);
+                    if constexpr (EPI == EPI_SWIGLU) {
+                        const uint32_t c = q * 8 + (el >> 5) * 4;
+                        uint2 wu, wg;
+                        wu.x = EL::pack2(u[0], u[1]);
+                        wu.y = EL::pack2(u[2], u[3]);
+                        wg.x = EL::pack2(g[0], g[1]);
+                        wg.y = EL::pack2(g[2], g[3]);
+                        stage_put<HB>(img, el & 31u, c, wu);
+                        stage_put<HB>(img, el & 31u, WN / 2 + c, wg);
+                    }
+                }
                 if constexpr (EPI == EPI_SWIGLU)
-                    stage_flush_split<HB, HM, WN / 2>(img, args.D + off_d + (uint64_t)row0 * Ne + col0, Ne, rows_valid,
+                    stage_flush_split<HB, 32, WN / 2>(img, args.D + off_d + (uint64_t)row0 * Ne + col0, Ne, rows_valid,
                                                       cols_valid, n_span, el);
 #pragma unroll
-                for (int i = 0; i < HF; ++i)
-#pragma unroll
-                    for (int j = 0; j < FN / 2; ++j)
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            uint2 wy;
-                            wy.x = ypack[i][j][q][0];
-                            wy.y = ypack[i][j][q][1];
-                            stage_put<YB>(img, i * 32 + (el & 31u), j * 32 + q * 8 + (el >> 5) * 4, wy);
-                        }
-                stage_flush<YB, HM>(img, args.ACT + off_d / 2 + (uint64_t)row0 * n_span + col0, n_span, rows_valid,
-                                    cols_valid, el);
+                for (int q = 0; q < 4; ++q) {
+                    uint2 wy;
+                    wy.x = ypack[q][0];
+                    wy.y = ypack[q][1];
+                    stage_put<YB>(img, el & 31u, q * 8 + (el >> 5) * 4, wy);
+                }
+                stage_flush<YB, 32>(img, args.ACT + off_d / 2 + (uint64_t)row0 * n_span + col0, n_span, rows_valid, cols_valid, el);
             }
         }
+#ifdef FMA_PROF
+        PROF_SEG(1);  // epilogue
+#endif
         cur = nxt;
     }
+#ifdef FMA_PROF
+    {
+        uint64_t t;
+        PROF_STAMP(t);
+        if (lane == 0) {
+            unsigned long long* o = fma_prof + ((size_t)blockIdx.x * 8 + wave) * 8;
+            o[0] = prof_wait; o[1] = prof_bar; o[2] = prof_steps; o[3] = t - prof_start; o[4] = prof_edge;
+            unsigned long long* o2 = fma_prof + 1024 * 8 * 8 + ((size_t)blockIdx.x * 8 + wave) * 8;
+            for (int i = 0; i < 6; ++i) o2[i] = prof_seg[i];
+        }
+    }
+#endif
 }
 
 // wavefronts per workgroup: kWavesM x kWavesN (2 x 4 = eight 128x64 wave tiles, 2 x 2 = four 128x128 wave tiles)
@@ -1070,6 +1059,12 @@ int launch_plain(const GemmArgs& args, bool a_kc, bool b_kc, hipStream_t st) {
 }  // namespace fmahip
 
 extern "C" {
+
+#ifdef FMA_PROF
+int fma_debug_prof(void* host, int64_t bytes) {
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(fmahip::gemm::fma_prof), (size_t)bytes, 0, hipMemcpyDeviceToHost);
+}
+#endif
 
 int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_arr, const uint32_t* N_arr,
                      const uint32_t* K_arr, int64_t E, int trans_a, int trans_b, float alpha, int dtype,
