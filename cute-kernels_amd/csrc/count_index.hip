@@ -167,16 +167,19 @@ __global__ __launch_bounds__(kReduceThreads) void count_reduce_kernel(const uint
     constexpr uint32_t parts = kReduceThreads / kReduceBins;
     uint32_t s = 0;
     if (e < E) {
-        // eight independent loads in flight per thread: the rows are few, the latency of each load is what costs
-        uint32_t b = part;
-        for (; b + 7 * parts < rows; b += 8 * parts) {
-            uint32_t r[8];
+        // the rows are few and the latency of a load is what costs: all of a thread's rows (32 of them when two
+        // workgroups per compute unit counted on 256 units) are requested before the first is added
+        constexpr int kInFlight = 32;
+        for (uint32_t b0 = part; b0 < rows; b0 += kInFlight * parts) {
+            uint32_t r[kInFlight];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) r[u] = partials[(uint64_t)(b + u * parts) * E + e];
+            for (int u = 0; u < kInFlight; ++u) {
+                const uint32_t b = b0 + u * parts;
+                r[u] = b < rows ? partials[(uint64_t)b * E + e] : 0u;
+            }
 #pragma unroll
-            for (int u = 0; u < 8; ++u) s += r[u];
+            for (int u = 0; u < kInFlight; ++u) s += r[u];
         }
-        for (; b < rows; b += parts) s += partials[(uint64_t)b * E + e];
     }
     s_sum[tid] = s;
     __syncthreads();

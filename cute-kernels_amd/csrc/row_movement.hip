@@ -11,7 +11,9 @@ namespace fmahip {
 namespace {
 
 constexpr int kRowThreads = 256;
-constexpr int kGatherRows = 4;  // rows per workgroup in the gather
+// rows per workgroup in the gather, tokens per workgroup in the dispatch: one each. Small one-shot workgroups stream
+// best on this part (dispatch at 4 / 2 / 1 tokens per workgroup: 92 / 87 / 74 us; gather at 4 / 2 / 1 rows: 81 / 80 / 79 us)
+constexpr int kGatherRows = 1;
 
 // One element standing in for a 16-byte vector.
 template <typename T>
@@ -47,7 +49,7 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_kernel(const U* __res
     for (int64_t v = threadIdx.x; v < vecs; v += kRowThreads) {
         U t[kGatherRows];
 #pragma unroll
-        for (int r = 0; r < kGatherRows; ++r) t[r] = src[r][v];
+        for (int r = 0; r < kGatherRows; ++r) t[r] = src[r][v];  // plain loads: a row is fetched once per expert choice
 #pragma unroll
         for (int r = 0; r < kGatherRows; ++r) {
             if (i0 + r < R) store_unit(out + (i0 + r) * vecs + v, t[r]);
@@ -57,7 +59,7 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_kernel(const U* __res
 
 // out[inv[t*k + j]] = x[t] for j < k: the same gather written from the token's side, so that every input row is
 // fetched once however many experts it is routed to
-constexpr int kDispatchTokens = 2;  // tokens per workgroup
+constexpr int kDispatchTokens = 1;
 template <typename U>
 __global__ __launch_bounds__(kRowThreads) void dispatch_rows_kernel(const U* __restrict__ x,
                                                                     const int32_t* __restrict__ inv, int64_t T,
@@ -66,7 +68,7 @@ __global__ __launch_bounds__(kRowThreads) void dispatch_rows_kernel(const U* __r
     for (int64_t v = threadIdx.x; v < vecs; v += kRowThreads) {
         U row[kDispatchTokens];
 #pragma unroll
-        for (int u = 0; u < kDispatchTokens; ++u) row[u] = x[(t0 + u < T ? t0 + u : T - 1) * vecs + v];
+        for (int u = 0; u < kDispatchTokens; ++u) row[u] = load_unit(x + (t0 + u < T ? t0 + u : T - 1) * vecs + v);
 #pragma unroll
         for (int u = 0; u < kDispatchTokens; ++u) {
             if (t0 + u < T) {
@@ -77,8 +79,10 @@ __global__ __launch_bounds__(kRowThreads) void dispatch_rows_kernel(const U* __r
     }
 }
 
-// y[t] = sum_j gates[t,j] * o[inv[t,j]]; one workgroup per token, fp32 accumulation in ascending j
-template <typename T, typename V>
+// y[t] = sum_j gates[t,j] * o[inv[t,j]]; one workgroup per token, fp32 accumulation in ascending j.
+// KC > 0: top_k known at compile time. All KC row loads of a vector position (of two positions per thread for KC <= 4)
+// are issued before the first multiply, as streaming loads: the expert rows are read exactly once.
+template <typename T, typename V, int KC>
 __global__ __launch_bounds__(kRowThreads) void combine_kernel(const V* __restrict__ o,
                                                               const int32_t* __restrict__ inv,
                                                               const T* __restrict__ gates, int64_t k, int64_t vecs,
@@ -87,35 +91,73 @@ __global__ __launch_bounds__(kRowThreads) void combine_kernel(const V* __restric
     const int64_t t = blockIdx.x;
     const int32_t* my_inv = inv + t * k;
     const T* my_gates = gates ? gates + t * k : nullptr;
-    for (int64_t v = threadIdx.x; v < vecs; v += kRowThreads) {
-        float acc[N];
+    if constexpr (KC > 0) {
+        constexpr int VU = KC <= 4 ? 2 : 1;  // vector positions in flight per thread
+        const V* rows[KC];
+        float g[KC];
 #pragma unroll
-        for (int c = 0; c < N; ++c) acc[c] = 0.0f;
-        int64_t j = 0;
-        for (; j + 4 <= k; j += 4) {
-            V r[4];
-            float g[4];
+        for (int j = 0; j < KC; ++j) {
+            rows[j] = o + (int64_t)my_inv[j] * vecs;
+            g[j] = my_gates ? Num<T>::up(my_gates[j]) : 1.0f;
+        }
+        for (int64_t v0 = threadIdx.x; v0 < vecs; v0 += (int64_t)VU * kRowThreads) {
+            V r[VU][KC];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                r[u] = load_unit(o + (int64_t)my_inv[j + u] * vecs + v);
-                g[u] = my_gates ? Num<T>::up(my_gates[j + u]) : 1.0f;
+            for (int u = 0; u < VU; ++u) {
+                const int64_t v = v0 + (int64_t)u * kRowThreads;
+                const int64_t vc = v < vecs ? v : v0;
+#pragma unroll
+                for (int j = 0; j < KC; ++j) r[u][j] = load_unit(rows[j] + vc);
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < VU; ++u) {
+                const int64_t v = v0 + (int64_t)u * kRowThreads;
+                if (v < vecs) {
+                    float acc[N];
 #pragma unroll
-                for (int c = 0; c < N; ++c) acc[c] = fmaf(g[u], Num<T>::up(r[u].v[c]), acc[c]);
+                    for (int c = 0; c < N; ++c) acc[c] = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < KC; ++j)
+#pragma unroll
+                        for (int c = 0; c < N; ++c) acc[c] = fmaf(g[j], Num<T>::up(r[u][j].v[c]), acc[c]);
+                    V w;
+#pragma unroll
+                    for (int c = 0; c < N; ++c) w.v[c] = Num<T>::down(acc[c]);
+                    store_unit(y + t * vecs + v, w);
+                }
             }
         }
-        for (; j < k; ++j) {
-            const V r = o[(int64_t)my_inv[j] * vecs + v];
-            const float g = my_gates ? Num<T>::up(my_gates[j]) : 1.0f;
+    } else {
+        for (int64_t v = threadIdx.x; v < vecs; v += kRowThreads) {
+            float acc[N];
 #pragma unroll
-            for (int c = 0; c < N; ++c) acc[c] = fmaf(g, Num<T>::up(r.v[c]), acc[c]);
+            for (int c = 0; c < N; ++c) acc[c] = 0.0f;
+            int64_t j = 0;
+            for (; j + 4 <= k; j += 4) {
+                V r[4];
+                float g[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    r[u] = load_unit(o + (int64_t)my_inv[j + u] * vecs + v);
+                    g[u] = my_gates ? Num<T>::up(my_gates[j + u]) : 1.0f;
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                    for (int c = 0; c < N; ++c) acc[c] = fmaf(g[u], Num<T>::up(r[u].v[c]), acc[c]);
+                }
+            }
+            for (; j < k; ++j) {
+                const V r = load_unit(o + (int64_t)my_inv[j] * vecs + v);
+                const float g = my_gates ? Num<T>::up(my_gates[j]) : 1.0f;
+#pragma unroll
+                for (int c = 0; c < N; ++c) acc[c] = fmaf(g, Num<T>::up(r.v[c]), acc[c]);
+            }
+            V w;
+#pragma unroll
+            for (int c = 0; c < N; ++c) w.v[c] = Num<T>::down(acc[c]);
+            store_unit(y + t * vecs + v, w);
         }
-        V w;
-#pragma unroll
-        for (int c = 0; c < N; ++c) w.v[c] = Num<T>::down(acc[c]);
-        y[t * vecs + v] = w;
     }
 }
 
@@ -186,8 +228,23 @@ template <typename T, typename V>
 int launch_combine(const void* o, const int32_t* inv, const void* gates, int64_t T_, int64_t k, int64_t H, void* y,
                    hipStream_t st) {
     const int64_t vecs = H / V::N;
-    hipLaunchKernelGGL((combine_kernel<T, V>), dim3((uint32_t)T_), dim3(kRowThreads), 0, st, (const V*)o, inv,
-                       (const T*)gates, k, vecs, (V*)y);
+#define FMA_COMBINE_CASE(KC)                                                                                     \
+    case KC:                                                                                                     \
+        hipLaunchKernelGGL((combine_kernel<T, V, KC>), dim3((uint32_t)T_), dim3(kRowThreads), 0, st, (const V*)o, inv, \
+                           (const T*)gates, k, vecs, (V*)y);                                                     \
+        break;
+    switch (sizeof(V) == 16 ? k : 0) {  // the element-wise form keeps the generic loop
+        FMA_COMBINE_CASE(1)
+        FMA_COMBINE_CASE(2)
+        FMA_COMBINE_CASE(3)
+        FMA_COMBINE_CASE(4)
+        FMA_COMBINE_CASE(6)
+        FMA_COMBINE_CASE(8)
+        default:
+            hipLaunchKernelGGL((combine_kernel<T, V, 0>), dim3((uint32_t)T_), dim3(kRowThreads), 0, st, (const V*)o, inv,
+                               (const T*)gates, k, vecs, (V*)y);
+    }
+#undef FMA_COMBINE_CASE
     return launch_status("combine");
 }
 

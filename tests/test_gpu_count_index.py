@@ -42,7 +42,7 @@ def test_count_16m_ids(kind, np_dtype, dtype):
     ids = O.make_ids(n, E, kind, seed=11, dtype=np_dtype)
     x = torch.from_numpy(ids).to(DEV)
     expect = c_oracle.continuous_count(ids, E)
-    for _ in range(3):  # back-to-back calls share one workspace: the ticket must come back to zero
+    for _ in range(3):  # back-to-back calls must not see each other's partial histograms
         got = to_np(continuous_count(x, E, kernel_backend=KernelBackend.cuda))
         assert np.array_equal(got, expect)
     assert int(got.astype(np.int64).sum()) == n
