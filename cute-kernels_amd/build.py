@@ -9,6 +9,7 @@ is not recompiled.
 
 import argparse
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -47,18 +48,49 @@ def _headers() -> list[str]:
     return headers
 
 
+# Sources whose kernels count their own outstanding memory operations (s_waitcnt vmcnt(N) with hand-counted N): a
+# register spill would add loads and stores of its own and shift those counts, so that LDS stages could be read before
+# the operands have landed. Their kernels must use no scratch memory; the build checks the compiler's resource report.
+NO_SCRATCH_SOURCES = {"grouped_gemm.hip": "grouped_gemm_kernel"}
+
+
+def _check_no_scratch(src: str, report: str, kernel_substring: str) -> None:
+    names = re.findall(r"Function Name: (\S+)", report)
+    scratch = re.findall(r"ScratchSize \[bytes/lane\]: (\d+)", report)
+    checked = 0
+    for name, size in zip(names, scratch):
+        if kernel_substring in name:
+            checked += 1
+            if int(size) != 0:
+                raise RuntimeError(f"{src}: kernel {name} uses {size} bytes of scratch per lane (register spills); "
+                                   "its hand-counted s_waitcnt values are only valid without scratch traffic")
+    if checked == 0:
+        raise RuntimeError(f"{src}: the compiler's resource report names no {kernel_substring} kernel")
+
+
 def _compile_one(src: str, force: bool) -> str:
     obj = os.path.join(OBJ_DIR, os.path.basename(src).replace(".hip", ".o"))
     if not force and os.path.exists(obj):
         newest = max(os.path.getmtime(p) for p in [src] + _headers())
         if os.path.getmtime(obj) >= newest:
             return obj
-    cmd = [HIPCC] + FLAGS + ["-c", src, "-o", obj]
+    guarded = NO_SCRATCH_SOURCES.get(os.path.basename(src))
+    cmd = [HIPCC] + FLAGS + (["-Rpass-analysis=kernel-resource-usage"] if guarded else []) + ["-c", src, "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
-    # hipcc's host pass warns that it does not know the packed-fp32 feature; that is harmless noise
-    err = "\n".join(line for line in proc.stderr.splitlines() if "packed-fp32-ops" not in line)
     if proc.returncode != 0:
+        err = "\n".join(line for line in proc.stderr.splitlines() if "packed-fp32-ops" not in line)
         raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+    stderr = proc.stderr
+    if guarded:
+        try:
+            _check_no_scratch(src, stderr, guarded)
+        except RuntimeError:
+            os.remove(obj)
+            raise
+        # the report (remarks with their source excerpts) is not repeated on the console; warnings are
+        stderr = "\n".join(line for line in stderr.splitlines() if "warning:" in line)
+    # hipcc's host pass warns that it does not know the packed-fp32 feature; that is harmless noise
+    err = "\n".join(line for line in stderr.splitlines() if "packed-fp32-ops" not in line)
     if err.strip():
         sys.stderr.write(err + "\n")
     return obj

@@ -592,7 +592,9 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     constexpr uint32_t kStepLoads = 2 * (32 / NW);  // load instructions per wavefront and K step
     // store instructions per wavefront and tile (stage_flush issues a fixed number)
     const uint32_t tile_stores = EPI == EPI_PLAIN ? WM * WN * 2 / 1024 : (EPI == EPI_SWIGLU ? WM * WN * 2 / 1024 : 0) + WM * WN / 1024;
-    // waits until at most n of this wavefront's loads and stores are outstanding (they complete in issue order)
+    // waits until at most n of this wavefront's loads and stores are outstanding (they complete in issue order).
+    // The counts passed here are the instructions this source issues: they are valid only while the compiler adds no
+    // memory instructions of its own, i.e. while the kernel has no register spills (the build fails if it has any).
     auto wait_outstanding = [&](uint32_t n) {
         if (n >= 40) __builtin_amdgcn_s_waitcnt(0x8f78);       // vmcnt(40)
         else if (n >= 32) __builtin_amdgcn_s_waitcnt(0x8f70);  // vmcnt(32)
@@ -1019,12 +1021,9 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
 #endif
 }
 
-// wavefronts per workgroup: kWavesM x kWavesN (2 x 4 = eight 128x64 wave tiles, 2 x 2 = four 128x128 wave tiles)
-#ifndef FMA_GEMM_WAVES_N
-#define FMA_GEMM_WAVES_N 4
-#endif
+// wavefronts per workgroup: kWavesM x kWavesN = eight 128x64 wave tiles (the hand-counted waits are written for eight)
 constexpr int kWavesM = 2;
-constexpr int kWavesN = FMA_GEMM_WAVES_N;
+constexpr int kWavesN = 4;
 
 // every instantiation the entry points launch (explicit, so that host stub and device code are both emitted)
 #define FMA_GEMM_INSTANTIATE(EL)                                                                             \

@@ -146,6 +146,9 @@ class MoE(nn.Module):
         return hidden_states, router_logits
 
     def _router_is_fusable(self, hidden_states: torch.Tensor) -> bool:
+        # the last three lines are the size limits of fma_router_topk (32-bit offsets into logits and choices): larger
+        # inputs take the library calls below instead of raising
+        T = hidden_states.size(0)
         return (
             self.fuse_router
             and hidden_states.is_cuda
@@ -154,6 +157,9 @@ class MoE(nn.Module):
             and self.hidden_size % 8 == 0
             and self.num_experts <= 1024
             and self.top_k <= 64
+            and self.hidden_size <= (1 << 24)
+            and T * self.num_experts <= 2**31 - 1
+            and T * self.top_k <= 2**31 - 1
         )
 
     def _compute_routing_weights(self, hidden_states: torch.Tensor) -> tuple[torch.Tensor]:

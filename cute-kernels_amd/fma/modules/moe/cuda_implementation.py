@@ -448,13 +448,16 @@ class _UpProjectionSwiglu(torch.autograd.Function):
     @staticmethod
     @ensure_contiguous
     def forward(
-        ctx, x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor
-    ) -> torch.Tensor:
+        ctx, x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor,
+        grad_enabled: bool,
+    ) -> torch.Tensor:  # fmt: skip
         _, N, K = weight.size()
         assert N % 16 == 0
         assert K % 8 == 0
         R = x.size(0)
-        needs_backward = any(ctx.needs_input_grad[:2])
+        # needs_input_grad only says that an input requires grad; under no_grad / inference_mode no backward will
+        # follow (grad mode is always off inside forward, so the caller passes what it was outside)
+        needs_backward = grad_enabled and any(ctx.needs_input_grad[:2])
         h = torch.empty(R, N, device=x.device, dtype=x.dtype) if needs_backward else None
         act = torch.empty(R, N // 2, device=x.device, dtype=x.dtype)
         grouped_gemm_swiglu_cuda(x, weight, M_array, h, act)
@@ -485,7 +488,7 @@ class _UpProjectionSwiglu(torch.autograd.Function):
                 A=h_grad, B=x, C=None, M_array=N_array, N_array=K_array, K_array=M_array,
                 output_shape=weight.size(), is_A_transposed=True, is_B_transposed=False,
             )
-        return x_grad, weight_grad, None, None, None
+        return x_grad, weight_grad, None, None, None, None
 
 
 # ---- the reference's padded grouping interface -------------------------------------------------------
@@ -650,4 +653,4 @@ def grouped_gemm_experts(
 def up_projection_swiglu_experts(
     x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor
 ) -> torch.Tensor:
-    return _UpProjectionSwiglu.apply(x, weight, M_array, N_array, K_array)
+    return _UpProjectionSwiglu.apply(x, weight, M_array, N_array, K_array, torch.is_grad_enabled())

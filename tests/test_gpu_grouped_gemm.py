@@ -353,3 +353,78 @@ def test_fused_swiglu_on_groups_of_few_rows(K):
     assert torch.equal(h, h_plain) and torch.equal(act, swiglu_packed(h_plain))
     expect = torch.cat([xe.float() @ w[e].float().T for e, xe in enumerate(x.split(M_list))])
     assert float((h.float() - expect).abs().max()) <= 2**-8 * float(expect.abs().max())
+
+
+def _exact_nt(x, w, M_list):
+    """h_e = x_e @ w_e^T in float64 on the CPU (exact for small integers), rows of all groups back to back"""
+    xs = x.cpu().double().split(M_list)
+    return torch.cat([xs[e] @ w[e].cpu().double().T for e in range(len(M_list))])
+
+
+def _small_group_case(M_list, N, K, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    E, R = len(M_list), sum(M_list)
+    x = torch.randint(-3, 4, (R, K), generator=g).to(dtype).to(DEV)
+    w = torch.randint(-3, 4, (E, N, K), generator=g).to(dtype).to(DEV)
+    return x, w, _u32(M_list), E, R
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("K", [64, 192, 1000])
+def test_half_width_tiles_many_small_groups(dtype, K):
+    # Launches made of groups of at most 64 rows only, whose last round of full-width tiles would be at most half full, run
+    # column tiles of half the width: 96 groups x 4 full-width tiles = 384 tiles = 1.5 rounds of 256 workgroups become 768
+    # half-width tiles, several rounds, several per group, the last one of every group partial (1000 = 7 * 128 + 104).
+    # Integers in [-3, 3]: |sum| <= 9000, exact in fp32 and, after rounding, compared as rounded values.
+    M_list = [1 + (7 * e) % 64 for e in range(96)]
+    N = 1000
+    x, w, M, E, R = _small_group_case(M_list, N, K, dtype, seed=K)
+    got = grouped_gemm(A=x, B=w, C=None, M_array=M, N_array=_u32([N] * E), K_array=_u32([K] * E), output_shape=(R, N),
+                       is_A_transposed=False, is_B_transposed=True)
+    expect = _exact_nt(x, w, M_list).to(dtype)
+    assert torch.equal(got.cpu(), expect)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("K", [64, 192, 1000])
+def test_half_width_tiles_fused_swiglu(dtype, K):
+    # the same launch shape through the fused epilogue: I = 520 -> 5 tiles of 128 + 128 columns per group at full width
+    # (480 tiles), 9 per group at half width, the last one 8 columns wide
+    M_list = [1 + (5 * e) % 64 for e in range(96)]
+    inter = 520
+    x, w, M, E, R = _small_group_case(M_list, 2 * inter, K, dtype, seed=K + 1)
+    h = torch.empty(R, 2 * inter, dtype=dtype, device=DEV)
+    act = torch.empty(R, inter, dtype=dtype, device=DEV)
+    grouped_gemm_swiglu_cuda(x, w, M, h, act)
+    assert torch.equal(h.cpu(), _exact_nt(x, w, M_list).to(dtype))
+    assert torch.equal(act, swiglu_packed(h))
+    act_only = torch.empty_like(act)
+    grouped_gemm_swiglu_cuda(x, w, M, None, act_only)
+    assert torch.equal(act_only, act)
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_half_width_decision_boundaries(fused):
+    # The width is decided per launch from the tile counts and the number of workgroups (one per compute unit). Launches
+    # just on either side of both thresholds: small groups only (half width while twice the tiles need at most 1.8 times
+    # the rounds: groups = units / 2 and units / 2 + 1, one tile each), and small groups beside a large one (half width
+    # while all tiles fill at most half of the workgroups).
+    from fma import _lib
+
+    units = _lib.load().fma_num_compute_units()
+    assert units >= 8
+    K, N = 192, 256
+    cases = [[16] * (units // 2), [16] * (units // 2 + 1), [300] + [16] * (units // 2 - 2), [300] + [16] * (units // 2 - 1)]
+    for i, M_list in enumerate(cases):
+        x, w, M, E, R = _small_group_case(M_list, 2 * N if fused else N, K, torch.bfloat16, seed=40 + i)
+        expect = _exact_nt(x, w, M_list).to(torch.bfloat16)
+        if fused:
+            h = torch.empty(R, 2 * N, dtype=torch.bfloat16, device=DEV)
+            act = torch.empty(R, N, dtype=torch.bfloat16, device=DEV)
+            grouped_gemm_swiglu_cuda(x, w, M, h, act)
+            assert torch.equal(h.cpu(), expect), f"case {i}"
+            assert torch.equal(act, swiglu_packed(h)), f"case {i}"
+        else:
+            got = grouped_gemm(A=x, B=w, C=None, M_array=M, N_array=_u32([N] * E), K_array=_u32([K] * E),
+                               output_shape=(R, N), is_A_transposed=False, is_B_transposed=True)
+            assert torch.equal(got.cpu(), expect), f"case {i}"

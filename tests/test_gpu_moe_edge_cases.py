@@ -116,6 +116,32 @@ def test_frozen_parameters_and_inference(dtype):
         _assert_same(y_full, moe(x, kernel_backend=KernelBackend.cuda)[0], "output under inference_mode")
 
 
+@pytest.mark.parametrize("mode", ["no_grad", "inference_mode"])
+def test_evaluation_with_trainable_weights_does_not_store_the_preactivation(mode, monkeypatch):
+    # a model whose parameters require grad, evaluated with autograd off (the usual eval / decode call): the fused
+    # up-projection must run without the [R, 2I] pre-activation buffer, and give the bits of the training forward
+    from fma.modules.moe import cuda_implementation as ci
+
+    torch.manual_seed(6)
+    moe = MoE(8, 2, 256, 512, swiglu_packed, True, False, 0.02).to(DEV).to(torch.bfloat16)
+    assert moe.fuse_swiglu and all(p.requires_grad for p in moe.parameters())
+    x = torch.randn(300, 256, device=DEV).bfloat16()
+    seen = []
+    real = ci.grouped_gemm_swiglu_cuda
+
+    def spy(x_, weight, M_array, h, act):
+        seen.append(h is not None)
+        return real(x_, weight, M_array, h, act)
+
+    monkeypatch.setattr(ci, "grouped_gemm_swiglu_cuda", spy)
+    y_train, _ = moe(x.clone().requires_grad_(), kernel_backend=KernelBackend.cuda)
+    assert seen == [True]
+    with torch.no_grad() if mode == "no_grad" else torch.inference_mode():
+        y_eval, _ = moe(x, kernel_backend=KernelBackend.cuda)
+    assert seen == [True, False], "the pre-activation was stored although no backward can follow"
+    _assert_same(y_train.detach(), y_eval, f"output under {mode}")
+
+
 @pytest.mark.parametrize("add_bias", [False, True])
 def test_training_step_is_bit_reproducible(add_bias):
     # nothing on the path accumulates with floating-point atomics (the reference's grouped rows, weight gradients and

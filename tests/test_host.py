@@ -144,3 +144,18 @@ def test_router_and_bias_host_logic():
     top1 = MoE(4, 1, 64, 128, swiglu_packed, True, False, 0.02)
     _, w1, s1 = top1._compute_routing_weights(torch.randn(5, 64))
     assert torch.equal(w1, torch.ones(5, 1)) and s1.shape == (5, 1)
+
+
+def test_build_refuses_gemm_kernels_with_register_spills():
+    # the grouped GEMM counts its outstanding memory operations by hand; the build reads the compiler's resource report
+    # and fails when one of its kernels uses scratch memory (spill traffic would shift those counts)
+    import build
+
+    clean = "remark: Function Name: _Zfoo19grouped_gemm_kernelIbar\nremark:     ScratchSize [bytes/lane]: 0\n"
+    build._check_no_scratch("grouped_gemm.hip", clean, "grouped_gemm_kernel")
+    spilled = clean.replace("[bytes/lane]: 0", "[bytes/lane]: 24")
+    with pytest.raises(RuntimeError, match="scratch"):
+        build._check_no_scratch("grouped_gemm.hip", spilled, "grouped_gemm_kernel")
+    with pytest.raises(RuntimeError, match="names no"):
+        build._check_no_scratch("grouped_gemm.hip", "remark: Function Name: other\n", "grouped_gemm_kernel")
+    assert "grouped_gemm.hip" in build.NO_SCRATCH_SOURCES
