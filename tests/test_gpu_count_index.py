@@ -7,6 +7,7 @@ import torch
 from fma import KernelBackend, continuous_count
 from fma.modules.moe.cuda_implementation import build_routing_index
 from oracle import c_oracle, moe_oracle as O
+from synthetic_inputs import make_ids, make_routing
 
 from gpu_util import DEV, to_np
 
@@ -39,7 +40,7 @@ def test_count_reference_generator(dtype):
 def test_count_16m_ids(kind, np_dtype, dtype):
     # the histogram benchmark configuration: 16 Mi ids in [0, 64), uniform and Zipf(1.2)
     n, E = 16 << 20, 64
-    ids = O.make_ids(n, E, kind, seed=11, dtype=np_dtype)
+    ids = make_ids(n, E, kind, seed=11, dtype=np_dtype)
     x = torch.from_numpy(ids).to(DEV)
     expect = c_oracle.continuous_count(ids, E)
     for _ in range(3):  # back-to-back calls must not see each other's partial histograms
@@ -50,7 +51,7 @@ def test_count_16m_ids(kind, np_dtype, dtype):
 
 @pytest.mark.parametrize("E", [2, 3, 72, 129, 1000, 4096, 16384])
 def test_count_bin_counts(E):
-    ids = O.make_ids(300_007, E, "zipf", seed=E, dtype=np.int64)
+    ids = make_ids(300_007, E, "zipf", seed=E, dtype=np.int64)
     got = to_np(continuous_count(torch.from_numpy(ids).to(DEV), E))
     assert np.array_equal(got, c_oracle.continuous_count(ids, E))
 
@@ -79,7 +80,7 @@ def test_count_edge_cases():
 )
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 def test_routing_index(T, E, k, kind, empty, dtype):
-    selected, _ = O.make_routing(T, E, k, kind, seed=T + E, empty_tail=empty)
+    selected, _ = make_routing(T, E, k, kind, seed=T + E, empty_tail=empty)
     expect = c_oracle.routing_index(selected.numpy(), E)
     counts, offsets, perm, eid, inv = build_routing_index(selected.to(dtype).to(DEV), E)
     assert np.array_equal(to_np(counts), expect["counts"])

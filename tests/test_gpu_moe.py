@@ -21,6 +21,7 @@ import torch.nn as nn
 
 from fma import KernelBackend, MoE, swiglu_packed
 from oracle import moe_oracle as O
+from synthetic_inputs import make_routing
 
 from gpu_util import DEV, rel_err
 
@@ -170,7 +171,7 @@ def test_moe_benchmark_shapes_against_fp32_oracle_on_gpu(name):
     c = CONFIGS[name]
     T, H, I, E, k = c["T"], c["H"], c["I"], c["E"], c["k"]
     g = torch.Generator().manual_seed(123)
-    selected, weights = O.make_routing(T, E, k, c["kind"], seed=17, empty_tail=c["empty"])
+    selected, weights = make_routing(T, E, k, c["kind"], seed=17, empty_tail=c["empty"])
     x = torch.randn(T, H, generator=g).bfloat16().to(DEV)
     dy = torch.randn(T, H, generator=g).bfloat16().to(DEV)
     moe = MoE(E, k, H, I, swiglu_packed, True, False, 0.02).to(torch.bfloat16).to(DEV)
@@ -206,7 +207,7 @@ def test_moe_size_independent_properties_at_full_shape():
     # token-permutation equivariance and linearity in the router weights, bit-level where the arithmetic allows
     T, H, I, E, k = 8192, 2048, 1408, 64, 8
     g = torch.Generator().manual_seed(5)
-    selected, weights = O.make_routing(T, E, k, "zipf", seed=19, empty_tail=4)
+    selected, weights = make_routing(T, E, k, "zipf", seed=19, empty_tail=4)
     x = torch.randn(T, H, generator=g).bfloat16().to(DEV)
     moe = MoE(E, k, H, I, swiglu_packed, True, False, 0.02).to(torch.bfloat16).to(DEV)
     sel, w = selected.to(DEV), weights.bfloat16().to(DEV)

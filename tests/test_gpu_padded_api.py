@@ -11,6 +11,7 @@ from fma.modules.moe.cuda_implementation import (
     ungroup_with_padding,
 )
 from oracle import moe_oracle as O
+from synthetic_inputs import make_routing
 
 from gpu_util import DEV
 
@@ -29,7 +30,7 @@ def test_padding_offsets_closed_form():
 @pytest.mark.parametrize("pad", [1, 8])
 @pytest.mark.parametrize("T,E,k,H,kind,empty", [(37, 4, 2, 64, "uniform", 0), (200, 16, 4, 128, "zipf", 3)])
 def test_group_and_ungroup_with_padding(pad, T, E, k, H, kind, empty):
-    selected, _ = O.make_routing(T, E, k, kind, seed=3, empty_tail=empty)
+    selected, _ = make_routing(T, E, k, kind, seed=3, empty_tail=empty)
     R = T * k
     freq, _, scattered, sorted_e, _ = build_routing_index(selected.to(DEV), E)
     torch.manual_seed(pad + T)

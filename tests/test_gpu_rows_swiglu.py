@@ -7,6 +7,7 @@ import torch
 from fma import KernelBackend, swiglu, swiglu_packed
 from fma.modules.moe.cuda_implementation import build_routing_index, combine, gather_rows, gather_rows_cuda
 from oracle import moe_oracle as O
+from synthetic_inputs import make_routing
 
 from gpu_util import DEV, rel_err
 
@@ -24,7 +25,7 @@ DTYPES = [torch.float32, torch.float16, torch.bfloat16]
 def test_gather_is_bit_exact(dtype, T, H, E, k):
     torch.manual_seed(T)
     x = torch.randn(T, H).to(dtype)
-    selected, _ = O.make_routing(T, E, k, "uniform", seed=1)
+    selected, _ = make_routing(T, E, k, "uniform", seed=1)
     idx = O.routing_index(selected.numpy(), E)
     _, _, perm, _, inv = build_routing_index(selected.to(DEV), E)
     got = gather_rows(x.to(DEV), perm, inv, k).cpu()  # token-side form (fma_dispatch_rows)
@@ -43,7 +44,7 @@ def test_gather_is_bit_exact(dtype, T, H, E, k):
 )
 def test_combine_forward_and_backward(dtype, T, H, E, k):
     torch.manual_seed(T + k)
-    selected, gates = O.make_routing(T, E, k, "uniform", seed=2)
+    selected, gates = make_routing(T, E, k, "uniform", seed=2)
     idx = O.routing_index(selected.numpy(), E)
     perm = torch.from_numpy(idx["perm"].astype(np.int64))
     o = torch.randn(T * k, H).to(dtype)
@@ -73,7 +74,7 @@ def test_combine_k1_unit_gate_is_the_inverse_permutation():
     T, H, E = 129, 256, 8
     torch.manual_seed(0)
     x = torch.randn(T, H).bfloat16().to(DEV)
-    selected, _ = O.make_routing(T, E, 1, "uniform", seed=3)
+    selected, _ = make_routing(T, E, 1, "uniform", seed=3)
     _, _, perm, _, inv = build_routing_index(selected.to(DEV), E)
     xg = gather_rows(x, perm, inv, 1)
     back = combine(xg, torch.ones(T, 1, dtype=torch.bfloat16, device=DEV), inv)

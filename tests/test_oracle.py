@@ -10,6 +10,7 @@ import torch
 import torch.nn.functional as F
 
 from oracle import c_oracle, moe_oracle as O
+from synthetic_inputs import make_routing
 
 
 # ---- continuous_count --------------------------------------------------------------------------------------
@@ -60,7 +61,7 @@ def test_count_size_one_shortcut():
 @pytest.mark.parametrize("impl", [O.routing_index, c_oracle.routing_index])
 @pytest.mark.parametrize("T,E,k,kind", [(7, 8, 2, "uniform"), (512, 8, 2, "uniform"), (300, 64, 8, "zipf"), (129, 128, 8, "uniform")])
 def test_index_matches_stable_sort(impl, T, E, k, kind):
-    selected, _ = O.make_routing(T, E, k, kind, seed=3, empty_tail=4 if kind == "zipf" else 0)
+    selected, _ = make_routing(T, E, k, kind, seed=3, empty_tail=4 if kind == "zipf" else 0)
     idx = impl(selected.numpy(), E)
     flat = selected.flatten()
     sorted_ids, sorted_slots = flat.sort(stable=True)
@@ -267,7 +268,7 @@ def test_layer_collapses_to_dense_mlp():
     assert torch.allclose(yb, (hb[:, :I] * F.silu(hb[:, I:])) @ w2[0].T + b2[0], atol=1e-5)
     # every expert adds its own bias: with zero weights the output is the gate-weighted sum of the chosen biases
     E, k = 5, 2
-    sel2, gates = O.make_routing(T, E, k, "uniform", seed=3)
+    sel2, gates = make_routing(T, E, k, "uniform", seed=3)
     bias_out = torch.randn(E, H)
     y0 = O.moe_experts(x, gates, sel2, torch.zeros(E, 2 * I, H), torch.zeros(E, H, I), O.swiglu_packed, None, bias_out)
     assert torch.allclose(y0, (gates.unsqueeze(-1) * bias_out[sel2]).sum(1), atol=1e-6)
@@ -280,7 +281,7 @@ def test_layer_against_per_token_loop():
     x = torch.randn(T, H, dtype=torch.float64)
     w1 = torch.randn(E, 2 * I, H, dtype=torch.float64) * 0.3
     w2 = torch.randn(E, H, I, dtype=torch.float64) * 0.3
-    selected, weights = O.make_routing(T, E, k, "uniform", seed=5)
+    selected, weights = make_routing(T, E, k, "uniform", seed=5)
     weights = weights.double()
     y = O.moe_experts(x, weights, selected, w1, w2)
     expect = torch.zeros(T, H, dtype=torch.float64)
@@ -298,7 +299,7 @@ def test_layer_token_permutation_equivariance_and_empty_expert_grads():
     x = torch.randn(T, H, dtype=torch.float64)
     w1 = (torch.randn(E, 2 * I, H, dtype=torch.float64) * 0.3).requires_grad_()
     w2 = (torch.randn(E, H, I, dtype=torch.float64) * 0.3).requires_grad_()
-    selected, weights = O.make_routing(T, E, k, "zipf", seed=7, empty_tail=2)
+    selected, weights = make_routing(T, E, k, "zipf", seed=7, empty_tail=2)
     weights = weights.double()
     y = O.moe_experts(x, weights, selected, w1, w2)
     p = torch.randperm(T)
@@ -312,7 +313,7 @@ def test_layer_token_permutation_equivariance_and_empty_expert_grads():
 def test_layer_gradcheck_fp64():
     torch.manual_seed(8)
     T, H, I, E, k = 6, 4, 4, 3, 2
-    selected, weights = O.make_routing(T, E, k, "uniform", seed=9)
+    selected, weights = make_routing(T, E, k, "uniform", seed=9)
     x = torch.randn(T, H, dtype=torch.float64, requires_grad=True)
     g = weights.double().requires_grad_()
     w1 = (torch.randn(E, 2 * I, H, dtype=torch.float64) * 0.5).requires_grad_()
