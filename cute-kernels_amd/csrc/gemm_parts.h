@@ -109,10 +109,9 @@ __device__ __forceinline__ s16x8 read_kc_frag(const uint8_t* p) { return *reinte
 // 16-byte buffer store of a staged piece. A lane whose offset is not below the descriptor's size stores nothing, so
 // every lane always executes the instruction: the number of stores a wavefront issues per tile is a compile-time
 // constant, which the wait for the next tile's first loads relies on.
-// NT = the non-temporal hint: the output tile is not read again by this kernel, and a workgroup's 128 KB of results
-// should not push operand panels out of the L2 (measured: +0.5 to +1.5 points of peak over plain stores). Only where a
-// store instruction covers whole 128-byte lines: streamed 64-byte pieces are not merged in the L2 and cost a
-// read-modify-write each (measured on the SwiGLU epilogue: +35 % fetched and +28 % written bytes).
+// NT = the non-temporal hint. Measured both ways on the three benchmark layers: with the hint the six GEMMs ran 0.5 to
+// 1.5 points of peak slower than with plain stores (22 of 24 comparisons), and streamed 64-byte pieces are not merged
+// in the L2 and cost a read-modify-write each (SwiGLU epilogue: +35 % fetched and +28 % written bytes). No caller sets it.
 template <bool NT>
 __device__ __forceinline__ void store_tile16(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint4 v) {
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc, (int)voff, 0, NT ? 2 : 0);
@@ -157,7 +156,7 @@ __device__ __forceinline__ void stage_flush(const Slice& img, uint16_t* origin, 
     for (uint32_t it = 0; it < ROWS / kRowsPerInst; ++it) {
         const uint32_t r = it * kRowsPerInst + lane / kChunks;
         const uint4 v = *reinterpret_cast<const uint4*>(img.at(stage_off<ROWB>(r, c16)));
-        store_tile16<(ROWB >= 128)>(rsrc, col_ok ? r * ldb + c16 * 16u : kOutOfRange, v);
+        store_tile16<false>(rsrc, col_ok ? r * ldb + c16 * 16u : kOutOfRange, v);
     }
 }
 
@@ -178,7 +177,7 @@ __device__ __forceinline__ void stage_flush_split(const Slice& img, uint16_t* or
     for (uint32_t it = 0; it < ROWS / kRowsPerInst; ++it) {
         const uint32_t r = it * kRowsPerInst + lane / kChunks;
         const uint4 v = *reinterpret_cast<const uint4*>(img.at(stage_off<ROWB>(r, c16)));
-        store_tile16<(HALF * 2 >= 128)>(rsrc, col_ok ? r * ldb + (window * second0 + in_window) * 2u : kOutOfRange, v);
+        store_tile16<false>(rsrc, col_ok ? r * ldb + (window * second0 + in_window) * 2u : kOutOfRange, v);
     }
 }
 
