@@ -180,8 +180,7 @@ def measure_workload(name, args, full):
     stream = torch.cuda.current_stream().cuda_stream
     BF16 = fma._lib.FMA_BF16
     counts, offsets, perm, eid, inv = ci.build_routing_index(selected_d, E)
-    N_fc, K_fc = moe.c_fc.N_array, moe.c_fc.K_array
-    N_pj, K_pj = moe.c_proj.N_array, moe.c_proj.K_array
+    N_pj, K_pj = moe.c_proj.N_array, moe.c_proj.K_array  # (the fp32 GEMM takes the three arrays)
     w1, w2 = moe.c_fc.weight.detach(), moe.c_proj.weight.detach()
     bf = dict(dtype=torch.bfloat16, device=dev)
     xg = torch.empty(R, H, **bf)
@@ -206,9 +205,12 @@ def measure_workload(name, args, full):
         if rc != 0:
             raise RuntimeError(lib.fma_last_error_string().decode())
 
-    def gemm(A, B, D, M, N, K, ta, tb):
-        ok(lib.fma_grouped_gemm(A.data_ptr(), B.data_ptr(), D.data_ptr(), M.data_ptr(), N.data_ptr(), K.data_ptr(),
-                                E, ta, tb, 1.0, BF16, stream))
+    VARY_M, VARY_K = fma._lib.FMA_VARY_M, fma._lib.FMA_VARY_K
+
+    def gemm(A, B, D, sizes, vary, m, n, kk, ta, tb):
+        # as the layer launches it: one size array (rows per expert) and the two dimensions all experts share by value
+        ok(lib.fma_grouped_gemm_ragged(A.data_ptr(), B.data_ptr(), D.data_ptr(), sizes.data_ptr(), E, vary, m, n, kk,
+                                       ta, tb, 1.0, BF16, stream))
 
     ok(lib.fma_gather_rows(x.data_ptr(), perm.data_ptr(), R, H, k, xg.data_ptr(), BF16, stream))
     iters = max(20, args.steps)
@@ -250,17 +252,17 @@ def measure_workload(name, args, full):
                                                   counts.data_ptr(), E, I, H, BF16, stream)),
          nbytes=R * H * s + w1_b + R * I * s)
     # the unfused pair the fused kernel above replaces (same bits): plain up-projection, then swiglu_forward below
-    mfma("up_projection_plain_fwd(NT)", 2.0 * R * 2 * I * H, lambda i: gemm(xg, w1, h, counts, N_fc, K_fc, 0, 1),
+    mfma("up_projection_plain_fwd(NT)", 2.0 * R * 2 * I * H, lambda i: gemm(xg, w1, h, counts, VARY_M, 0, 2 * I, H, 0, 1),
          nbytes=R * H * s + w1_b + R * 2 * I * s)
-    mfma("down_projection_fwd(NT)", 2.0 * R * I * H, lambda i: gemm(a, w2, o, counts, N_pj, K_pj, 0, 1),
+    mfma("down_projection_fwd(NT)", 2.0 * R * I * H, lambda i: gemm(a, w2, o, counts, VARY_M, 0, H, I, 0, 1),
          nbytes=R * I * s + w2_b + R * H * s)
-    mfma("down_projection_dgrad(NN)", 2.0 * R * I * H, lambda i: gemm(d_o, w2, da, counts, K_pj, N_pj, 0, 0),
+    mfma("down_projection_dgrad(NN)", 2.0 * R * I * H, lambda i: gemm(d_o, w2, da, counts, VARY_M, 0, I, H, 0, 0),
          nbytes=R * H * s + w2_b + R * I * s)
-    mfma("down_projection_wgrad(TN)", 2.0 * R * I * H, lambda i: gemm(d_o, a, dw2, N_pj, K_pj, counts, 1, 0),
+    mfma("down_projection_wgrad(TN)", 2.0 * R * I * H, lambda i: gemm(d_o, a, dw2, counts, VARY_K, H, I, 0, 1, 0),
          nbytes=R * H * s + R * I * s + w2_b)
-    mfma("up_projection_dgrad(NN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, w1, dxg, counts, K_fc, N_fc, 0, 0),
+    mfma("up_projection_dgrad(NN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, w1, dxg, counts, VARY_M, 0, H, 2 * I, 0, 0),
          nbytes=R * 2 * I * s + w1_b + R * H * s)
-    mfma("up_projection_wgrad(TN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, xg, dw1, N_fc, K_fc, counts, 1, 0),
+    mfma("up_projection_wgrad(TN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, xg, dw1, counts, VARY_K, 2 * I, H, 0, 1, 0),
          nbytes=R * 2 * I * s + R * H * s + w1_b)
 
     # the fp32 grouped GEMM (fp32 matrix instruction, 157.3 TFLOP/s peak) on the down-projection's forward shape;
@@ -284,7 +286,7 @@ def measure_workload(name, args, full):
         lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), None, a.data_ptr(),
                                                  counts_dec.data_ptr(), E, I, H, BF16, stream)), n=30, gemm_kernel=True)
     hbm(f"small_batch_down_fwd(NT, {M_dec} rows per expert)", w2_b + R_dec * (H + I) * s,
-        lambda i: gemm(a, w2, o, counts_dec, N_pj, K_pj, 0, 1), n=30, gemm_kernel=True)
+        lambda i: gemm(a, w2, o, counts_dec, VARY_M, 0, H, I, 0, 1), n=30, gemm_kernel=True)
 
     # calibration for the profiler's FETCH_SIZE / WRITE_SIZE counters: a plain device copy of known size (ATen's
     # elementwise copy kernel): reads 1 GiB, writes 1 GiB

@@ -51,7 +51,7 @@ def _headers() -> list[str]:
 # Sources whose kernels count their own outstanding memory operations (s_waitcnt vmcnt(N) with hand-counted N): a
 # register spill would add loads and stores of its own and shift those counts, so that LDS stages could be read before
 # the operands have landed. Their kernels must use no scratch memory; the build checks the compiler's resource report.
-NO_SCRATCH_SOURCES = {"grouped_gemm.hip": "grouped_gemm_kernel"}
+NO_SCRATCH_SOURCES = {"grouped_gemm.hip": "grouped_gemm_kernel", "grouped_gemm_ragged.hip": "ragged_gemm_kernel"}
 
 
 def _check_no_scratch(src: str, report: str, kernel_substring: str) -> None:

@@ -152,12 +152,17 @@ __device__ __forceinline__ void stage_flush(const Slice& img, uint16_t* origin, 
     const uint32_t ldb = ld * 2u;
     const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(origin, rows_valid * ldb);
     const bool col_ok = c16 * 8u < cols_valid;
+    // The image is written as 8-byte and read as 16-byte vectors: two types that type-based alias analysis treats as
+    // never overlapping, so without these fences the compiler may move the reads above the writes that feed them (or the
+    // next image's writes above these reads). The LDS itself executes a wavefront's accesses in order.
+    asm volatile("" ::: "memory");
 #pragma unroll
     for (uint32_t it = 0; it < ROWS / kRowsPerInst; ++it) {
         const uint32_t r = it * kRowsPerInst + lane / kChunks;
         const uint4 v = *reinterpret_cast<const uint4*>(img.at(stage_off<ROWB>(r, c16)));
         store_tile16<false>(rsrc, col_ok ? r * ldb + c16 * 16u : kOutOfRange, v);
     }
+    asm volatile("" ::: "memory");
 }
 
 // Like stage_flush for an image whose row holds two windows of HALF columns each: window 0 goes to columns 0.. of the
@@ -173,13 +178,244 @@ __device__ __forceinline__ void stage_flush_split(const Slice& img, uint16_t* or
     const uint32_t ldb = ld * 2u;
     const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(origin, rows_valid * ldb);
     const bool col_ok = in_window < cols_valid;
+    asm volatile("" ::: "memory");  // (see stage_flush)
 #pragma unroll
     for (uint32_t it = 0; it < ROWS / kRowsPerInst; ++it) {
         const uint32_t r = it * kRowsPerInst + lane / kChunks;
         const uint4 v = *reinterpret_cast<const uint4*>(img.at(stage_off<ROWB>(r, c16)));
         store_tile16<false>(rsrc, col_ok ? r * ldb + (window * second0 + in_window) * 2u : kOutOfRange, v);
     }
+    asm volatile("" ::: "memory");
 }
+
+// The same staging written in assembly, for an epilogue that runs while direct-to-LDS loads of the next tile are in
+// flight: the compiler orders every LDS store of its own behind all such loads (s_waitcnt vmcnt), whatever LDS object they
+// write, which would make the epilogue wait for the operands of the next tile. The LDS executes a wavefront's accesses
+// in order, so the reads below see the writes above them without any wait; each flush waits for its own reads.
+// `image` is the LDS byte address of the wavefront's staging slice.
+template <int ROWB>
+__device__ __forceinline__ void stage_put_quiet(uint32_t image, uint32_t m, uint32_t col, uint2 v) {
+    const uint32_t addr = image + stage_off<ROWB>(m, col >> 3) + ((col >> 2) & 1u) * 8u;
+    asm volatile("ds_write_b64 %0, %1" ::"v"(addr), "v"(__builtin_bit_cast(uint64_t, v)) : "memory");
+}
+// two 16-byte reads of the image (at byte offsets off0 and off1), complete on return
+__device__ __forceinline__ void stage_get2_quiet(uint32_t image, uint32_t off0, uint32_t off1, u32x4& v0, u32x4& v1) {
+    asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %3\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&v"(v0), "=&v"(v1)
+                 : "v"(image + off0), "v"(image + off1)
+                 : "memory");
+}
+// stage_flush for images of exactly two store instructions (ROWS * ROWB == 2048)
+template <int ROWB, int ROWS>
+__device__ __forceinline__ void stage_flush_quiet(uint32_t image, uint16_t* origin, uint32_t ld, uint32_t rows_valid,
+                                                  uint32_t cols_valid, uint32_t lane) {
+    constexpr uint32_t kChunks = ROWB / 16;
+    constexpr uint32_t kRowsPerInst = 64 / kChunks;
+    static_assert(ROWS == 2 * kRowsPerInst, "two store instructions per image");
+    const uint32_t c16 = lane % kChunks;
+    const uint32_t ldb = ld * 2u;
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(origin, rows_valid * ldb);
+    const bool col_ok = c16 * 8u < cols_valid;
+    const uint32_t r0 = lane / kChunks, r1 = kRowsPerInst + lane / kChunks;
+    u32x4 v0, v1;
+    stage_get2_quiet(image, stage_off<ROWB>(r0, c16), stage_off<ROWB>(r1, c16), v0, v1);
+    store_tile16<false>(rsrc, col_ok ? r0 * ldb + c16 * 16u : kOutOfRange, __builtin_bit_cast(uint4, v0));
+    store_tile16<false>(rsrc, col_ok ? r1 * ldb + c16 * 16u : kOutOfRange, __builtin_bit_cast(uint4, v1));
+}
+template <int ROWB, int ROWS, int HALF>
+__device__ __forceinline__ void stage_flush_split_quiet(uint32_t image, uint16_t* origin, uint32_t ld, uint32_t rows_valid,
+                                                        uint32_t cols_valid, uint32_t second0, uint32_t lane) {
+    constexpr uint32_t kChunks = ROWB / 16;
+    constexpr uint32_t kRowsPerInst = 64 / kChunks;
+    static_assert(ROWS == 2 * kRowsPerInst, "two store instructions per image");
+    const uint32_t c16 = lane % kChunks;
+    const uint32_t in_window = (c16 * 8u) % HALF;
+    const uint32_t window = (c16 * 8u) / HALF;
+    const uint32_t ldb = ld * 2u;
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(origin, rows_valid * ldb);
+    const bool col_ok = in_window < cols_valid;
+    const uint32_t r0 = lane / kChunks, r1 = kRowsPerInst + lane / kChunks;
+    const uint32_t col_off = (window * second0 + in_window) * 2u;
+    u32x4 v0, v1;
+    stage_get2_quiet(image, stage_off<ROWB>(r0, c16), stage_off<ROWB>(r1, c16), v0, v1);
+    store_tile16<false>(rsrc, col_ok ? r0 * ldb + col_off : kOutOfRange, __builtin_bit_cast(uint4, v0));
+    store_tile16<false>(rsrc, col_ok ? r1 * ldb + col_off : kOutOfRange, __builtin_bit_cast(uint4, v1));
+}
+
+// ---- tile geometry and the two LDS layouts of an operand tile ----------------------------------------------------
+constexpr int BM = 256;
+constexpr int BN = 256;
+constexpr int BK = 64;
+constexpr int kRowBytes = BK * 2;           // 128: row of a [row][64 k] tile
+constexpr int kTRowBytes = BM * 2;          // 512: row of a [64 k][256 out] tile
+constexpr int kTileBytes = BM * kRowBytes;  // 32 KB per operand per stage, either layout
+constexpr int kGroupM = 8;                  // m-tiles that share one column sweep of the tile order
+constexpr int kXcds = 8;
+
+__device__ __forceinline__ uint32_t phys_row(uint32_t r) { return (r & ~15u) | ((r & 7u) << 1) | ((r >> 3) & 1u); }
+__device__ __forceinline__ uint32_t logical_row(uint32_t pr) {
+    return (pr & ~15u) | ((pr & 15u) >> 1) | ((pr & 1u) << 3);
+}
+// [row][64 k] tile: byte offset of 16-byte chunk `chunk` of row r
+__device__ __forceinline__ uint32_t kc_off(uint32_t r, uint32_t chunk) {
+    return phys_row(r) * kRowBytes + ((chunk ^ (r & 7u)) << 4);
+}
+// [64 k][256 out] tile: byte offset, for k slice 0, of the first transposing read of the fragment that starts at out
+// row r0 (a multiple of 32). Slice ks adds 16 rows, the second read of a fragment (k + 4) adds 4 rows.
+__device__ __forceinline__ uint32_t mc_frag_off(uint32_t r0, uint32_t lane) {
+    const uint32_t g = lane >> 4, j = lane & 15u;
+    const uint32_t q = j & 3u, kr = j >> 2;
+    const uint32_t chunk = (r0 >> 3) + 2u * (g & 1u) + (q >> 1);
+    return (8u * (g >> 1) + kr) * kTRowBytes + ((chunk ^ (4u * kr)) << 4) + (q & 1u) * 8u;
+}
+
+// Operand with the reduction dimension contiguous: tile [256 rows][64 k]. A wavefront instruction moves 8 physical rows
+// (1 KB); NI instructions per wavefront and K step. SPLIT: tile rows 128..255 come from a second row range (base1).
+template <int NW, bool SPLIT>
+struct LoaderK {
+    static constexpr int NI = 32 / NW;
+    static constexpr uint32_t kRowsPerInst = NW * 8;
+    const uint16_t* base0;  // first element of tile row 0
+    const uint16_t* base1;  // SPLIT: first element of tile row 128
+    uint32_t bytes;         // valid bytes from a base: rows inside the operand x row pitch
+    uint32_t ldb;           // row pitch in bytes
+    uint32_t voff;          // this lane's offset: its row of instruction 0, its 16-byte chunk
+    uint32_t chunk;         // this lane's logical chunk (the same for every instruction)
+    uint32_t kdim;
+    uint32_t wave;
+
+    // rows_valid: rows of the tile (of each half when SPLIT) that exist in the operand; the rest arrives as zeros
+    __device__ __forceinline__ void setup(const uint16_t* b0, const uint16_t* b1, uint32_t rows_valid, uint32_t kdim_,
+                                          uint32_t wave_, uint32_t lane) {
+        static_assert(NW % 2 == 0, "chunk is per lane only for an even number of wavefronts");
+        base0 = b0;
+        base1 = b1;
+        kdim = kdim_;
+        wave = wave_;
+        ldb = kdim_ * 2u;
+        bytes = rows_valid * ldb;
+        const uint32_t r = logical_row(wave_ * 8u + (lane >> 3));
+        chunk = (lane & 7u) ^ (r & 7u);
+        voff = r * ldb + chunk * 16u;
+    }
+
+    __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0) const { issue_range<0, NI>(tile, k0); }
+    // instructions I0 .. I1-1 of the K step at k0
+    template <int I0, int I1>
+    __device__ __forceinline__ void issue_range(uint8_t* tile, uint32_t k0) const {
+        uint32_t v = voff;
+        // last, partial K step: chunks past the end of K are pushed out of range, which zero-fills them
+        if (k0 + BK > kdim && k0 + chunk * 8u >= kdim) v = kOutOfRange;
+        const __amdgpu_buffer_rsrc_t r0 = make_rsrc(base0, bytes);
+        const __amdgpu_buffer_rsrc_t r1 = make_rsrc(SPLIT ? base1 : base0, bytes);
+#pragma unroll
+        for (int i = I0; i < I1; ++i) {
+            const bool second = SPLIT && i >= NI / 2;
+            const uint32_t row = (uint32_t)(second ? i - NI / 2 : i) * kRowsPerInst;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(second ? r1 : r0, (lds_void*)(tile + (i * NW + wave) * 1024), 16, v,
+                                                     k0 * 2u + row * ldb, 0, 0);
+        }
+    }
+    // the same NI loads through buffer_load_lds_quiet
+    __device__ __forceinline__ void issue_quiet(uint8_t* tile, uint32_t k0) const {
+        uint32_t v = voff;
+        if (k0 + BK > kdim && k0 + chunk * 8u >= kdim) v = kOutOfRange;
+        const u32x4 r0 = make_rsrc_words(base0, bytes);
+        const u32x4 r1 = make_rsrc_words(SPLIT ? base1 : base0, bytes);
+        const uint32_t lds0 = lds_address(tile) + wave * 1024u;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const bool second = SPLIT && i >= NI / 2;
+            const uint32_t row = (uint32_t)(second ? i - NI / 2 : i) * kRowsPerInst;
+            buffer_load_lds_quiet(second ? r1 : r0, v, k0 * 2u + row * ldb, lds0 + (uint32_t)(i * NW) * 1024u);
+        }
+    }
+    // only the instruction that covers tile rows 0 .. NW*8-1, to the LDS address lds_base (a tile with few rows)
+    __device__ __forceinline__ void issue_quiet_first_rows(uint32_t lds_base, uint32_t k0) const {
+        uint32_t v = voff;
+        if (k0 + BK > kdim && k0 + chunk * 8u >= kdim) v = kOutOfRange;
+        buffer_load_lds_quiet(make_rsrc_words(base0, bytes), v, k0 * 2u, lds_base + wave * 1024u);
+    }
+    // the NI loads with the first half of the tile's 1 KB pieces going to lds_lo and the second half to lds_hi
+    __device__ __forceinline__ void issue_quiet_halves(uint32_t lds_lo, uint32_t lds_hi, uint32_t k0) const {
+        uint32_t v = voff;
+        if (k0 + BK > kdim && k0 + chunk * 8u >= kdim) v = kOutOfRange;
+        const u32x4 r0 = make_rsrc_words(base0, bytes);
+        const u32x4 r1 = make_rsrc_words(SPLIT ? base1 : base0, bytes);
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const bool second = SPLIT && i >= NI / 2;
+            const uint32_t row = (uint32_t)(second ? i - NI / 2 : i) * kRowsPerInst;
+            const uint32_t lds = (i < NI / 2 ? lds_lo + (uint32_t)(i * NW) * 1024u : lds_hi + (uint32_t)((i - NI / 2) * NW) * 1024u) + wave * 1024u;
+            buffer_load_lds_quiet(second ? r1 : r0, v, k0 * 2u + row * ldb, lds);
+        }
+    }
+};
+
+// Operand stored [reduction][out] (out contiguous): tile [64 k][256 out]. A wavefront instruction moves two k rows
+// (2 x 512 B). Rows past the end of the reduction are out of the descriptor's range (zeros); columns past the end of
+// the operand's rows read whatever follows, which only reaches outputs that are never stored.
+template <int NW>
+struct LoaderT {
+    static constexpr int NI = 32 / NW;
+    const uint16_t* base;  // row 0 of the group's operand, first column of the tile
+    uint32_t ldb;          // row pitch in bytes
+    uint32_t col_bytes;    // byte offset of the tile's first column inside a row
+    uint32_t voff;
+    uint32_t kdim;
+    uint32_t wave;
+
+    __device__ __forceinline__ void setup(const uint16_t* group_base, uint32_t ld, uint32_t kdim_, uint32_t out0,
+                                          uint32_t wave_, uint32_t lane) {
+        base = group_base + out0;
+        ldb = ld * 2u;
+        col_bytes = out0 * 2u;
+        kdim = kdim_;
+        wave = wave_;
+        const uint32_t khalf = lane >> 5;  // which of the two rows of an instruction this lane loads
+        const uint32_t krow = wave_ * 2u + khalf;
+        voff = khalf * ldb + (((lane & 31u) ^ (4u * (krow & 3u))) << 4);
+    }
+
+    __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0) const { issue_range<0, NI>(tile, k0); }
+    template <int I0, int I1>
+    __device__ __forceinline__ void issue_range(uint8_t* tile, uint32_t k0) const {
+        // rows of this K step that exist (none at all when the step lies past the end: everything is zero-filled)
+        const uint32_t rows = k0 >= kdim ? 0u : (kdim - k0 < (uint32_t)BK ? kdim - k0 : (uint32_t)BK);
+        const __amdgpu_buffer_rsrc_t r = make_rsrc(base + (uint64_t)k0 * (ldb / 2u), rows ? rows * ldb - col_bytes : 0u);
+#pragma unroll
+        for (int i = I0; i < I1; ++i) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(tile + (i * NW + wave) * 1024), 16, voff,
+                                                     (uint32_t)(i * NW + wave) * 2u * ldb, 0, 0);
+        }
+    }
+    __device__ __forceinline__ void issue_quiet(uint8_t* tile, uint32_t k0) const {
+        const uint32_t rows = k0 >= kdim ? 0u : (kdim - k0 < (uint32_t)BK ? kdim - k0 : (uint32_t)BK);
+        const u32x4 r = make_rsrc_words(base + (uint64_t)k0 * (ldb / 2u), rows ? rows * ldb - col_bytes : 0u);
+        const uint32_t lds0 = lds_address(tile) + wave * 1024u;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            buffer_load_lds_quiet(r, voff, (uint32_t)(i * NW + wave) * 2u * ldb, lds0 + (uint32_t)(i * NW) * 1024u);
+        }
+    }
+    // the NI loads with k rows 0..31 of the step going to lds_lo and k rows 32..63 to lds_hi
+    __device__ __forceinline__ void issue_quiet_halves(uint32_t lds_lo, uint32_t lds_hi, uint32_t k0) const {
+        const uint32_t rows = k0 >= kdim ? 0u : (kdim - k0 < (uint32_t)BK ? kdim - k0 : (uint32_t)BK);
+        const u32x4 r = make_rsrc_words(base + (uint64_t)k0 * (ldb / 2u), rows ? rows * ldb - col_bytes : 0u);
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const uint32_t lds = (i < NI / 2 ? lds_lo + (uint32_t)(i * NW) * 1024u : lds_hi + (uint32_t)((i - NI / 2) * NW) * 1024u) + wave * 1024u;
+            buffer_load_lds_quiet(r, voff, (uint32_t)(i * NW + wave) * 2u * ldb, lds);
+        }
+    }
+};
+
+__device__ __forceinline__ s16x8 read_tr_frag(const uint8_t* p) {
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p + 4 * kTRowBytes));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 
 // Scheduling hint for one k slice: MFMAS matrix instructions with READS LDS reads spread evenly between them.
 template <int R, int MFMAS, int READS>

@@ -31,14 +31,6 @@
 namespace fmahip {
 namespace gemm {
 
-constexpr int BM = 256;
-constexpr int BN = 256;
-constexpr int BK = 64;
-constexpr int kRowBytes = BK * 2;           // 128: row of a [row][64 k] tile
-constexpr int kTRowBytes = BM * 2;          // 512: row of a [64 k][256 out] tile
-constexpr int kTileBytes = BM * kRowBytes;  // 32 KB per operand per stage, either layout
-constexpr int kGroupM = 8;                  // m-tiles that share one column sweep of the tile order
-constexpr int kXcds = 8;
 // how the load instructions of a K step are spread over the slices after the barrier that frees their stage
 #ifndef FMA_PF_DIST
 #define FMA_PF_DIST 4
@@ -73,171 +65,6 @@ struct GemmArgs {
     uint32_t const_k;
     float alpha;
 };
-
-__device__ __forceinline__ uint32_t phys_row(uint32_t r) { return (r & ~15u) | ((r & 7u) << 1) | ((r >> 3) & 1u); }
-__device__ __forceinline__ uint32_t logical_row(uint32_t pr) {
-    return (pr & ~15u) | ((pr & 15u) >> 1) | ((pr & 1u) << 3);
-}
-// [row][64 k] tile: byte offset of 16-byte chunk `chunk` of row r
-__device__ __forceinline__ uint32_t kc_off(uint32_t r, uint32_t chunk) {
-    return phys_row(r) * kRowBytes + ((chunk ^ (r & 7u)) << 4);
-}
-// [64 k][256 out] tile: byte offset, for k slice 0, of the first transposing read of the fragment that starts at out
-// row r0 (a multiple of 32). Slice ks adds 16 rows, the second read of a fragment (k + 4) adds 4 rows.
-__device__ __forceinline__ uint32_t mc_frag_off(uint32_t r0, uint32_t lane) {
-    const uint32_t g = lane >> 4, j = lane & 15u;
-    const uint32_t q = j & 3u, kr = j >> 2;
-    const uint32_t chunk = (r0 >> 3) + 2u * (g & 1u) + (q >> 1);
-    return (8u * (g >> 1) + kr) * kTRowBytes + ((chunk ^ (4u * kr)) << 4) + (q & 1u) * 8u;
-}
-
-// Operand with the reduction dimension contiguous: tile [256 rows][64 k]. A wavefront instruction moves 8 physical rows
-// (1 KB); NI instructions per wavefront and K step. SPLIT: tile rows 128..255 come from a second row range (base1).
-template <int NW, bool SPLIT>
-struct LoaderK {
-    static constexpr int NI = 32 / NW;
-    static constexpr uint32_t kRowsPerInst = NW * 8;
-    const uint16_t* base0;  // first element of tile row 0
-    const uint16_t* base1;  // SPLIT: first element of tile row 128
-    uint32_t bytes;         // valid bytes from a base: rows inside the operand x row pitch
-    uint32_t ldb;           // row pitch in bytes
-    uint32_t voff;          // this lane's offset: its row of instruction 0, its 16-byte chunk
-    uint32_t chunk;         // this lane's logical chunk (the same for every instruction)
-    uint32_t kdim;
-    uint32_t wave;
-
-    // rows_valid: rows of the tile (of each half when SPLIT) that exist in the operand; the rest arrives as zeros
-    __device__ __forceinline__ void setup(const uint16_t* b0, const uint16_t* b1, uint32_t rows_valid, uint32_t kdim_,
-                                          uint32_t wave_, uint32_t lane) {
-        static_assert(NW % 2 == 0, "chunk is per lane only for an even number of wavefronts");
-        base0 = b0;
-        base1 = b1;
-        kdim = kdim_;
-        wave = wave_;
-        ldb = kdim_ * 2u;
-        bytes = rows_valid * ldb;
-        const uint32_t r = logical_row(wave_ * 8u + (lane >> 3));
-        chunk = (lane & 7u) ^ (r & 7u);
-        voff = r * ldb + chunk * 16u;
-    }
-
-    __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0) const { issue_range<0, NI>(tile, k0); }
-    // instructions I0 .. I1-1 of the K step at k0
-    template <int I0, int I1>
-    __device__ __forceinline__ void issue_range(uint8_t* tile, uint32_t k0) const {
-        uint32_t v = voff;
-        // last, partial K step: chunks past the end of K are pushed out of range, which zero-fills them
-        if (k0 + BK > kdim && k0 + chunk * 8u >= kdim) v = kOutOfRange;
-        const __amdgpu_buffer_rsrc_t r0 = make_rsrc(base0, bytes);
-        const __amdgpu_buffer_rsrc_t r1 = make_rsrc(SPLIT ? base1 : base0, bytes);
-#pragma unroll
-        for (int i = I0; i < I1; ++i) {
-            const bool second = SPLIT && i >= NI / 2;
-            const uint32_t row = (uint32_t)(second ? i - NI / 2 : i) * kRowsPerInst;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(second ? r1 : r0, (lds_void*)(tile + (i * NW + wave) * 1024), 16, v,
-                                                     k0 * 2u + row * ldb, 0, 0);
-        }
-    }
-    // the same NI loads through buffer_load_lds_quiet
-    __device__ __forceinline__ void issue_quiet(uint8_t* tile, uint32_t k0) const {
-        uint32_t v = voff;
-        if (k0 + BK > kdim && k0 + chunk * 8u >= kdim) v = kOutOfRange;
-        const u32x4 r0 = make_rsrc_words(base0, bytes);
-        const u32x4 r1 = make_rsrc_words(SPLIT ? base1 : base0, bytes);
-        const uint32_t lds0 = lds_address(tile) + wave * 1024u;
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const bool second = SPLIT && i >= NI / 2;
-            const uint32_t row = (uint32_t)(second ? i - NI / 2 : i) * kRowsPerInst;
-            buffer_load_lds_quiet(second ? r1 : r0, v, k0 * 2u + row * ldb, lds0 + (uint32_t)(i * NW) * 1024u);
-        }
-    }
-    // only the instruction that covers tile rows 0 .. NW*8-1, to the LDS address lds_base (a tile with few rows)
-    __device__ __forceinline__ void issue_quiet_first_rows(uint32_t lds_base, uint32_t k0) const {
-        uint32_t v = voff;
-        if (k0 + BK > kdim && k0 + chunk * 8u >= kdim) v = kOutOfRange;
-        buffer_load_lds_quiet(make_rsrc_words(base0, bytes), v, k0 * 2u, lds_base + wave * 1024u);
-    }
-    // the NI loads with the first half of the tile's 1 KB pieces going to lds_lo and the second half to lds_hi
-    __device__ __forceinline__ void issue_quiet_halves(uint32_t lds_lo, uint32_t lds_hi, uint32_t k0) const {
-        uint32_t v = voff;
-        if (k0 + BK > kdim && k0 + chunk * 8u >= kdim) v = kOutOfRange;
-        const u32x4 r0 = make_rsrc_words(base0, bytes);
-        const u32x4 r1 = make_rsrc_words(SPLIT ? base1 : base0, bytes);
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const bool second = SPLIT && i >= NI / 2;
-            const uint32_t row = (uint32_t)(second ? i - NI / 2 : i) * kRowsPerInst;
-            const uint32_t lds = (i < NI / 2 ? lds_lo + (uint32_t)(i * NW) * 1024u : lds_hi + (uint32_t)((i - NI / 2) * NW) * 1024u) + wave * 1024u;
-            buffer_load_lds_quiet(second ? r1 : r0, v, k0 * 2u + row * ldb, lds);
-        }
-    }
-};
-
-// Operand stored [reduction][out] (out contiguous): tile [64 k][256 out]. A wavefront instruction moves two k rows
-// (2 x 512 B). Rows past the end of the reduction are out of the descriptor's range (zeros); columns past the end of
-// the operand's rows read whatever follows, which only reaches outputs that are never stored.
-template <int NW>
-struct LoaderT {
-    static constexpr int NI = 32 / NW;
-    const uint16_t* base;  // row 0 of the group's operand, first column of the tile
-    uint32_t ldb;          // row pitch in bytes
-    uint32_t col_bytes;    // byte offset of the tile's first column inside a row
-    uint32_t voff;
-    uint32_t kdim;
-    uint32_t wave;
-
-    __device__ __forceinline__ void setup(const uint16_t* group_base, uint32_t ld, uint32_t kdim_, uint32_t out0,
-                                          uint32_t wave_, uint32_t lane) {
-        base = group_base + out0;
-        ldb = ld * 2u;
-        col_bytes = out0 * 2u;
-        kdim = kdim_;
-        wave = wave_;
-        const uint32_t khalf = lane >> 5;  // which of the two rows of an instruction this lane loads
-        const uint32_t krow = wave_ * 2u + khalf;
-        voff = khalf * ldb + (((lane & 31u) ^ (4u * (krow & 3u))) << 4);
-    }
-
-    __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0) const { issue_range<0, NI>(tile, k0); }
-    template <int I0, int I1>
-    __device__ __forceinline__ void issue_range(uint8_t* tile, uint32_t k0) const {
-        // rows of this K step that exist (none at all when the step lies past the end: everything is zero-filled)
-        const uint32_t rows = k0 >= kdim ? 0u : (kdim - k0 < (uint32_t)BK ? kdim - k0 : (uint32_t)BK);
-        const __amdgpu_buffer_rsrc_t r = make_rsrc(base + (uint64_t)k0 * (ldb / 2u), rows ? rows * ldb - col_bytes : 0u);
-#pragma unroll
-        for (int i = I0; i < I1; ++i) {
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(tile + (i * NW + wave) * 1024), 16, voff,
-                                                     (uint32_t)(i * NW + wave) * 2u * ldb, 0, 0);
-        }
-    }
-    __device__ __forceinline__ void issue_quiet(uint8_t* tile, uint32_t k0) const {
-        const uint32_t rows = k0 >= kdim ? 0u : (kdim - k0 < (uint32_t)BK ? kdim - k0 : (uint32_t)BK);
-        const u32x4 r = make_rsrc_words(base + (uint64_t)k0 * (ldb / 2u), rows ? rows * ldb - col_bytes : 0u);
-        const uint32_t lds0 = lds_address(tile) + wave * 1024u;
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            buffer_load_lds_quiet(r, voff, (uint32_t)(i * NW + wave) * 2u * ldb, lds0 + (uint32_t)(i * NW) * 1024u);
-        }
-    }
-    // the NI loads with k rows 0..31 of the step going to lds_lo and k rows 32..63 to lds_hi
-    __device__ __forceinline__ void issue_quiet_halves(uint32_t lds_lo, uint32_t lds_hi, uint32_t k0) const {
-        const uint32_t rows = k0 >= kdim ? 0u : (kdim - k0 < (uint32_t)BK ? kdim - k0 : (uint32_t)BK);
-        const u32x4 r = make_rsrc_words(base + (uint64_t)k0 * (ldb / 2u), rows ? rows * ldb - col_bytes : 0u);
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const uint32_t lds = (i < NI / 2 ? lds_lo + (uint32_t)(i * NW) * 1024u : lds_hi + (uint32_t)((i - NI / 2) * NW) * 1024u) + wave * 1024u;
-            buffer_load_lds_quiet(r, voff, (uint32_t)(i * NW + wave) * 2u * ldb, lds);
-        }
-    }
-};
-
-__device__ __forceinline__ s16x8 read_tr_frag(const uint8_t* p) {
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p);
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p + 4 * kTRowBytes));
-    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
 
 template <typename EL, int NWM, int NWN, bool A_KC, bool B_KC, int EPI>
 __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmArgs args) {
@@ -1030,9 +857,7 @@ constexpr int kWavesN = 4;
     template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, true, true, EPI_PLAIN>(const GemmArgs);  \
     template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, true, false, EPI_PLAIN>(const GemmArgs); \
     template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, false, true, EPI_PLAIN>(const GemmArgs); \
-    template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, false, false, EPI_PLAIN>(const GemmArgs); \
-    template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, true, true, EPI_SWIGLU>(const GemmArgs); \
-    template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, true, true, EPI_SWIGLU_ACT>(const GemmArgs);
+    template __global__ void grouped_gemm_kernel<EL, kWavesM, kWavesN, false, false, EPI_PLAIN>(const GemmArgs);
 FMA_GEMM_INSTANTIATE(ElemBf16)
 FMA_GEMM_INSTANTIATE(ElemF16)
 #undef FMA_GEMM_INSTANTIATE
@@ -1093,44 +918,6 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
     args.E = (uint32_t)E;
     args.alpha = alpha;
     return dtype == FMA_BF16 ? launch_plain<ElemBf16>(args, a_kc, b_kc, st) : launch_plain<ElemF16>(args, a_kc, b_kc, st);
-}
-
-int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, const uint32_t* M_arr, int64_t E,
-                            int64_t I, int64_t K, int dtype, void* stream) {
-    using namespace fmahip;
-    using namespace fmahip::gemm;
-    FMA_REQUIRE(dtype == FMA_BF16 || dtype == FMA_F16, dtype_bytes(dtype) ? FMA_ERR_UNSUPPORTED : FMA_ERR_BAD_DTYPE,
-                "grouped_gemm_swiglu: bf16 and fp16 operands are implemented (dtype code %d)", dtype);
-    FMA_REQUIRE(E >= 0, FMA_ERR_BAD_SIZE, "grouped_gemm_swiglu: negative group count %lld", (long long)E);
-    FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "grouped_gemm_swiglu: E=%lld exceeds the limit %d",
-                (long long)E, FMA_MAX_GROUPS);
-    // the upper bounds are those of the kernel's 32-bit tile offsets; this entry point has no scalar path beyond them
-    FMA_REQUIRE(I >= 8 && I % 8 == 0 && 2 * I < (1ll << 23), FMA_ERR_BAD_SIZE,
-                "grouped_gemm_swiglu: intermediate size %lld must be a positive multiple of 8 below 2^22", (long long)I);
-    FMA_REQUIRE(K >= 8 && K % 8 == 0 && K < (1ll << 21), FMA_ERR_BAD_SIZE,
-                "grouped_gemm_swiglu: K=%lld must be a positive multiple of 8 below 2^21", (long long)K);
-    if (E == 0) return FMA_OK;
-    FMA_REQUIRE(x && W && act && M_arr, FMA_ERR_NULL_POINTER, "grouped_gemm_swiglu: NULL pointer");
-    FMA_REQUIRE(aligned16(x) && aligned16(W) && aligned16(act) && aligned16(h), FMA_ERR_MISALIGNED,
-                "grouped_gemm_swiglu: x, W, h and act must be 16-byte aligned");
-    GemmArgs args{};
-    args.A = (const uint16_t*)x;
-    args.B = (const uint16_t*)W;
-    args.D = (uint16_t*)h;
-    args.ACT = (uint16_t*)act;
-    args.M_arr = M_arr;
-    args.N_arr = nullptr;
-    args.K_arr = nullptr;
-    args.E = (uint32_t)E;
-    args.const_n = (uint32_t)(2 * I);
-    args.const_k = (uint32_t)K;
-    args.alpha = 1.0f;
-    // whether h is stored is a compile-time property of the kernel: the epilogue is then one straight-line block
-    if (h)
-        return dtype == FMA_BF16 ? launch<ElemBf16, true, true, EPI_SWIGLU>(args, (hipStream_t)stream)
-                                 : launch<ElemF16, true, true, EPI_SWIGLU>(args, (hipStream_t)stream);
-    return dtype == FMA_BF16 ? launch<ElemBf16, true, true, EPI_SWIGLU_ACT>(args, (hipStream_t)stream)
-                             : launch<ElemF16, true, true, EPI_SWIGLU_ACT>(args, (hipStream_t)stream);
 }
 
 }  // extern "C"

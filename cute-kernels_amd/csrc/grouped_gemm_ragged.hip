@@ -1,0 +1,955 @@
+// Grouped GEMM for launches whose groups differ in ONE dimension (every grouped GEMM of an MoE layer: rows per expert
+// in forward and input gradient, reduction length per expert in the weight gradient) for gfx950: bf16 or fp16 operands,
+// fp32 accumulation on the matrix cores, optional SwiGLU epilogue. The tile kernel of grouped_gemm.hip (256x256x64
+// tiles, eight wavefronts, two LDS stages filled by direct global -> LDS loads, the same LDS layouts and K loop) with a
+// different tile boundary:
+//
+//  * With two dimensions known on the host, a group's operand offsets follow from one 32-bit prefix of the varying
+//    dimension, so the group table takes 10 bytes per group instead of 30. The LDS that frees (16 KB) is a staging
+//    buffer of its own for the epilogue, which therefore no longer needs a piece of an operand stage.
+//  * The operand loads run as ONE stream over the tile sequence: the load slots of a tile's last two K steps carry the
+//    first two K steps of the NEXT tile (the loaders of both tiles are kept, a scalar select picks one per step), so that
+//    when a tile's K loop ends the next tile's first step is already in LDS and its second on the way. The tile boundary
+//    is then the epilogue alone: no loader set-up, no burst of 16 loads per wavefront competing with the 16 stores for the
+//    compute unit's one address path, no wait for first operands, no barrier.
+//  * The epilogue's stores stay outstanding across the start of the next tile: they are issued after that tile's first
+//    loads, and loads and stores of a wavefront complete in issue order, so the first K step waits for "all but the
+//    stores and the newest prefetch" (an exact count) and the second for everything, two K steps after the stores went out.
+//  * A K loop always runs an even number of steps (a step of zeros is appended to an odd reduction length), so every tile
+//    starts in LDS stage 0 and the loop body stays two straight-line steps.
+//  * Tiles that break the pattern (groups of at most 64 rows on their three-stage loop, groups without reduction, groups
+//    that need the element-wise path) start cold: the tile before them lets its last two load slots fetch nothing and
+//    drains, and they issue their first loads themselves, followed by as many stores outside every buffer as an epilogue
+//    issues, so that the waits of the K loop are the same constants in both cases.
+#include "gemm_parts.h"
+
+namespace fmahip {
+namespace gemm {
+namespace ragged {
+
+#ifndef FMA_PF_DIST
+#define FMA_PF_DIST 4
+#endif
+constexpr uint32_t kPfDist = FMA_PF_DIST;  // K steps between a line's prefetch and the step that loads it
+
+constexpr int NWM = 2, NWN = 4, NW = NWM * NWN, NT = NW * 64;
+constexpr int WM = BM / NWM, WN = BN / NWN;  // 128 x 64 per wavefront
+constexpr int FM = WM / 32, FN = WN / 32;    // 4 x 2 accumulator blocks of 32 x 32
+constexpr int kStageBytes = 2048;            // epilogue staging per wavefront: 16 rows of 128 bytes or 32 rows of 64
+
+struct Args {
+    const uint16_t* A;
+    const uint16_t* B;
+    uint16_t* D;            // plain: output; swiglu: pre-activation h (may be NULL)
+    uint16_t* ACT;          // swiglu only: activation output
+    const uint32_t* sizes;  // E values of the varying dimension
+    uint32_t E;
+    uint32_t m, n, k;  // the dimensions all groups share (the varying one is ignored)
+    float alpha;
+};
+
+// s_waitcnt immediate: vmcnt(vm), and lgkmcnt(0) too if lgkm0 (expcnt untouched)
+constexpr int waitcnt_imm(int vm, bool lgkm0) {
+    return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | ((lgkm0 ? 0 : 15) << 8);
+}
+
+// The per-tile part of a loader's state (everything else depends on lane, wavefront and the shared dimensions only)
+template <bool KC>
+struct Feed {
+    const uint16_t* base0;
+    const uint16_t* base1;  // second row range of a split [row][k] tile
+    uint32_t extent;        // [row][k] tile: valid bytes from a base; [k][out] tile: reduction length
+    uint32_t ldb;           // row pitch of the operand in bytes
+    uint32_t col_bytes;     // [k][out] tile: byte offset of the tile's first column inside a row
+};
+
+#ifdef FMA_PROF
+__device__ unsigned long long fma_prof[1024 * 8 * 8];
+#define PROF_STAMP(t) asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t))
+#endif
+
+template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K>
+__global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
+    static_assert(EPI == EPI_PLAIN || (A_KC && B_KC && !VARY_K), "the SwiGLU epilogue exists for the NT layout only");
+
+    // one array per stage and operand: distinct LDS objects let the compiler see that a direct-to-LDS load
+    // into one stage cannot alias the fragment reads of the other, so it does not wait for the load first
+    __shared__ __attribute__((aligned(1024))) uint8_t s_a0[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t s_b0[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t s_a1[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t s_b1[kTileBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t s_stage[NW * kStageBytes];
+    __shared__ uint32_t s_pf[64];  // where the dwords fetched by the L2 prefetch end up (never read)
+    // The group table, one LDS object: first tile of the group at position p of the tile sequence, exclusive prefix of the
+    // varying dimension over the groups, and which group is at position p.
+    __shared__ uint32_t s_table[2 * (FMA_MAX_GROUPS + 1) + FMA_MAX_GROUPS / 2];
+    uint32_t* const s_tile_start = s_table;
+    uint32_t* const s_prefix = s_table + (FMA_MAX_GROUPS + 1);
+    uint16_t* const s_order = reinterpret_cast<uint16_t*>(s_table + 2 * (FMA_MAX_GROUPS + 1));
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wm = wave / NWN;
+    const uint32_t wn = wave % NWN;
+    const uint32_t E = args.E;
+
+    // The compiler orders LDS accesses behind direct-to-LDS loads in flight per LDS object: an access to an object that
+    // some load has written waits for the loads into THAT object only, an access to an object no load has ever written
+    // waits for all of them. The group table is read while the next tile's operand loads are in flight, so it gets
+    // one load that fetches nothing, here, to be known as an object of its own.
+    {
+        const __amdgpu_buffer_rsrc_t nowhere = make_rsrc(args.A, 0u);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(nowhere, (lds_void*)s_table, 4, kOutOfRange, 0, 0, 0);
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, false));
+        __syncthreads();
+    }
+
+    // The size array is read through the constant address space: with a wavefront-uniform index that is a scalar load
+    // (nothing writes the array while the kernel runs), not a vector load that every tile would wait for.
+    typedef const __attribute__((address_space(4))) uint32_t* const_u32_ptr;
+    const const_u32_ptr sizes = (const_u32_ptr)args.sizes;
+    auto group_m = [&](uint32_t e) { return VARY_K ? args.m : sizes[e]; };
+    auto group_k = [&](uint32_t e) { return VARY_K ? sizes[e] : args.k; };
+    const uint32_t Ne = args.n;
+    constexpr bool kCanNarrow = A_KC && B_KC;
+    constexpr uint32_t kTileN = EPI != EPI_PLAIN ? BN / 2 : BN;  // columns of the tile grid one tile covers
+    const uint32_t n_span = EPI != EPI_PLAIN ? Ne / 2 : Ne;      // columns the tile grid runs over
+    bool narrow = false;
+    auto tiles_of = [&](uint32_t m) -> uint32_t {
+        if (m == 0 || Ne == 0) return 0;
+        const uint32_t width = (kCanNarrow && narrow && m <= 64u) ? kTileN / 2 : kTileN;
+        return ((m + BM - 1) / BM) * ((n_span + width - 1) / width);
+    };
+
+    // ---- order of the groups in the tile sequence: by K steps per tile, longest first (see grouped_gemm.hip) ----
+    {
+        uint32_t* const key = reinterpret_cast<uint32_t*>(s_a0);  // K steps per tile of group e; 0 if it has no tiles
+        const uint32_t key0 = tiles_of(group_m(0)) ? (group_k(0) + BK - 1) / BK : 0u;
+        bool differs = false;
+        for (uint32_t e = tid; e < E; e += NT) {
+            const uint32_t k = tiles_of(group_m(e)) ? (group_k(e) + BK - 1) / BK : 0u;
+            key[e] = k;
+            differs = differs || k != key0;
+        }
+        if (__syncthreads_or(differs)) {
+            for (uint32_t e = tid; e < E; e += NT) {
+                const uint32_t mine = key[e];
+                uint32_t rank = 0;
+                for (uint32_t j = 0; j < E; ++j) {
+                    const uint32_t other = key[j];
+                    rank += (other > mine || (other == mine && j < e)) ? 1u : 0u;
+                }
+                s_order[rank] = (uint16_t)e;
+            }
+        } else {
+            for (uint32_t e = tid; e < E; e += NT) s_order[e] = (uint16_t)e;
+        }
+        __syncthreads();
+    }
+
+    if constexpr (kCanNarrow) {
+        // half-width column tiles for groups of at most 64 rows when that fills the workgroups better (grouped_gemm.hip)
+        uint32_t mine_small = 0, mine_other = 0;
+        for (uint32_t e = tid; e < E; e += NT) {
+            const uint32_t m = group_m(e), t = tiles_of(m);
+            if (m <= 64u) mine_small += t;
+            else mine_other += t;
+        }
+        uint32_t* const total = reinterpret_cast<uint32_t*>(s_a0);
+        if (tid < 2) total[tid] = 0;
+        __syncthreads();
+        if (mine_small) atomicAdd(total, mine_small);
+        if (mine_other) atomicAdd(total + 1, mine_other);
+        __syncthreads();
+        const uint32_t t_small = uniform(total[0]), t_other = uniform(total[1]), g = gridDim.x;
+        const uint32_t rounds = (t_small + t_other + g - 1) / g;
+        const uint32_t half_rounds = (2 * t_small + g - 1) / g;
+        narrow = t_other == 0 ? half_rounds * 10u <= 2u * rounds * 9u : (t_small + t_other) * 2u <= g;
+        __syncthreads();
+    }
+
+    // ---- group table, built by wavefront 0: exclusive prefix of tiles over the order above, exclusive prefix of the
+    // varying dimension over the groups as they lie in memory ----
+    if (wave == 0) {
+        uint32_t carry_t = 0, carry_s = 0;
+        for (uint32_t base = 0; base < E; base += 64) {
+            const uint32_t e = base + lane;
+            uint32_t sz = 0, t = 0;
+            if (e < E) {
+                sz = sizes[e];
+                t = tiles_of(group_m(s_order[e]));  // the group at position e of the tile sequence
+            }
+            const uint32_t it = wave_inclusive_scan<uint32_t>(t);
+            const uint32_t is = wave_inclusive_scan<uint32_t>(sz);
+            if (e < E) {
+                s_tile_start[e] = carry_t + it - t;
+                s_prefix[e] = carry_s + is - sz;
+            }
+            carry_t += __shfl(it, 63, 64);
+            carry_s += __shfl(is, 63, 64);
+        }
+        if (lane == 0) {
+            s_tile_start[E] = carry_t;
+            s_prefix[E] = carry_s;
+        }
+    }
+    __syncthreads();
+    const uint32_t total_tiles = s_tile_start[E];
+
+    // first tile row of B fragment j of this wavefront
+    auto b_frag_row = [&](int j) -> uint32_t {
+        if constexpr (EPI != EPI_PLAIN) {
+            return j < FN / 2 ? wn * (WN / 2) + j * 32 : BN / 2 + wn * (WN / 2) + (j - FN / 2) * 32;
+        } else {
+            return wn * WN + j * 32;
+        }
+    };
+    // per-lane LDS byte offsets of this wavefront's fragments for k slice 0 (slice ks adds a constant)
+    uint32_t a_off[FM], b_off[FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        const uint32_t r0 = wm * WM + i * 32;
+        a_off[i] = A_KC ? r0 * kRowBytes : mc_frag_off(r0, lane);
+    }
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+        const uint32_t r0 = b_frag_row(j);
+        b_off[j] = B_KC ? r0 * kRowBytes : mc_frag_off(r0, lane);
+    }
+    uint32_t kc_slice[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) kc_slice[ks] = kc_off(lane & 31u, (uint32_t)ks * 2u + (lane >> 5));
+
+    // workgroup id -> position in the round of gridDim.x tiles: workgroups of one XCD take 32 neighbours
+    const uint32_t grid = gridDim.x;
+    const uint32_t per_xcd = grid / kXcds;
+    const uint32_t slot = (grid % kXcds == 0) ? (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds : blockIdx.x;
+
+    // Everything that identifies one output tile; the same in every lane.
+    struct Tile {
+        bool valid, fast;
+        uint32_t Me, Ke, m0, n0, n_lim;  // n_lim: first column past the tile (kTileN columns wide, or half of that)
+        uint64_t off_a, off_b, off_d;
+        uint32_t pf_r, pf_c;  // position of the tile in its XCD's 8 x 4 block of tiles (row, column)
+    };
+    auto lookup = [&](uint32_t round) -> Tile {
+        Tile t{};
+        const uint32_t v = round * grid + ((round & 1u) ? grid - 1u - slot : slot);
+        if ((uint64_t)round * grid >= total_tiles || v >= total_tiles) return t;
+        uint32_t lo = 0, hi = E;
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (s_tile_start[mid + 1] <= v) lo = mid + 1;
+            else hi = mid;
+        }
+        const uint32_t pos = uniform(lo);
+        const uint32_t e = uniform((uint32_t)s_order[pos]);
+        t.valid = true;
+        t.Me = group_m(e);
+        t.Ke = group_k(e);
+        const uint32_t tiles_m = (t.Me + BM - 1) / BM;
+        const uint32_t tile_n = (kCanNarrow && narrow && t.Me <= 64u) ? kTileN / 2 : kTileN;
+        const uint32_t tiles_n = (n_span + tile_n - 1) / tile_n;
+        const uint32_t local = v - uniform(s_tile_start[pos]);
+        const uint32_t band = kGroupM * tiles_n;
+        const uint32_t first_m = (local / band) * kGroupM;
+        const uint32_t band_m = tiles_m - first_m < (uint32_t)kGroupM ? tiles_m - first_m : (uint32_t)kGroupM;
+        const uint32_t mt = first_m + (local % band) % band_m;
+        const uint32_t nt = (local % band) / band_m;
+        t.pf_r = (local % band) % band_m;
+        t.pf_c = nt & 3u;
+        t.m0 = mt * BM;
+        t.n0 = nt * tile_n;
+        t.n_lim = n_span - t.n0 < tile_n ? n_span : t.n0 + tile_n;
+        // packed element offsets of the group: the varying dimension's prefix times the other dimension of the operand
+        const uint64_t before = uniform(s_prefix[e]);
+        if constexpr (VARY_K) {
+            t.off_a = before * args.m;
+            t.off_b = before * Ne;
+            t.off_d = (uint64_t)e * args.m * Ne;
+        } else {
+            t.off_a = before * args.k;
+            t.off_b = (uint64_t)e * Ne * args.k;
+            t.off_d = before * Ne;
+        }
+        // 16-byte accesses need every contiguous dimension a multiple of 8 elements and packed group bases that stayed
+        // multiples of 8; loads and stores address a tile with 32-bit byte offsets below 2^31 (grouped_gemm.hip)
+        bool fast = (Ne % 8u == 0) && (Ne < (1u << 23)) && (t.off_a % 8u == 0) && (t.off_b % 8u == 0) && (t.off_d % 8u == 0);
+        if (A_KC || B_KC) fast = fast && (t.Ke % 8u == 0) && (t.Ke < (1u << 21));
+        if (!A_KC) fast = fast && (t.Me % 8u == 0) && (t.Me < (1u << 23));
+        if (EPI != EPI_PLAIN) fast = fast && (n_span % 8u == 0);
+        t.fast = fast;
+        return t;
+    };
+    auto k_steps = [&](const Tile& t) { return (t.Ke + BK - 1) / BK; };
+    // groups of at most 64 rows run a K loop of their own with a third LDS stage (grouped_gemm.hip); they start cold
+    auto is_thin = [&](const Tile& t) { return A_KC && t.Me <= 64u && k_steps(t) >= 3u; };
+    // a tile whose first two K steps can be fetched by the tile before it, and which can fetch the next tile's
+    auto streams = [&](const Tile& t) { return t.valid && t.fast && t.Ke > 0 && !is_thin(t); };
+
+    // ---- loaders: `cur` feeds the tile being computed, `nxt` the tile after it ----
+    LoaderK<NW, false> lk_a;
+    LoaderK<NW, EPI != EPI_PLAIN> lk_b;
+    LoaderT<NW> lt_a, lt_b;
+    Feed<A_KC> fa_cur{}, fa_nxt{};
+    Feed<B_KC> fb_cur{}, fb_nxt{};
+    uint32_t va_cur = 0, va_nxt = 0, vb_cur = 0, vb_nxt = 0;  // the loaders' per-lane offsets (they depend on the pitch)
+    // sets a loader object up for tile t and keeps what is specific to the tile
+    auto setup_a = [&](const Tile& t, Feed<A_KC>& f, uint32_t& v) {
+        const uint16_t* Ae = args.A + t.off_a;
+        if constexpr (A_KC) {
+            lk_a.setup(Ae + (uint64_t)t.m0 * t.Ke, nullptr, t.Me - t.m0 < (uint32_t)BM ? t.Me - t.m0 : (uint32_t)BM, t.Ke, wave, lane);
+            f = Feed<A_KC>{lk_a.base0, nullptr, lk_a.bytes, lk_a.ldb, 0u};
+            v = lk_a.voff;
+        } else {
+            lt_a.setup(Ae, t.Me, t.Ke, t.m0, wave, lane);
+            f = Feed<A_KC>{lt_a.base, nullptr, t.Ke, lt_a.ldb, lt_a.col_bytes};
+            v = lt_a.voff;
+        }
+    };
+    auto setup_b = [&](const Tile& t, Feed<B_KC>& f, uint32_t& v) {
+        const uint16_t* Be = args.B + t.off_b;
+        if constexpr (B_KC) {
+            if constexpr (EPI != EPI_PLAIN) {
+                // tile rows 0..127: "up" rows n0.. of the weight; rows 128..255: "gate" rows I + n0..
+                lk_b.setup(Be + (uint64_t)t.n0 * t.Ke, Be + (uint64_t)(n_span + t.n0) * t.Ke, t.n_lim - t.n0, t.Ke, wave, lane);
+            } else {
+                lk_b.setup(Be + (uint64_t)t.n0 * t.Ke, nullptr, t.n_lim - t.n0, t.Ke, wave, lane);
+            }
+            f = Feed<B_KC>{lk_b.base0, lk_b.base1, lk_b.bytes, lk_b.ldb, 0u};
+            v = lk_b.voff;
+        } else {
+            lt_b.setup(Be, Ne, t.Ke, t.n0, wave, lane);
+            f = Feed<B_KC>{lt_b.base, nullptr, t.Ke, lt_b.ldb, lt_b.col_bytes};
+            v = lt_b.voff;
+        }
+    };
+    // points a loader object at a feed (what depends on lane and wavefront only stays as the last setup left it)
+    auto aim_a = [&](const Feed<A_KC>& f, uint32_t v) {
+        if constexpr (A_KC) { lk_a.base0 = f.base0; lk_a.bytes = f.extent; lk_a.ldb = f.ldb; lk_a.kdim = f.ldb / 2u; lk_a.voff = v; }
+        else { lt_a.base = f.base0; lt_a.kdim = f.extent; lt_a.ldb = f.ldb; lt_a.col_bytes = f.col_bytes; lt_a.voff = v; }
+    };
+    auto aim_b = [&](const Feed<B_KC>& f, uint32_t v) {
+        if constexpr (B_KC) { lk_b.base0 = f.base0; lk_b.base1 = f.base1; lk_b.bytes = f.extent; lk_b.ldb = f.ldb; lk_b.kdim = f.ldb / 2u; lk_b.voff = v; }
+        else { lt_b.base = f.base0; lt_b.kdim = f.extent; lt_b.ldb = f.ldb; lt_b.col_bytes = f.col_bytes; lt_b.voff = v; }
+    };
+
+    // ---- L2 prefetch by designated workgroups (grouped_gemm.hip): one 4-byte load per shared line, kPfDist steps ahead ----
+    constexpr bool kPrefetch = A_KC == B_KC;
+    uint32_t pf_voff = kOutOfRange;
+    const uint16_t* pf_base = nullptr;
+    uint32_t pf_bytes = 0, pf_ldb = 0, pf_col_bytes = 0, pf_kdim = 0, pf_steps = 0;
+    const bool pf_is_b = (wave & 1u) != 0;
+    const bool pf_t = pf_is_b ? !B_KC : !A_KC;
+    auto setup_prefetch = [&](const Tile& t) {
+        if constexpr (!kPrefetch) return;
+        const uint32_t p = wave >> 1;
+        pf_steps = k_steps(t);
+        if (!pf_is_b) {
+            const uint32_t i = p * 16u + lane;
+            if constexpr (A_KC) {
+                pf_base = fa_cur.base0; pf_bytes = fa_cur.extent;
+                pf_voff = lane < 16u ? (4u * i + t.pf_c) * (t.Ke * 2u) : kOutOfRange;
+            } else {
+                pf_base = fa_cur.base0; pf_ldb = fa_cur.ldb; pf_col_bytes = fa_cur.col_bytes; pf_kdim = t.Ke;
+                pf_voff = lane < 16u ? i * fa_cur.ldb + t.pf_c * 128u : kOutOfRange;
+            }
+        } else {
+            if constexpr (B_KC) {
+                pf_bytes = fb_cur.extent;
+                if constexpr (EPI != EPI_PLAIN) {
+                    pf_base = (p >> 1) ? fb_cur.base1 : fb_cur.base0;
+                    pf_voff = lane < 8u ? (8u * ((p & 1u) * 8u + lane) + t.pf_r) * (t.Ke * 2u) : kOutOfRange;
+                } else {
+                    pf_base = fb_cur.base0;
+                    pf_voff = lane < 8u ? (8u * (p * 8u + lane) + t.pf_r) * (t.Ke * 2u) : kOutOfRange;
+                }
+            } else {
+                pf_base = fb_cur.base0; pf_ldb = fb_cur.ldb; pf_col_bytes = fb_cur.col_bytes; pf_kdim = t.Ke;
+                pf_voff = lane < 8u ? (2u * (p * 8u + lane) + (t.pf_r >> 2)) * fb_cur.ldb + (t.pf_r & 3u) * 128u : kOutOfRange;
+            }
+        }
+    };
+    // requests this wavefront's lines of K step `kstep` of the current tile (nothing past its last step)
+    auto issue_prefetch = [&](uint32_t kstep) {
+        if constexpr (!kPrefetch) return;
+        const uint32_t k0 = kstep * (uint32_t)BK;
+        const bool inside = kstep < pf_steps;
+        const uint32_t rows = k0 >= pf_kdim ? 0u : (pf_kdim - k0 < (uint32_t)BK ? pf_kdim - k0 : (uint32_t)BK);
+        const uint16_t* base = pf_t ? pf_base + (uint64_t)k0 * (pf_ldb / 2u) : pf_base;
+        const uint32_t bytes = !inside ? 0u : (pf_t ? (rows ? rows * pf_ldb - pf_col_bytes : 0u) : pf_bytes);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(make_rsrc(base, bytes), (lds_void*)s_pf, 4, pf_voff, pf_t ? 0u : k0 * 2u, 0, 0);
+    };
+
+    constexpr int kLoads = 32 / NW;                // load instructions per wavefront, operand and K step
+    constexpr uint32_t kStepLoads = 2 * kLoads;    // per wavefront and K step
+    // store instructions per wavefront and tile (the epilogue issues a fixed number)
+    constexpr uint32_t kTileStores = EPI == EPI_PLAIN ? WM * WN * 2 / 1024 : (EPI == EPI_SWIGLU ? WM * WN * 2 / 1024 : 0) + WM * WN / 1024;
+
+    // loads of one K step of the CURRENT loaders' aim into `stage` (compiler-visible: placed by the scheduling hints)
+    auto issue_a = [&](int stage, uint32_t k0) {
+        if constexpr (A_KC) lk_a.template issue_range<0, kLoads>(stage ? s_a1 : s_a0, k0);
+        else lt_a.template issue_range<0, kLoads>(stage ? s_a1 : s_a0, k0);
+    };
+    auto issue_b = [&](int stage, uint32_t k0) {
+        if constexpr (B_KC) lk_b.template issue_range<0, kLoads>(stage ? s_b1 : s_b0, k0);
+        else lt_b.template issue_range<0, kLoads>(stage ? s_b1 : s_b0, k0);
+    };
+    // ... and written in assembly, for a cold start
+    auto issue_quiet = [&](int stage, uint32_t k0) {
+        if constexpr (A_KC) lk_a.issue_quiet(stage ? s_a1 : s_a0, k0);
+        else lt_a.issue_quiet(stage ? s_a1 : s_a0, k0);
+        if constexpr (B_KC) lk_b.issue_quiet(stage ? s_b1 : s_b0, k0);
+        else lt_b.issue_quiet(stage ? s_b1 : s_b0, k0);
+    };
+
+#ifdef FMA_PROF
+    uint64_t p_start, p_t0 = 0, p_t1 = 0, p_seg[6] = {0, 0, 0, 0, 0, 0}, p_tiles = 0;
+    PROF_STAMP(p_start);
+#endif
+    uint32_t round = 0;
+    Tile cur = lookup(0), nxt = lookup(1);
+    bool streamed = false;  // the first two K steps of `cur` were fetched by the tile before it
+    while (cur.valid) {
+        const uint32_t Me = cur.Me, Ke = cur.Ke, m0 = cur.m0, n0 = cur.n0, n_lim = cur.n_lim;
+        const uint64_t off_d = cur.off_d;
+
+        if (!streamed) {
+            if (!cur.fast) {
+                if constexpr (EPI == EPI_PLAIN) {
+                    scalar_tile<EL, A_KC, B_KC, BM, BN>(args.A + cur.off_a, args.B + cur.off_b, args.D + off_d, Me, Ne, Ke, m0, n0,
+                                                        args.alpha, NT);
+                }
+                cur = nxt;
+                nxt = lookup(round + 2);
+                ++round;
+                continue;
+            }
+            setup_a(cur, fa_cur, va_cur);
+            setup_b(cur, fb_cur, vb_cur);
+        }
+        setup_prefetch(cur);
+        const uint32_t KT = (Ke + BK - 1) / BK;
+        const uint32_t KT2 = (KT + 1u) & ~1u;  // steps of the K loop: an odd count gets a step of zeros
+        const bool thin = is_thin(cur);
+        // the next tile's first two K steps ride on this tile's last two load slots
+        const bool stream_next = streams(cur) && streams(nxt);
+        if (stream_next) {
+            setup_a(nxt, fa_nxt, va_nxt);
+            setup_b(nxt, fb_nxt, vb_nxt);
+        } else {
+            // a feed that fetches nothing: every load of it zero-fills
+            fa_nxt = fa_cur;
+            fb_nxt = fb_cur;
+            fa_nxt.extent = 0u;
+            fb_nxt.extent = 0u;
+            va_nxt = va_cur;
+            vb_nxt = vb_cur;
+        }
+        // (the set-ups above left the loader objects aimed at the last tile set up)
+        aim_a(fa_cur, va_cur);
+        aim_b(fb_cur, vb_cur);
+
+        f32x16 acc[FM][FN];
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.0f;
+
+        // MFMA operand fragments of one 16-wide k slice, double buffered in registers. The K loop exists in four
+        // versions, for wavefronts whose first FA = 4, 2, 1 or 0 row blocks (of 32 rows) hold rows of the group.
+        typename EL::frag fa[2][FM], fb[2][FN];
+        auto load_frags = [&](auto fa_c, int stage, int ks, int buf) {
+            constexpr int FA = decltype(fa_c)::value;
+            if constexpr (FA > 0) {
+                const uint8_t* ta = stage ? s_a1 : s_a0;
+                const uint8_t* tb = stage ? s_b1 : s_b0;
+#pragma unroll
+                for (int i = 0; i < FA; ++i) {
+                    if constexpr (A_KC) fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_kc_frag(ta + a_off[i] + kc_slice[ks]));
+                    else fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_tr_frag(ta + a_off[i] + ks * 16 * kTRowBytes));
+                }
+#pragma unroll
+                for (int j = 0; j < FN; ++j) {
+                    if constexpr (B_KC) fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_kc_frag(tb + b_off[j] + kc_slice[ks]));
+                    else fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_tr_frag(tb + b_off[j] + ks * 16 * kTRowBytes));
+                }
+            }
+        };
+        auto mma = [&](auto fa_c, int buf) {
+            constexpr int FA = decltype(fa_c)::value;
+#pragma unroll
+            for (int i = 0; i < FA; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = EL::mfma(fb[buf][j], fa[buf][i], acc[i][j]);
+        };
+
+        // ---- one K step (see grouped_gemm.hip for the placement of barrier, waits and loads) ----
+        // WAIT: the s_waitcnt immediate in front of the barrier. The loads issued after the barrier are those of step
+        // kt + 2: of this tile, or, in the last two steps, steps 0 and 1 of the next tile (or nothing).
+        // SRC: which tile the loads issued in the step belong to: 0 the current one, 1 the next one (the loaders are aimed
+        // by the caller in both cases), 2 decided here (first steps of a tile, and the versions for tiles with few rows).
+        auto step = [&](auto fa_c, auto wait_c, auto src_c, int stage, uint32_t kt) {
+            constexpr int FA = decltype(fa_c)::value;
+            constexpr int SRC = decltype(src_c)::value;
+            constexpr int kReads = (A_KC ? FA : 2 * FA) + (B_KC ? FN : 2 * FN);
+            load_frags(fa_c, stage, 1, 1);
+            mma(fa_c, 0);
+            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, 0>();
+            load_frags(fa_c, stage, 2, 0);
+            mma(fa_c, 1);
+            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, 0>();
+            load_frags(fa_c, stage, 3, 1);
+            mma(fa_c, 0);
+            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, 0>();
+            // every load of step kt+1 has landed and every LDS read of this stage has returned
+            __builtin_amdgcn_s_waitcnt(decltype(wait_c)::value);
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            load_frags(fa_c, stage ^ 1, 0, 0);
+            uint32_t k0;
+            if constexpr (SRC == 0) {
+                k0 = (kt + 2u) * (uint32_t)BK;
+            } else if constexpr (SRC == 1) {
+                k0 = (kt + 2u - KT2) * (uint32_t)BK;
+            } else {
+                const bool of_next = kt + 2u >= KT2;
+                k0 = (of_next ? kt + 2u - KT2 : kt + 2u) * (uint32_t)BK;
+                aim_a(Feed<A_KC>{of_next ? fa_nxt.base0 : fa_cur.base0, nullptr, of_next ? fa_nxt.extent : fa_cur.extent,
+                                 of_next ? fa_nxt.ldb : fa_cur.ldb, of_next ? fa_nxt.col_bytes : fa_cur.col_bytes},
+                      of_next ? va_nxt : va_cur);
+                aim_b(Feed<B_KC>{of_next ? fb_nxt.base0 : fb_cur.base0, of_next ? fb_nxt.base1 : fb_cur.base1,
+                                 of_next ? fb_nxt.extent : fb_cur.extent, of_next ? fb_nxt.ldb : fb_cur.ldb,
+                                 of_next ? fb_nxt.col_bytes : fb_cur.col_bytes},
+                      of_next ? vb_nxt : vb_cur);
+            }
+            issue_a(stage, k0);
+            issue_b(stage, k0);
+            // the prefetch goes out behind this step's loads (the empty statement orders it: the wait of the next step
+            // counts on it being the newest load)
+            if constexpr (kPrefetch) asm volatile("" : "+v"(pf_voff));
+            issue_prefetch(kt + kPfDist);
+            mma(fa_c, 1);
+            if constexpr (FA > 0) {
+                __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
+                spread_mfma_vmem<0, FA * FN, (int)kStepLoads>();
+                if constexpr (kPrefetch) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            }
+        };
+        // waits of a step: all but the newest load when that is the previous step's prefetch; in a tile's first step the
+        // stores of the previous epilogue (or the cold start's stand-ins) are newer than the loads waited for as well
+        using WaitStep = std::integral_constant<int, waitcnt_imm(kPrefetch ? 1 : 0, true)>;
+        using WaitFirst = std::integral_constant<int, waitcnt_imm((int)kTileStores + (kPrefetch ? 1 : 0), true)>;
+
+        Tile nn{};  // the tile after next
+        const uint32_t tile_rows = Me - m0 < (uint32_t)BM ? Me - m0 : (uint32_t)BM;
+        const uint32_t wave_rows = tile_rows > wm * WM ? tile_rows - wm * WM : 0u;
+        const bool has_columns = n0 + wn * (EPI != EPI_PLAIN ? WN / 2 : WN) < n_lim;
+        const uint32_t row_blocks = has_columns ? uniform((wave_rows + 31u) / 32u) : 0u;
+        if (thin) {
+            // three LDS stages in the space a tile of at most 64 rows leaves unused (grouped_gemm.hip); cold start
+            constexpr uint32_t kThinLoads = 1 + kLoads;
+            static_assert(kThinLoads == 5, "the waits below are written for five loads per step");
+            const uint8_t* const a_at[3] = {s_a0, s_a1, s_a0 + 8192};
+            const uint8_t* const b_lo[3] = {s_b0, s_b1, s_a0 + 16384};
+            const uint8_t* const b_hi[3] = {s_b0 + 16384, s_b1 + 16384, s_a1 + 16384};
+            auto issue_thin = [&](int st, uint32_t k0) {
+                if constexpr (A_KC) lk_a.issue_quiet_first_rows(lds_address(a_at[st]), k0);
+                if constexpr (B_KC) lk_b.issue_quiet_halves(lds_address(b_lo[st]), lds_address(b_hi[st]), k0);
+                else lt_b.issue_quiet_halves(lds_address(b_lo[st]), lds_address(b_hi[st]), k0);
+            };
+            issue_thin(0, 0);
+            issue_thin(1, BK);
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm((int)kThinLoads, false));
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            issue_thin(2, 2 * BK);
+            auto thin_loop = [&](auto fa_c) {
+                constexpr int FA = decltype(fa_c)::value;
+                auto thin_step = [&](int st, uint32_t kt) {
+                    if constexpr (FA > 0) {
+#pragma unroll
+                        for (int ks = 0; ks < 4; ++ks) {
+                            typename EL::frag ta[FA], tb[FN];
+#pragma unroll
+                            for (int i = 0; i < FA; ++i)
+                                ta[i] = __builtin_bit_cast(typename EL::frag, read_kc_frag(a_at[st] + a_off[i] + kc_slice[ks]));
+#pragma unroll
+                            for (int j = 0; j < FN; ++j) {
+                                if constexpr (B_KC) {
+                                    const uint8_t* half = b_frag_row(j) < 128u ? b_lo[st] + b_off[j] : b_hi[st] + (b_off[j] - 128u * kRowBytes);
+                                    tb[j] = __builtin_bit_cast(typename EL::frag, read_kc_frag(half + kc_slice[ks]));
+                                } else {
+                                    const uint8_t* half = ks < 2 ? b_lo[st] + ks * 16 * kTRowBytes : b_hi[st] + (ks - 2) * 16 * kTRowBytes;
+                                    tb[j] = __builtin_bit_cast(typename EL::frag, read_tr_frag(half + b_off[j]));
+                                }
+                            }
+#pragma unroll
+                            for (int i = 0; i < FA; ++i)
+#pragma unroll
+                                for (int j = 0; j < FN; ++j) acc[i][j] = EL::mfma(tb[j], ta[i], acc[i][j]);
+                        }
+                    }
+                    __builtin_amdgcn_s_waitcnt(waitcnt_imm((int)kThinLoads, false));
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    issue_thin(st, (kt + 3) * BK);
+                };
+                uint32_t kt = 0;
+                for (; kt + 2 < KT; kt += 3) {
+                    thin_step(0, kt);
+                    thin_step(1, kt + 1);
+                    thin_step(2, kt + 2);
+                }
+                if (kt < KT) thin_step(0, kt);
+                if (kt + 1 < KT) thin_step(1, kt + 1);
+            };
+            if (row_blocks == 2) thin_loop(std::integral_constant<int, 2>{});
+            else if (row_blocks == 1) thin_loop(std::integral_constant<int, 1>{});
+            else thin_loop(std::integral_constant<int, 0>{});
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, false));
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        } else if (KT > 0) {
+            if (!streamed) {
+                // cold start: the first two K steps, then as many stores outside every buffer as an epilogue issues
+                issue_quiet(0, 0);
+                issue_quiet(1, BK);
+                const __amdgpu_buffer_rsrc_t nowhere = make_rsrc(args.D, 0u);
+#pragma unroll
+                for (uint32_t i = 0; i < kTileStores; ++i)  // (distinct offsets: identical stores would be merged into one)
+                    store_tile16<false>(nowhere, kOutOfRange + i * 16u, uint4{0u, 0u, 0u, 0u});
+                // the first step's loads have landed; the second step's, and the stand-in stores, may be out
+                __builtin_amdgcn_s_waitcnt(waitcnt_imm((int)(kStepLoads + kTileStores), false));
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            }
+            issue_prefetch(kPfDist - 1);
+#ifdef FMA_PROF
+            PROF_STAMP(p_t1);
+            if (p_t0) p_seg[3] += p_t1 - p_t0;  // tile top: set-ups, accumulators cleared
+            p_t0 = p_t1;
+#endif
+            using SrcCur = std::integral_constant<int, 0>;
+            using SrcNext = std::integral_constant<int, 1>;
+            using SrcEither = std::integral_constant<int, 2>;
+            auto k_loop = [&](auto fa_c) {
+                constexpr int FA = decltype(fa_c)::value;
+                load_frags(fa_c, 0, 0, 0);
+                step(fa_c, WaitFirst{}, SrcEither{}, 0, 0);
+                step(fa_c, WaitStep{}, SrcEither{}, 1, 1);
+#ifdef FMA_PROF
+                PROF_STAMP(p_t1);
+                p_seg[4] += p_t1 - p_t0;  // the first two K steps
+                p_t0 = p_t1;
+#endif
+                if constexpr (FA == FM) {
+                    // full tiles: the steps in the middle load from the current tile and the last two from the next, each
+                    // with the loaders aimed once, so that the loop body carries no selects
+                    if (KT2 > 2u) {
+                        aim_a(fa_cur, va_cur);
+                        aim_b(fb_cur, vb_cur);
+                        uint32_t kt = 2;
+                        for (; kt + 2u < KT2; kt += 2) {  // two steps per iteration without a branch between them
+                            step(fa_c, WaitStep{}, SrcCur{}, 0, kt);
+                            step(fa_c, WaitStep{}, SrcCur{}, 1, kt + 1);
+                        }
+                        aim_a(fa_nxt, va_nxt);
+                        aim_b(fb_nxt, vb_nxt);
+                        step(fa_c, WaitStep{}, SrcNext{}, 0, kt);
+                        step(fa_c, WaitStep{}, SrcNext{}, 1, kt + 1);
+                    }
+                } else {
+                    for (uint32_t kt = 2; kt < KT2; kt += 2) {
+                        step(fa_c, WaitStep{}, SrcEither{}, 0, kt);
+                        step(fa_c, WaitStep{}, SrcEither{}, 1, kt + 1);
+                    }
+                }
+            };
+            static_assert(FM == 4, "the versions below are for four row blocks per wavefront");
+            if (row_blocks > 2) k_loop(std::integral_constant<int, 4>{});
+            else if (row_blocks == 2) k_loop(std::integral_constant<int, 2>{});
+            else if (row_blocks == 1) k_loop(std::integral_constant<int, 1>{});
+            else k_loop(std::integral_constant<int, 0>{});
+            if (!stream_next) {
+                // nothing rides behind this tile: its last two load slots zero-filled the stages; they must have landed,
+                // and every wavefront must be past its last read, before anyone starts cold
+                __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, false));
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            }
+        }
+
+#ifdef FMA_PROF
+        PROF_STAMP(p_t1);
+        p_seg[0] += p_t1 - p_t0;  // rest of the K loop
+        p_t0 = p_t1;
+        p_seg[5] += KT2 > 2 ? KT2 - 2 : 0;
+        ++p_tiles;
+#endif
+        // the tile after next is looked up here: scalar work beside an epilogue that is bound by the store path
+        nn = lookup(round + 2);
+#ifdef FMA_PROF
+        PROF_STAMP(p_t1);
+        p_seg[1] += p_t1 - p_t0;  // look-up
+        p_t0 = p_t1;
+#endif
+
+        // ---- epilogue: through this wavefront's 2 KB of the staging buffer, 16 rows of 128 bytes at a time ----
+        // A lane holds row (lane & 31), columns q*8 + (lane >> 5)*4 + 0..3 of each 32x32 accumulator block.
+        // (the lane id is made opaque so that the per-lane address arithmetic is redone per tile, not hoisted out of the
+        // tile loop where it would occupy registers throughout the K loop)
+        uint32_t el = lane;
+        asm volatile("" : "+v"(el));
+        const uint32_t img = lds_address(s_stage) + wave * (uint32_t)kStageBytes;
+        if (EPI == EPI_PLAIN && args.alpha != 1.0f) {
+            const float alpha = args.alpha;
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j) acc[i][j] *= alpha;
+        }
+        const bool upper = ((el >> 4) & 1u) != 0;  // this lane's row lies in the second 16 rows of its 32-row block
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            const uint32_t row0 = m0 + wm * WM + i * 32;  // first output row of this block
+            if constexpr (EPI == EPI_PLAIN) {
+                const uint32_t col0 = n0 + wn * WN;
+                const uint32_t cols_valid = col0 < n_lim ? n_lim - col0 : 0u;
+                uint2 w[FN][4];
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const f32x16& c = acc[i][j];
+                        w[j][q].x = EL::pack2(c[q * 4 + 0], c[q * 4 + 1]);
+                        w[j][q].y = EL::pack2(c[q * 4 + 2], c[q * 4 + 3]);
+                    }
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    if (upper == (half == 1)) {
+#pragma unroll
+                        for (int j = 0; j < FN; ++j)
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) stage_put_quiet<WN * 2>(img, el & 15u, j * 32 + q * 8 + (el >> 5) * 4, w[j][q]);
+                    }
+                    const uint32_t r0 = row0 + half * 16;
+                    const uint32_t rows_valid = r0 < Me ? (Me - r0 < 16u ? Me - r0 : 16u) : 0u;
+                    stage_flush_quiet<WN * 2, 16>(img, args.D + off_d + (uint64_t)r0 * Ne + col0, Ne, rows_valid, cols_valid, el);
+                }
+            } else {
+                // first the rounded pre-activation (32 "up" columns | 32 "gate" columns per row), then the activation
+                constexpr int HB = WN * 2;
+                constexpr int YB = WN;
+                static_assert(FN == 2, "one up block and one gate block per wavefront and row block");
+                const uint32_t col0 = n0 + wn * (WN / 2);
+                const uint32_t cols_valid = col0 < n_lim ? n_lim - col0 : 0u;
+                uint32_t ypack[4][2];
+                uint2 wu[4], wg[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float u[4], g[4], y[4];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        u[x] = EL::round(acc[i][0][q * 4 + x]);
+                        g[x] = EL::round(acc[i][1][q * 4 + x]);
+                        y[x] = u[x] * g[x] * sigmoid_for<typename EL::act_t>(g[x]);
+                    }
+                    ypack[q][0] = EL::pack2(y[0], y[1]);
+                    ypack[q][1] = EL::pack2(y[2], y[3]);
+                    if constexpr (EPI == EPI_SWIGLU) {
+                        wu[q].x = EL::pack2(u[0], u[1]);
+                        wu[q].y = EL::pack2(u[2], u[3]);
+                        wg[q].x = EL::pack2(g[0], g[1]);
+                        wg[q].y = EL::pack2(g[2], g[3]);
+                    }
+                }
+                if constexpr (EPI == EPI_SWIGLU) {
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        if (upper == (half == 1)) {
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) {
+                                const uint32_t c = q * 8 + (el >> 5) * 4;
+                                stage_put_quiet<HB>(img, el & 15u, c, wu[q]);
+                                stage_put_quiet<HB>(img, el & 15u, WN / 2 + c, wg[q]);
+                            }
+                        }
+                        const uint32_t r0 = row0 + half * 16;
+                        const uint32_t rows_valid = r0 < Me ? (Me - r0 < 16u ? Me - r0 : 16u) : 0u;
+                        stage_flush_split_quiet<HB, 16, WN / 2>(img, args.D + off_d + (uint64_t)r0 * Ne + col0, Ne, rows_valid, cols_valid,
+                                                          n_span, el);
+                    }
+                }
+                const uint32_t rows_valid = row0 < Me ? (Me - row0 < 32u ? Me - row0 : 32u) : 0u;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    uint2 wy;
+                    wy.x = ypack[q][0];
+                    wy.y = ypack[q][1];
+                    stage_put_quiet<YB>(img, el & 31u, q * 8 + (el >> 5) * 4, wy);
+                }
+                stage_flush_quiet<YB, 32>(img, args.ACT + off_d / 2 + (uint64_t)row0 * n_span + col0, n_span, rows_valid, cols_valid, el);
+            }
+        }
+
+#ifdef FMA_PROF
+        PROF_STAMP(p_t1);
+        p_seg[2] += p_t1 - p_t0;  // epilogue
+        p_t0 = p_t1;
+#endif
+        // ---- on to the next tile ----
+        streamed = stream_next;
+        if (stream_next) {
+            fa_cur = fa_nxt;
+            fb_cur = fb_nxt;
+            va_cur = va_nxt;
+            vb_cur = vb_nxt;
+        }
+        cur = nxt;
+        nxt = nn;
+        ++round;
+    }
+#ifdef FMA_PROF
+    {
+        uint64_t t;
+        PROF_STAMP(t);
+        if (lane == 0) {
+            unsigned long long* o = fma_prof + ((size_t)blockIdx.x * 8 + wave) * 8;
+            for (int i = 0; i < 6; ++i) o[i] = p_seg[i];
+            o[6] = p_tiles;
+            o[7] = t - p_start;
+        }
+    }
+#endif
+}
+
+// every instantiation the entry points launch (explicit, so that host stub and device code are both emitted)
+#define FMA_RAGGED_INSTANTIATE(EL)                                                                          \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, false>(const Args);                  \
+    template __global__ void ragged_gemm_kernel<EL, true, false, EPI_PLAIN, false>(const Args);                 \
+    template __global__ void ragged_gemm_kernel<EL, false, true, EPI_PLAIN, false>(const Args);                 \
+    template __global__ void ragged_gemm_kernel<EL, false, false, EPI_PLAIN, false>(const Args);                \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, true>(const Args);                   \
+    template __global__ void ragged_gemm_kernel<EL, true, false, EPI_PLAIN, true>(const Args);                  \
+    template __global__ void ragged_gemm_kernel<EL, false, true, EPI_PLAIN, true>(const Args);                  \
+    template __global__ void ragged_gemm_kernel<EL, false, false, EPI_PLAIN, true>(const Args);                 \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU, false>(const Args);                 \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false>(const Args);
+FMA_RAGGED_INSTANTIATE(ElemBf16)
+FMA_RAGGED_INSTANTIATE(ElemF16)
+#undef FMA_RAGGED_INSTANTIATE
+
+template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K>
+int launch(const Args& args, hipStream_t st) {
+    int cus = num_compute_units();
+    if (cus <= 0) cus = 256;
+    hipLaunchKernelGGL((ragged_gemm_kernel<EL, A_KC, B_KC, EPI, VARY_K>), dim3((uint32_t)cus), dim3(NT), 0, st, args);
+    return launch_status("grouped_gemm_ragged");
+}
+
+template <typename EL, bool VARY_K>
+int launch_plain(const Args& args, bool a_kc, bool b_kc, hipStream_t st) {
+    if (a_kc && b_kc) return launch<EL, true, true, EPI_PLAIN, VARY_K>(args, st);
+    if (a_kc && !b_kc) return launch<EL, true, false, EPI_PLAIN, VARY_K>(args, st);
+    if (!a_kc && b_kc) return launch<EL, false, true, EPI_PLAIN, VARY_K>(args, st);
+    return launch<EL, false, false, EPI_PLAIN, VARY_K>(args, st);
+}
+
+}  // namespace ragged
+}  // namespace gemm
+}  // namespace fmahip
+
+extern "C" {
+
+#ifdef FMA_PROF
+int fma_debug_prof(void* host, int64_t bytes) {
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(fmahip::gemm::ragged::fma_prof), (size_t)bytes, 0, hipMemcpyDeviceToHost);
+}
+#endif
+
+int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_t* sizes, int64_t E, int vary,
+                            int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, float alpha, int dtype,
+                            void* stream) {
+    using namespace fmahip;
+    using namespace fmahip::gemm;
+    FMA_REQUIRE(dtype == FMA_BF16 || dtype == FMA_F16, dtype_bytes(dtype) ? FMA_ERR_UNSUPPORTED : FMA_ERR_BAD_DTYPE,
+                "grouped_gemm_ragged: bf16 and fp16 operands are implemented (dtype code %d)", dtype);
+    FMA_REQUIRE(vary == FMA_VARY_M || vary == FMA_VARY_K, FMA_ERR_BAD_SIZE,
+                "grouped_gemm_ragged: vary must be FMA_VARY_M or FMA_VARY_K (got %d)", vary);
+    FMA_REQUIRE(E >= 0, FMA_ERR_BAD_SIZE, "grouped_gemm_ragged: negative group count %lld", (long long)E);
+    FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "grouped_gemm_ragged: E=%lld exceeds the limit %d",
+                (long long)E, FMA_MAX_GROUPS);
+    if (vary == FMA_VARY_M) M = 0;
+    else K = 0;
+    FMA_REQUIRE(M >= 0 && N >= 0 && K >= 0 && M <= 0xffffffffll && N <= 0xffffffffll && K <= 0xffffffffll, FMA_ERR_BAD_SIZE,
+                "grouped_gemm_ragged: dimensions must lie in [0, 2^32) (M=%lld N=%lld K=%lld)", (long long)M, (long long)N,
+                (long long)K);
+    if (E == 0) return FMA_OK;
+    FMA_REQUIRE(A && B && D && sizes, FMA_ERR_NULL_POINTER, "grouped_gemm_ragged: NULL pointer");
+    FMA_REQUIRE(aligned16(A) && aligned16(B) && aligned16(D), FMA_ERR_MISALIGNED,
+                "grouped_gemm_ragged: A, B and D must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const bool a_kc = trans_a == 0;  // A stored [M, K]: reduction dim contiguous
+    const bool b_kc = trans_b != 0;  // B stored [N, K]: reduction dim contiguous
+    ragged::Args args{};
+    args.A = (const uint16_t*)A;
+    args.B = (const uint16_t*)B;
+    args.D = (uint16_t*)D;
+    args.ACT = nullptr;
+    args.sizes = sizes;
+    args.E = (uint32_t)E;
+    args.m = (uint32_t)M;
+    args.n = (uint32_t)N;
+    args.k = (uint32_t)K;
+    args.alpha = alpha;
+    if (vary == FMA_VARY_K)
+        return dtype == FMA_BF16 ? ragged::launch_plain<ElemBf16, true>(args, a_kc, b_kc, st)
+                                 : ragged::launch_plain<ElemF16, true>(args, a_kc, b_kc, st);
+    return dtype == FMA_BF16 ? ragged::launch_plain<ElemBf16, false>(args, a_kc, b_kc, st)
+                             : ragged::launch_plain<ElemF16, false>(args, a_kc, b_kc, st);
+}
+
+int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, const uint32_t* M_arr, int64_t E,
+                            int64_t I, int64_t K, int dtype, void* stream) {
+    using namespace fmahip;
+    using namespace fmahip::gemm;
+    FMA_REQUIRE(dtype == FMA_BF16 || dtype == FMA_F16, dtype_bytes(dtype) ? FMA_ERR_UNSUPPORTED : FMA_ERR_BAD_DTYPE,
+                "grouped_gemm_swiglu: bf16 and fp16 operands are implemented (dtype code %d)", dtype);
+    FMA_REQUIRE(E >= 0, FMA_ERR_BAD_SIZE, "grouped_gemm_swiglu: negative group count %lld", (long long)E);
+    FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "grouped_gemm_swiglu: E=%lld exceeds the limit %d",
+                (long long)E, FMA_MAX_GROUPS);
+    // the upper bounds are those of the kernel's 32-bit tile offsets; this entry point has no scalar path beyond them
+    FMA_REQUIRE(I >= 8 && I % 8 == 0 && 2 * I < (1ll << 23), FMA_ERR_BAD_SIZE,
+                "grouped_gemm_swiglu: intermediate size %lld must be a positive multiple of 8 below 2^22", (long long)I);
+    FMA_REQUIRE(K >= 8 && K % 8 == 0 && K < (1ll << 21), FMA_ERR_BAD_SIZE,
+                "grouped_gemm_swiglu: K=%lld must be a positive multiple of 8 below 2^21", (long long)K);
+    if (E == 0) return FMA_OK;
+    FMA_REQUIRE(x && W && act && M_arr, FMA_ERR_NULL_POINTER, "grouped_gemm_swiglu: NULL pointer");
+    FMA_REQUIRE(aligned16(x) && aligned16(W) && aligned16(act) && aligned16(h), FMA_ERR_MISALIGNED,
+                "grouped_gemm_swiglu: x, W, h and act must be 16-byte aligned");
+    ragged::Args args{};
+    args.A = (const uint16_t*)x;
+    args.B = (const uint16_t*)W;
+    args.D = (uint16_t*)h;
+    args.ACT = (uint16_t*)act;
+    args.sizes = M_arr;
+    args.E = (uint32_t)E;
+    args.m = 0;
+    args.n = (uint32_t)(2 * I);
+    args.k = (uint32_t)K;
+    args.alpha = 1.0f;
+    hipStream_t st = (hipStream_t)stream;
+    // whether h is stored is a compile-time property of the kernel: the epilogue is then one straight-line block
+    if (h)
+        return dtype == FMA_BF16 ? ragged::launch<ElemBf16, true, true, EPI_SWIGLU, false>(args, st)
+                                 : ragged::launch<ElemF16, true, true, EPI_SWIGLU, false>(args, st);
+    return dtype == FMA_BF16 ? ragged::launch<ElemBf16, true, true, EPI_SWIGLU_ACT, false>(args, st)
+                             : ragged::launch<ElemF16, true, true, EPI_SWIGLU_ACT, false>(args, st);
+}
+
+}  // extern "C"

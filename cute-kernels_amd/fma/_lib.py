@@ -19,6 +19,7 @@ _LIB_PATH = os.environ.get("FMA_HIP_LIBRARY") or os.path.join(os.path.dirname(os
 _ABI_VERSION = 1
 
 FMA_F32, FMA_F16, FMA_BF16 = 0, 1, 2
+FMA_VARY_M, FMA_VARY_K = 0, 1
 _DTYPE_CODE = {torch.float32: FMA_F32, torch.float16: FMA_F16, torch.bfloat16: FMA_BF16}
 
 _p = ctypes.c_void_p
@@ -44,6 +45,7 @@ SIGNATURES = {
     "fma_swiglu_forward": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i32, _p]),
     "fma_swiglu_backward": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _p]),
     "fma_grouped_gemm": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _i32, _i32, _f32, _i32, _p]),
+    "fma_grouped_gemm_ragged": (_i32, [_p, _p, _p, _p, _i64, _i32, _i64, _i64, _i64, _i32, _i32, _f32, _i32, _p]),
     "fma_grouped_gemm_swiglu": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "fma_expert_bias_add": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "fma_expert_bias_grad_workspace_bytes": (_i64, [_i64, _i64, _i64]),

@@ -124,6 +124,49 @@ def combine_backward_cuda(
     _lib.check(rc, "combine_backward_cuda")
 
 
+@custom_op(f"{LIBRARY_NAME}::grouped_gemm_ragged_cuda", mutates_args={"output"})
+def grouped_gemm_ragged_cuda(
+    A: torch.Tensor, B: torch.Tensor, output: torch.Tensor, sizes: torch.Tensor, vary_k: bool, M: int, N: int, K: int,
+    is_A_transposed: bool, is_B_transposed: bool,
+) -> None:  # fmt: skip
+    """grouped_gemm for groups that differ in one dimension: `sizes` holds the rows of the groups (M is ignored) or, with
+    vary_k, their reduction lengths (K is ignored); the other two dimensions are plain integers (fma_grouped_gemm_ragged)."""
+    _lib.require_gpu(A, B, output, sizes)
+    assert A.dtype == B.dtype == output.dtype and A.dtype in (torch.bfloat16, torch.float16)
+    assert sizes.dtype == torch.uint32 and sizes.is_contiguous()
+    assert A.is_contiguous() and B.is_contiguous() and output.is_contiguous()
+    if output.numel() == 0:
+        return
+    # an operand without elements is never read, but the entry point rejects NULL: any valid device address stands in
+    a_ptr = A.data_ptr() if A.numel() else output.data_ptr()
+    b_ptr = B.data_ptr() if B.numel() else output.data_ptr()
+    with torch.cuda.device(A.device):
+        rc = _lib.load().fma_grouped_gemm_ragged(
+            a_ptr, b_ptr, output.data_ptr(), sizes.data_ptr(), sizes.numel(),
+            _lib.FMA_VARY_K if vary_k else _lib.FMA_VARY_M, M, N, K, int(is_A_transposed), int(is_B_transposed), 1.0,
+            _lib.dtype_code(A.dtype), _lib.current_stream(A.device),
+        )
+    _lib.check(rc, "grouped_gemm_ragged_cuda")
+
+
+def _expert_gemm(
+    A: torch.Tensor, B: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor,
+    output_shape: tuple[int, ...], vary: str, M: int, N: int, K: int, is_A_transposed: bool, is_B_transposed: bool,
+) -> torch.Tensor:  # fmt: skip
+    """One grouped GEMM of the expert path. `vary` names the array that holds the per-expert sizes ("M" or "K" of this
+    product); the other two dimensions are the module's constants M, N, K. 16-bit operands go through the entry point
+    that takes them by value, fp32 through `grouped_gemm` with the three arrays."""
+    if A.dtype in (torch.bfloat16, torch.float16):
+        output = A.new_empty(tuple(output_shape))
+        sizes = M_array if vary == "M" else K_array
+        grouped_gemm_ragged_cuda(A, B, output, sizes, vary == "K", M, N, K, is_A_transposed, is_B_transposed)
+        return output
+    return grouped_gemm(
+        A=A, B=B, C=None, M_array=M_array, N_array=N_array, K_array=K_array, output_shape=output_shape,
+        is_A_transposed=is_A_transposed, is_B_transposed=is_B_transposed,
+    )
+
+
 @custom_op(f"{LIBRARY_NAME}::grouped_gemm_swiglu_cuda", mutates_args={"h", "act"})
 def grouped_gemm_swiglu_cuda(
     x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, h: torch.Tensor | None, act: torch.Tensor
@@ -360,16 +403,8 @@ class _GroupedGemmExperts(torch.autograd.Function):
         assert N % 8 == 0
         assert K % 8 == 0
 
-        output = grouped_gemm(
-            A=x,
-            B=weight,
-            C=None,
-            M_array=M_array,
-            N_array=N_array,
-            K_array=K_array,
-            output_shape=(x.size(0), N),
-            is_A_transposed=False,
-            is_B_transposed=True,
+        output = _expert_gemm(
+            x, weight, M_array, N_array, K_array, (x.size(0), N), "M", 0, N, K, is_A_transposed=False, is_B_transposed=True
         )
 
         ctx.save_for_backward(x, weight, M_array, K_array, N_array)
@@ -380,34 +415,21 @@ class _GroupedGemmExperts(torch.autograd.Function):
     @ensure_contiguous
     def backward(ctx, output_grad: torch.Tensor) -> tuple[torch.Tensor | None]:
         x, weight, M_array, K_array, N_array = ctx.saved_tensors
+        _, N, K = weight.size()
         x_grad = weight_grad = None
 
         if ctx.needs_input_grad[0]:
             # dx_e = dy_e @ W_e : A = dy [sum(M), N], B = W_e stored [N, K] as a [K_gemm = N, N_gemm = K] matrix
-            x_grad = grouped_gemm(
-                A=output_grad,
-                B=weight,
-                C=None,
-                M_array=M_array,
-                N_array=K_array,
-                K_array=N_array,
-                output_shape=x.size(),
-                is_A_transposed=False,
-                is_B_transposed=False,
+            x_grad = _expert_gemm(
+                output_grad, weight, M_array, K_array, N_array, x.size(), "M", 0, K, N,
+                is_A_transposed=False, is_B_transposed=False,
             )
 
         if ctx.needs_input_grad[1]:
             # dW_e = dy_e^T @ x_e : both operands are stored with the reduction dim (the M_e rows) as row index
-            weight_grad = grouped_gemm(
-                A=output_grad,
-                B=x,
-                C=None,
-                M_array=N_array,
-                N_array=K_array,
-                K_array=M_array,
-                output_shape=weight.size(),
-                is_A_transposed=True,
-                is_B_transposed=False,
+            weight_grad = _expert_gemm(
+                output_grad, x, N_array, K_array, M_array, weight.size(), "K", N, K, 0,
+                is_A_transposed=True, is_B_transposed=False,
             )
 
         return x_grad, weight_grad, None, None, None
@@ -477,16 +499,17 @@ class _UpProjectionSwiglu(torch.autograd.Function):
         swiglu_backward_cuda(
             gate=gate, up=up, output_grad=act_grad, gate_grad=gate_grad, up_grad=up_grad, BLOCK_SIZE=1024
         )
+        _, N, K = weight.size()
         x_grad = weight_grad = None
         if ctx.needs_input_grad[0]:
-            x_grad = grouped_gemm(
-                A=h_grad, B=weight, C=None, M_array=M_array, N_array=K_array, K_array=N_array,
-                output_shape=x.size(), is_A_transposed=False, is_B_transposed=False,
+            x_grad = _expert_gemm(
+                h_grad, weight, M_array, K_array, N_array, x.size(), "M", 0, K, N,
+                is_A_transposed=False, is_B_transposed=False,
             )
         if ctx.needs_input_grad[1]:
-            weight_grad = grouped_gemm(
-                A=h_grad, B=x, C=None, M_array=N_array, N_array=K_array, K_array=M_array,
-                output_shape=weight.size(), is_A_transposed=True, is_B_transposed=False,
+            weight_grad = _expert_gemm(
+                h_grad, x, N_array, K_array, M_array, weight.size(), "K", N, K, 0,
+                is_A_transposed=True, is_B_transposed=False,
             )
         return x_grad, weight_grad, None, None, None, None
 

@@ -175,6 +175,24 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
                      const uint32_t* K_arr, int64_t E, int trans_a, int trans_b, float alpha, int dtype,
                      void* stream);
 
+/* which dimension differs between the groups of fma_grouped_gemm_ragged */
+#define FMA_VARY_M 0
+#define FMA_VARY_K 1
+
+/* fma_grouped_gemm for launches in which the groups differ in ONE dimension only, the case of every grouped GEMM of an
+ * MoE layer: `sizes` (E uint32, device memory) holds the rows M_e of the groups (vary == FMA_VARY_M: forward and
+ * input gradient; M is ignored) or their reduction lengths K_e (vary == FMA_VARY_K: weight gradient; K is ignored);
+ * the other two dimensions are the same for all groups and are passed by value. Same results, bit for bit, as
+ * fma_grouped_gemm with N_arr / K_arr (M_arr / N_arr) filled with those constants. Knowing them on the host lets the
+ * kernel keep a third of the group table and run the operand loads as one stream across tile boundaries, which is
+ * what the layer's GEMMs are launched through. dtype: FMA_BF16 or FMA_F16 (fp32 callers use fma_grouped_gemm).
+ * Replaces the same grouped_gemm_cuda calls as fma_grouped_gemm, as _GroupedGemmExperts makes them with
+ * N_array / K_array = full_like(M_array, N / K) (fma/modules/moe/__init__.py:82-83,
+ * fma/modules/moe/cuda_implementation/__init__.py:28-78). */
+int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_t* sizes, int64_t E, int vary,
+                            int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, float alpha, int dtype,
+                            void* stream);
+
 /* Up-projection with SwiGLU fused into the epilogue. For each expert e with M_e rows (rows of all experts
  * packed back to back, sum M_e = R):
  *   h_e   = x_e[M_e, K] * W_e[2I, K]^T            (rounded to dtype; written to h if h != NULL)
