@@ -237,13 +237,16 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         Tile t{};
         const uint32_t v = round * grid + ((round & 1u) ? grid - 1u - slot : slot);
         if ((uint64_t)round * grid >= total_tiles || v >= total_tiles) return t;
-        uint32_t lo = 0, hi = E;
-        while (lo < hi) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (s_tile_start[mid + 1] <= v) lo = mid + 1;
-            else hi = mid;
+        // position of the group that holds tile v: the number of groups whose tiles end at or before v. Every lane
+        // compares one table entry per 64 groups and a ballot counts them (a binary search would be ten dependent LDS
+        // round trips for 1024 groups; this is one per 64 groups, issued back to back).
+        uint32_t groups_before = 0;
+        for (uint32_t base = 0; base < E; base += 64u) {
+            const uint32_t p = base + lane;
+            const bool ends_before = p < E && s_tile_start[p + 1] <= v;
+            groups_before += (uint32_t)__builtin_popcountll(__ballot(ends_before));
         }
-        const uint32_t pos = uniform(lo);
+        const uint32_t pos = uniform(groups_before);
         const uint32_t e = uniform((uint32_t)s_order[pos]);
         t.valid = true;
         t.Me = group_m(e);
