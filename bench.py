@@ -209,8 +209,8 @@ def measure_workload(name, args, full):
 
     def gemm(A, B, D, sizes, vary, m, n, kk, ta, tb):
         # as the layer launches it: one size array (rows per expert) and the two dimensions all experts share by value
-        ok(lib.fma_grouped_gemm_ragged(A.data_ptr(), B.data_ptr(), D.data_ptr(), sizes.data_ptr(), E, vary, m, n, kk,
-                                       ta, tb, 1.0, BF16, stream))
+        ok(lib.fma_grouped_gemm_ragged(A.data_ptr(), B.data_ptr(), D.data_ptr(), sizes.data_ptr(), None, E, vary, m, n,
+                                       kk, ta, tb, 1.0, BF16, stream))
 
     ok(lib.fma_gather_rows(x.data_ptr(), perm.data_ptr(), R, H, k, xg.data_ptr(), BF16, stream))
     iters = max(20, args.steps)
@@ -243,12 +243,12 @@ def measure_workload(name, args, full):
 
     w1_b, w2_b = E * 2 * I * H * s, E * H * I * s  # bytes of the two weight tensors
     mfma("up_projection_swiglu_fwd(NT)", 2.0 * R * 2 * I * H,
-         lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), h.data_ptr(), a.data_ptr(),
+         lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), None, h.data_ptr(), a.data_ptr(),
                                                   counts.data_ptr(), E, I, H, BF16, stream)),
          nbytes=R * H * s + w1_b + R * 3 * I * s)
     # the same launch as a forward without a backward runs it: the pre-activation h is not stored
     mfma("up_projection_swiglu_fwd_inference(NT, h not stored)", 2.0 * R * 2 * I * H,
-         lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), None, a.data_ptr(),
+         lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), None, None, a.data_ptr(),
                                                   counts.data_ptr(), E, I, H, BF16, stream)),
          nbytes=R * H * s + w1_b + R * I * s)
     # the unfused pair the fused kernel above replaces (same bits): plain up-projection, then swiglu_forward below
@@ -283,7 +283,7 @@ def measure_workload(name, args, full):
     R_dec = M_dec * E
     counts_dec = torch.full((E,), M_dec, dtype=torch.int32, device=dev).view(torch.uint32)
     hbm(f"small_batch_up_fwd(NT + SwiGLU, {M_dec} rows per expert, h not stored)", w1_b + R_dec * (H + I) * s,
-        lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), None, a.data_ptr(),
+        lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), None, None, a.data_ptr(),
                                                  counts_dec.data_ptr(), E, I, H, BF16, stream)), n=30, gemm_kernel=True)
     hbm(f"small_batch_down_fwd(NT, {M_dec} rows per expert)", w2_b + R_dec * (H + I) * s,
         lambda i: gemm(a, w2, o, counts_dec, VARY_M, 0, H, I, 0, 1), n=30, gemm_kernel=True)

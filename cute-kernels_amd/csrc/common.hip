@@ -49,7 +49,7 @@ extern "C" {
 
 const char* fma_last_error_string(void) { return fmahip::g_error; }
 
-int fma_abi_version(void) { return 1; }
+int fma_abi_version(void) { return 2; }
 
 int fma_num_compute_units(void) { return fmahip::num_compute_units(); }
 

@@ -77,6 +77,14 @@ __device__ __forceinline__ void buffer_load_lds_quiet(u32x4 rsrc, uint32_t voff,
                  : "=&s"(saved_m0)
                  : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr));
 }
+// the 4-byte form of the same load (64 lanes x 4 bytes = 256 bytes of LDS per instruction)
+__device__ __forceinline__ void buffer_load_lds_quiet_b32(u32x4 rsrc, uint32_t voff, uint32_t soff, uint32_t lds_addr) {
+    uint32_t saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %4\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds\n\t"
+                 "s_mov_b32 m0, %0"
+                 : "=&s"(saved_m0)
+                 : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr));
+}
 __device__ __forceinline__ uint32_t lds_address(const uint8_t* p) {
     return (uint32_t)(uintptr_t)(lds_void*)const_cast<uint8_t*>(p);
 }
@@ -197,6 +205,18 @@ template <int ROWB>
 __device__ __forceinline__ void stage_put_quiet(uint32_t image, uint32_t m, uint32_t col, uint2 v) {
     const uint32_t addr = image + stage_off<ROWB>(m, col >> 3) + ((col >> 2) & 1u) * 8u;
     asm volatile("ds_write_b64 %0, %1" ::"v"(addr), "v"(__builtin_bit_cast(uint64_t, v)) : "memory");
+}
+// eight 8-byte reads at LDS byte addresses a[0..7], complete on return (written in assembly for the same reason)
+__device__ __forceinline__ void lds_read8x8_quiet(const uint32_t (&a)[8], uint2 (&v)[8]) {
+    uint64_t r[8];
+    asm volatile("ds_read_b64 %0, %8\n\tds_read_b64 %1, %9\n\tds_read_b64 %2, %10\n\tds_read_b64 %3, %11\n\t"
+                 "ds_read_b64 %4, %12\n\tds_read_b64 %5, %13\n\tds_read_b64 %6, %14\n\tds_read_b64 %7, %15\n\t"
+                 "s_waitcnt lgkmcnt(0)"
+                 : "=&v"(r[0]), "=&v"(r[1]), "=&v"(r[2]), "=&v"(r[3]), "=&v"(r[4]), "=&v"(r[5]), "=&v"(r[6]), "=&v"(r[7])
+                 : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(a[4]), "v"(a[5]), "v"(a[6]), "v"(a[7])
+                 : "memory");
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = __builtin_bit_cast(uint2, r[i]);
 }
 // two 16-byte reads of the image (at byte offsets off0 and off1), complete on return
 __device__ __forceinline__ void stage_get2_quiet(uint32_t image, uint32_t off0, uint32_t off1, u32x4& v0, u32x4& v1) {

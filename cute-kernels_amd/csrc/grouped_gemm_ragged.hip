@@ -43,6 +43,7 @@ struct Args {
     uint16_t* D;            // plain: output; swiglu: pre-activation h (may be NULL)
     uint16_t* ACT;          // swiglu only: activation output
     const uint32_t* sizes;  // E values of the varying dimension
+    const uint16_t* bias;   // BIAS kernels: [E, n] added to the rounded product before anything else
     uint32_t E;
     uint32_t m, n, k;  // the dimensions all groups share (the varying one is ignored)
     float alpha;
@@ -68,9 +69,10 @@ __device__ unsigned long long fma_prof[1024 * 8 * 8];
 #define PROF_STAMP(t) asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t))
 #endif
 
-template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K>
+template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K, bool BIAS>
 __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     static_assert(EPI == EPI_PLAIN || (A_KC && B_KC && !VARY_K), "the SwiGLU epilogue exists for the NT layout only");
+    static_assert(!BIAS || (A_KC && B_KC && !VARY_K), "the bias term exists for the forward (NT) layout only");
 
     // one array per stage and operand: distinct LDS objects let the compiler see that a direct-to-LDS load
     // into one stage cannot alias the fragment reads of the other, so it does not wait for the load first
@@ -80,6 +82,9 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     __shared__ __attribute__((aligned(1024))) uint8_t s_b1[kTileBytes];
     __shared__ __attribute__((aligned(1024))) uint8_t s_stage[NW * kStageBytes];
     __shared__ uint32_t s_pf[64];  // where the dwords fetched by the L2 prefetch end up (never read)
+    // BIAS: per wavefront, the bias values of the tile's 256 columns (plain) or 128 "up" | 128 "gate" columns
+    constexpr int kBiasBytes = 512;
+    __shared__ __attribute__((aligned(256))) uint8_t s_bias[BIAS ? NW * kBiasBytes : 16];
     // The group table, one LDS object: first tile of the group at position p of the tile sequence, exclusive prefix of the
     // varying dimension over the groups, and which group is at position p.
     __shared__ uint32_t s_table[2 * (FMA_MAX_GROUPS + 1) + FMA_MAX_GROUPS / 2];
@@ -230,6 +235,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     struct Tile {
         bool valid, fast;
         uint32_t Me, Ke, m0, n0, n_lim;  // n_lim: first column past the tile (kTileN columns wide, or half of that)
+        uint32_t e;                      // the group
         uint64_t off_a, off_b, off_d;
         uint32_t pf_r, pf_c;  // position of the tile in its XCD's 8 x 4 block of tiles (row, column)
     };
@@ -249,6 +255,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         const uint32_t pos = uniform(groups_before);
         const uint32_t e = uniform((uint32_t)s_order[pos]);
         t.valid = true;
+        t.e = e;
         t.Me = group_m(e);
         t.Ke = group_k(e);
         const uint32_t tiles_m = (t.Me + BM - 1) / BM;
@@ -544,10 +551,23 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             }
         };
         // waits of a step: all but the newest load when that is the previous step's prefetch; in a tile's first step the
-        // stores of the previous epilogue (or the cold start's stand-ins) are newer than the loads waited for as well
+        // stores of the previous epilogue (or the cold start's stand-ins) and the two loads of the bias tile are newer
+        // than the loads waited for as well
         using WaitStep = std::integral_constant<int, waitcnt_imm(kPrefetch ? 1 : 0, true)>;
-        using WaitFirst = std::integral_constant<int, waitcnt_imm((int)kTileStores + (kPrefetch ? 1 : 0), true)>;
+        using WaitFirst = std::integral_constant<int, waitcnt_imm((int)kTileStores + (kPrefetch ? 1 : 0) + (BIAS ? 2 : 0), true)>;
 
+        // BIAS: this tile's bias values into this wavefront's 512 bytes of LDS: two 256-byte loads, complete (loads and
+        // stores complete in issue order) long before the epilogue reads them. Columns past the end zero-fill.
+        auto issue_bias = [&]() {
+            if constexpr (BIAS) {
+                const uint16_t* row = args.bias + (uint64_t)cur.e * Ne;
+                const u32x4 rs = make_rsrc_words(row, Ne * 2u);
+                const uint32_t to = lds_address(s_bias) + wave * (uint32_t)kBiasBytes;
+                const uint32_t second = EPI != EPI_PLAIN ? n_span * 2u : 256u;  // byte offset of the second 128 columns
+                buffer_load_lds_quiet_b32(rs, n0 * 2u + lane * 4u, 0u, to);
+                buffer_load_lds_quiet_b32(rs, n0 * 2u + second + lane * 4u, 0u, to + 256u);
+            }
+        };
         Tile nn{};  // the tile after next
         const uint32_t tile_rows = Me - m0 < (uint32_t)BM ? Me - m0 : (uint32_t)BM;
         const uint32_t wave_rows = tile_rows > wm * WM ? tile_rows - wm * WM : 0u;
@@ -565,6 +585,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 if constexpr (B_KC) lk_b.issue_quiet_halves(lds_address(b_lo[st]), lds_address(b_hi[st]), k0);
                 else lt_b.issue_quiet_halves(lds_address(b_lo[st]), lds_address(b_hi[st]), k0);
             };
+            issue_bias();
             issue_thin(0, 0);
             issue_thin(1, BK);
             __builtin_amdgcn_s_waitcnt(waitcnt_imm((int)kThinLoads, false));
@@ -631,6 +652,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
             }
+            issue_bias();
             issue_prefetch(kPfDist - 1);
 #ifdef FMA_PROF
             PROF_STAMP(p_t1);
@@ -694,6 +716,10 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         p_seg[5] += KT2 > 2 ? KT2 - 2 : 0;
         ++p_tiles;
 #endif
+        if (BIAS && KT == 0) {  // a group without reduction: the result is the bias
+            issue_bias();
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, false));
+        }
         // the tile after next is looked up here: scalar work beside an epilogue that is bound by the store path
         nn = lookup(round + 2);
 #ifdef FMA_PROF
@@ -717,6 +743,38 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 for (int j = 0; j < FN; ++j) acc[i][j] *= alpha;
         }
         const bool upper = ((el >> 4) & 1u) != 0;  // this lane's row lies in the second 16 rows of its 32-row block
+        // BIAS: the eight groups of four columns this lane holds of every row block: [j][q], as fp32
+        float bias_f[FN][4][4];
+        if constexpr (BIAS) {
+            uint32_t at[8];
+            uint2 raw[8];
+            const uint32_t mine = lds_address(s_bias) + wave * (uint32_t)kBiasBytes;
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    // plain: column wn*64 + j*32 + ...; swiglu: "up" (j = 0) in the first 256 bytes, "gate" in the second
+                    const uint32_t c = (EPI == EPI_PLAIN ? wn * WN + j * 32 : j * 128 + wn * (WN / 2)) + q * 8 + (el >> 5) * 4;
+                    at[j * 4 + q] = mine + c * 2u;
+                }
+            lds_read8x8_quiet(at, raw);
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const uint2 r = raw[j * 4 + q];
+                    bias_f[j][q][0] = EL::from_bits((uint16_t)(r.x & 0xffffu));
+                    bias_f[j][q][1] = EL::from_bits((uint16_t)(r.x >> 16));
+                    bias_f[j][q][2] = EL::from_bits((uint16_t)(r.y & 0xffffu));
+                    bias_f[j][q][3] = EL::from_bits((uint16_t)(r.y >> 16));
+                }
+        }
+        // the value that is stored (plain) or activated (swiglu): the rounded product, plus the bias rounded again, which is
+        // what the product followed by a separate bias pass gives
+        auto with_bias = [&](float product, int j, int q, int x) -> float {
+            if constexpr (BIAS) return EL::round(product) + bias_f[j][q][x];
+            else return product;
+        };
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
             const uint32_t row0 = m0 + wm * WM + i * 32;  // first output row of this block
@@ -729,8 +787,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         const f32x16& c = acc[i][j];
-                        w[j][q].x = EL::pack2(c[q * 4 + 0], c[q * 4 + 1]);
-                        w[j][q].y = EL::pack2(c[q * 4 + 2], c[q * 4 + 3]);
+                        w[j][q].x = EL::pack2(with_bias(c[q * 4 + 0], j, q, 0), with_bias(c[q * 4 + 1], j, q, 1));
+                        w[j][q].y = EL::pack2(with_bias(c[q * 4 + 2], j, q, 2), with_bias(c[q * 4 + 3], j, q, 3));
                     }
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
@@ -758,8 +816,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                     float u[4], g[4], y[4];
 #pragma unroll
                     for (int x = 0; x < 4; ++x) {
-                        u[x] = EL::round(acc[i][0][q * 4 + x]);
-                        g[x] = EL::round(acc[i][1][q * 4 + x]);
+                        u[x] = EL::round(with_bias(acc[i][0][q * 4 + x], 0, q, x));
+                        g[x] = EL::round(with_bias(acc[i][1][q * 4 + x], 1, q, x));
                         y[x] = u[x] * g[x] * sigmoid_for<typename EL::act_t>(g[x]);
                     }
                     ypack[q][0] = EL::pack2(y[0], y[1]);
@@ -833,25 +891,28 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
 
 // every instantiation the entry points launch (explicit, so that host stub and device code are both emitted)
 #define FMA_RAGGED_INSTANTIATE(EL)                                                                          \
-    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, false>(const Args);                  \
-    template __global__ void ragged_gemm_kernel<EL, true, false, EPI_PLAIN, false>(const Args);                 \
-    template __global__ void ragged_gemm_kernel<EL, false, true, EPI_PLAIN, false>(const Args);                 \
-    template __global__ void ragged_gemm_kernel<EL, false, false, EPI_PLAIN, false>(const Args);                \
-    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, true>(const Args);                   \
-    template __global__ void ragged_gemm_kernel<EL, true, false, EPI_PLAIN, true>(const Args);                  \
-    template __global__ void ragged_gemm_kernel<EL, false, true, EPI_PLAIN, true>(const Args);                  \
-    template __global__ void ragged_gemm_kernel<EL, false, false, EPI_PLAIN, true>(const Args);                 \
-    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU, false>(const Args);                 \
-    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false>(const Args);
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, false, false>(const Args);           \
+    template __global__ void ragged_gemm_kernel<EL, true, false, EPI_PLAIN, false, false>(const Args);          \
+    template __global__ void ragged_gemm_kernel<EL, false, true, EPI_PLAIN, false, false>(const Args);          \
+    template __global__ void ragged_gemm_kernel<EL, false, false, EPI_PLAIN, false, false>(const Args);         \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, true, false>(const Args);            \
+    template __global__ void ragged_gemm_kernel<EL, true, false, EPI_PLAIN, true, false>(const Args);           \
+    template __global__ void ragged_gemm_kernel<EL, false, true, EPI_PLAIN, true, false>(const Args);           \
+    template __global__ void ragged_gemm_kernel<EL, false, false, EPI_PLAIN, true, false>(const Args);          \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU, false, false>(const Args);          \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false, false>(const Args);      \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, false, true>(const Args);            \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU, false, true>(const Args);           \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false, true>(const Args);
 FMA_RAGGED_INSTANTIATE(ElemBf16)
 FMA_RAGGED_INSTANTIATE(ElemF16)
 #undef FMA_RAGGED_INSTANTIATE
 
-template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K>
+template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K, bool BIAS = false>
 int launch(const Args& args, hipStream_t st) {
     int cus = num_compute_units();
     if (cus <= 0) cus = 256;
-    hipLaunchKernelGGL((ragged_gemm_kernel<EL, A_KC, B_KC, EPI, VARY_K>), dim3((uint32_t)cus), dim3(NT), 0, st, args);
+    hipLaunchKernelGGL((ragged_gemm_kernel<EL, A_KC, B_KC, EPI, VARY_K, BIAS>), dim3((uint32_t)cus), dim3(NT), 0, st, args);
     return launch_status("grouped_gemm_ragged");
 }
 
@@ -875,8 +936,8 @@ int fma_debug_prof(void* host, int64_t bytes) {
 }
 #endif
 
-int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_t* sizes, int64_t E, int vary,
-                            int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, float alpha, int dtype,
+int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_t* sizes, const void* bias, int64_t E,
+                            int vary, int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, float alpha, int dtype,
                             void* stream) {
     using namespace fmahip;
     using namespace fmahip::gemm;
@@ -899,17 +960,29 @@ int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_
     hipStream_t st = (hipStream_t)stream;
     const bool a_kc = trans_a == 0;  // A stored [M, K]: reduction dim contiguous
     const bool b_kc = trans_b != 0;  // B stored [N, K]: reduction dim contiguous
+    FMA_REQUIRE(!bias || (vary == FMA_VARY_M && a_kc && b_kc && alpha == 1.0f), FMA_ERR_UNSUPPORTED,
+                "grouped_gemm_ragged: a bias is added in the forward form only (rows vary, A not transposed, B transposed, "
+                "alpha 1)");
+    // (with these sizes every tile takes the matrix-instruction path, the only one that adds the bias)
+    FMA_REQUIRE(!bias || (N % 8 == 0 && K % 8 == 0 && N < (1 << 23) && K < (1 << 21)), FMA_ERR_UNSUPPORTED,
+                "grouped_gemm_ragged: with a bias, N and K must be multiples of 8, N < 2^23 and K < 2^21");
+    FMA_REQUIRE(!bias || (reinterpret_cast<uintptr_t>(bias) & 3u) == 0, FMA_ERR_MISALIGNED,
+                "grouped_gemm_ragged: the bias must be 4-byte aligned");
     ragged::Args args{};
     args.A = (const uint16_t*)A;
     args.B = (const uint16_t*)B;
     args.D = (uint16_t*)D;
     args.ACT = nullptr;
     args.sizes = sizes;
+    args.bias = (const uint16_t*)bias;
     args.E = (uint32_t)E;
     args.m = (uint32_t)M;
     args.n = (uint32_t)N;
     args.k = (uint32_t)K;
     args.alpha = alpha;
+    if (bias)
+        return dtype == FMA_BF16 ? ragged::launch<ElemBf16, true, true, EPI_PLAIN, false, true>(args, st)
+                                 : ragged::launch<ElemF16, true, true, EPI_PLAIN, false, true>(args, st);
     if (vary == FMA_VARY_K)
         return dtype == FMA_BF16 ? ragged::launch_plain<ElemBf16, true>(args, a_kc, b_kc, st)
                                  : ragged::launch_plain<ElemF16, true>(args, a_kc, b_kc, st);
@@ -917,8 +990,8 @@ int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_
                              : ragged::launch_plain<ElemF16, false>(args, a_kc, b_kc, st);
 }
 
-int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, const uint32_t* M_arr, int64_t E,
-                            int64_t I, int64_t K, int dtype, void* stream) {
+int fma_grouped_gemm_swiglu(const void* x, const void* W, const void* bias, void* h, void* act, const uint32_t* M_arr,
+                            int64_t E, int64_t I, int64_t K, int dtype, void* stream) {
     using namespace fmahip;
     using namespace fmahip::gemm;
     FMA_REQUIRE(dtype == FMA_BF16 || dtype == FMA_F16, dtype_bytes(dtype) ? FMA_ERR_UNSUPPORTED : FMA_ERR_BAD_DTYPE,
@@ -935,7 +1008,10 @@ int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, co
     FMA_REQUIRE(x && W && act && M_arr, FMA_ERR_NULL_POINTER, "grouped_gemm_swiglu: NULL pointer");
     FMA_REQUIRE(aligned16(x) && aligned16(W) && aligned16(act) && aligned16(h), FMA_ERR_MISALIGNED,
                 "grouped_gemm_swiglu: x, W, h and act must be 16-byte aligned");
+    FMA_REQUIRE((reinterpret_cast<uintptr_t>(bias) & 3u) == 0, FMA_ERR_MISALIGNED,
+                "grouped_gemm_swiglu: the bias must be 4-byte aligned");
     ragged::Args args{};
+    args.bias = (const uint16_t*)bias;
     args.A = (const uint16_t*)x;
     args.B = (const uint16_t*)W;
     args.D = (uint16_t*)h;
@@ -948,6 +1024,13 @@ int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, co
     args.alpha = 1.0f;
     hipStream_t st = (hipStream_t)stream;
     // whether h is stored is a compile-time property of the kernel: the epilogue is then one straight-line block
+    if (bias) {
+        if (h)
+            return dtype == FMA_BF16 ? ragged::launch<ElemBf16, true, true, EPI_SWIGLU, false, true>(args, st)
+                                     : ragged::launch<ElemF16, true, true, EPI_SWIGLU, false, true>(args, st);
+        return dtype == FMA_BF16 ? ragged::launch<ElemBf16, true, true, EPI_SWIGLU_ACT, false, true>(args, st)
+                                 : ragged::launch<ElemF16, true, true, EPI_SWIGLU_ACT, false, true>(args, st);
+    }
     if (h)
         return dtype == FMA_BF16 ? ragged::launch<ElemBf16, true, true, EPI_SWIGLU, false>(args, st)
                                  : ragged::launch<ElemF16, true, true, EPI_SWIGLU, false>(args, st);

@@ -16,7 +16,7 @@ import torch
 _LIB_NAME = "libfma_hip.so"
 # FMA_HIP_LIBRARY names another build of the same library (e.g. one compiled with different tuning macros)
 _LIB_PATH = os.environ.get("FMA_HIP_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
-_ABI_VERSION = 1
+_ABI_VERSION = 2
 
 FMA_F32, FMA_F16, FMA_BF16 = 0, 1, 2
 FMA_VARY_M, FMA_VARY_K = 0, 1
@@ -45,8 +45,8 @@ SIGNATURES = {
     "fma_swiglu_forward": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i32, _p]),
     "fma_swiglu_backward": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _p]),
     "fma_grouped_gemm": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _i32, _i32, _f32, _i32, _p]),
-    "fma_grouped_gemm_ragged": (_i32, [_p, _p, _p, _p, _i64, _i32, _i64, _i64, _i64, _i32, _i32, _f32, _i32, _p]),
-    "fma_grouped_gemm_swiglu": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
+    "fma_grouped_gemm_ragged": (_i32, [_p, _p, _p, _p, _p, _i64, _i32, _i64, _i64, _i64, _i32, _i32, _f32, _i32, _p]),
+    "fma_grouped_gemm_swiglu": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "fma_expert_bias_add": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "fma_expert_bias_grad_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "fma_expert_bias_grad": (_i32, [_p, _p, _i64, _i64, _i64, _p, _p, _i64, _i32, _p]),

@@ -43,19 +43,18 @@ class Experts(nn.Module):
 
     def cuda_forward(self, input: torch.Tensor, expert_frequency: torch.Tensor) -> torch.Tensor:
         # the reference's cuda_forward (fma/modules/moe/__init__.py:89-92) silently drops the bias; here it is added
-        # to the rows of every expert, which is what its torch_forward computes (:98-105)
-        output = grouped_gemm_experts(
-            x=input, weight=self.weight, M_array=expert_frequency, N_array=self.N_array, K_array=self.K_array
+        # to the rows of every expert (in the GEMM's epilogue for 16-bit types), which is what its torch_forward
+        # computes (:98-105)
+        return grouped_gemm_experts(
+            x=input, weight=self.weight, M_array=expert_frequency, N_array=self.N_array, K_array=self.K_array,
+            bias=self.bias,
         )
-        if self.bias is not None:
-            output = add_expert_bias(output, self.bias, expert_frequency)
-        return output
 
     def cuda_forward_swiglu(self, input: torch.Tensor, expert_frequency: torch.Tensor) -> torch.Tensor:
         """up-projection with swiglu_packed fused into the GEMM epilogue: returns [sum(M), out_features / 2]"""
-        assert self.bias is None, "the fused epilogue has no bias term: use cuda_forward followed by the activation"
         return up_projection_swiglu_experts(
-            x=input, weight=self.weight, M_array=expert_frequency, N_array=self.N_array, K_array=self.K_array
+            x=input, weight=self.weight, M_array=expert_frequency, N_array=self.N_array, K_array=self.K_array,
+            bias=self.bias,
         )
 
     def extra_repr(self) -> str:
@@ -114,7 +113,6 @@ class MoE(nn.Module):
         self.fuse_swiglu = (
             is_glu
             and _is_swiglu_packed(activation_function)
-            and not add_bias
             and self.hidden_size % 8 == 0
             and self.intermediate_size % 8 == 0
         )

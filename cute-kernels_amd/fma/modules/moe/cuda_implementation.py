@@ -127,14 +127,16 @@ def combine_backward_cuda(
 @custom_op(f"{LIBRARY_NAME}::grouped_gemm_ragged_cuda", mutates_args={"output"})
 def grouped_gemm_ragged_cuda(
     A: torch.Tensor, B: torch.Tensor, output: torch.Tensor, sizes: torch.Tensor, vary_k: bool, M: int, N: int, K: int,
-    is_A_transposed: bool, is_B_transposed: bool,
+    is_A_transposed: bool, is_B_transposed: bool, bias: torch.Tensor | None = None,
 ) -> None:  # fmt: skip
     """grouped_gemm for groups that differ in one dimension: `sizes` holds the rows of the groups (M is ignored) or, with
-    vary_k, their reduction lengths (K is ignored); the other two dimensions are plain integers (fma_grouped_gemm_ragged)."""
-    _lib.require_gpu(A, B, output, sizes)
+    vary_k, their reduction lengths (K is ignored); the other two dimensions are plain integers (fma_grouped_gemm_ragged).
+    `bias` [E, N] is added to the rows of every group in the epilogue (forward form only)."""
+    _lib.require_gpu(A, B, output, sizes, bias)
     assert A.dtype == B.dtype == output.dtype and A.dtype in (torch.bfloat16, torch.float16)
     assert sizes.dtype == torch.uint32 and sizes.is_contiguous()
     assert A.is_contiguous() and B.is_contiguous() and output.is_contiguous()
+    assert bias is None or (bias.shape == (sizes.numel(), N) and bias.dtype == A.dtype and bias.is_contiguous())
     if output.numel() == 0:
         return
     # an operand without elements is never read, but the entry point rejects NULL: any valid device address stands in
@@ -142,7 +144,7 @@ def grouped_gemm_ragged_cuda(
     b_ptr = B.data_ptr() if B.numel() else output.data_ptr()
     with torch.cuda.device(A.device):
         rc = _lib.load().fma_grouped_gemm_ragged(
-            a_ptr, b_ptr, output.data_ptr(), sizes.data_ptr(), sizes.numel(),
+            a_ptr, b_ptr, output.data_ptr(), sizes.data_ptr(), _lib.ptr(bias), sizes.numel(),
             _lib.FMA_VARY_K if vary_k else _lib.FMA_VARY_M, M, N, K, int(is_A_transposed), int(is_B_transposed), 1.0,
             _lib.dtype_code(A.dtype), _lib.current_stream(A.device),
         )
@@ -152,15 +154,17 @@ def grouped_gemm_ragged_cuda(
 def _expert_gemm(
     A: torch.Tensor, B: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor,
     output_shape: tuple[int, ...], vary: str, M: int, N: int, K: int, is_A_transposed: bool, is_B_transposed: bool,
+    bias: torch.Tensor | None = None,
 ) -> torch.Tensor:  # fmt: skip
     """One grouped GEMM of the expert path. `vary` names the array that holds the per-expert sizes ("M" or "K" of this
     product); the other two dimensions are the module's constants M, N, K. 16-bit operands go through the entry point
-    that takes them by value, fp32 through `grouped_gemm` with the three arrays."""
+    that takes them by value (the only one with a bias term), fp32 through `grouped_gemm` with the three arrays."""
     if A.dtype in (torch.bfloat16, torch.float16):
         output = A.new_empty(tuple(output_shape))
         sizes = M_array if vary == "M" else K_array
-        grouped_gemm_ragged_cuda(A, B, output, sizes, vary == "K", M, N, K, is_A_transposed, is_B_transposed)
+        grouped_gemm_ragged_cuda(A, B, output, sizes, vary == "K", M, N, K, is_A_transposed, is_B_transposed, bias)
         return output
+    assert bias is None
     return grouped_gemm(
         A=A, B=B, C=None, M_array=M_array, N_array=N_array, K_array=K_array, output_shape=output_shape,
         is_A_transposed=is_A_transposed, is_B_transposed=is_B_transposed,
@@ -169,9 +173,10 @@ def _expert_gemm(
 
 @custom_op(f"{LIBRARY_NAME}::grouped_gemm_swiglu_cuda", mutates_args={"h", "act"})
 def grouped_gemm_swiglu_cuda(
-    x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, h: torch.Tensor | None, act: torch.Tensor
-) -> None:
-    _lib.require_gpu(x, weight, M_array, h, act)
+    x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, h: torch.Tensor | None, act: torch.Tensor,
+    bias: torch.Tensor | None = None,
+) -> None:  # fmt: skip
+    _lib.require_gpu(x, weight, M_array, h, act, bias)
     E, N, K = weight.shape
     assert N % 2 == 0
     inter = N // 2
@@ -179,13 +184,14 @@ def grouped_gemm_swiglu_cuda(
     assert x.shape == (R, K) and act.shape == (R, inter) and (h is None or h.shape == (R, N))
     assert x.dtype == weight.dtype == act.dtype and (h is None or h.dtype == x.dtype)
     assert M_array.dtype == torch.uint32 and M_array.numel() == E
-    for t in (x, weight, M_array, h, act):
+    assert bias is None or (bias.shape == (E, N) and bias.dtype == x.dtype)
+    for t in (x, weight, M_array, h, act, bias):
         assert t is None or t.is_contiguous()
     if act.numel() == 0:
         return  # no rows routed anywhere (or no output columns): nothing to compute, and empty tensors have no address
     with torch.cuda.device(x.device):
         rc = _lib.load().fma_grouped_gemm_swiglu(
-            x.data_ptr(), weight.data_ptr(), _lib.ptr(h), act.data_ptr(), M_array.data_ptr(), E, inter, K,
+            x.data_ptr(), weight.data_ptr(), _lib.ptr(bias), _lib.ptr(h), act.data_ptr(), M_array.data_ptr(), E, inter, K,
             _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
         )
     _lib.check(rc, "grouped_gemm_swiglu_cuda")
@@ -389,14 +395,15 @@ class _Combine(torch.autograd.Function):
 
 
 class _GroupedGemmExperts(torch.autograd.Function):
-    """y_e = x_e @ W_e^T per expert; the three GEMMs of the reference's _GroupedGemmExperts
-    (fma/modules/moe/cuda_implementation/__init__.py:15-80)."""
+    """y_e = x_e @ W_e^T (+ bias_e, 16-bit types: added in the GEMM's epilogue) per expert; the three GEMMs of the
+    reference's _GroupedGemmExperts (fma/modules/moe/cuda_implementation/__init__.py:15-80)."""
 
     @staticmethod
     @ensure_contiguous
     def forward(
-        ctx, x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor
-    ) -> torch.Tensor:
+        ctx, x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor,
+        bias: torch.Tensor | None = None,
+    ) -> torch.Tensor:  # fmt: skip
         # x -> sum(M) x K, weight -> E x N x K
         _, N, K = weight.size()
 
@@ -404,7 +411,8 @@ class _GroupedGemmExperts(torch.autograd.Function):
         assert K % 8 == 0
 
         output = _expert_gemm(
-            x, weight, M_array, N_array, K_array, (x.size(0), N), "M", 0, N, K, is_A_transposed=False, is_B_transposed=True
+            x, weight, M_array, N_array, K_array, (x.size(0), N), "M", 0, N, K, is_A_transposed=False, is_B_transposed=True,
+            bias=bias,
         )
 
         ctx.save_for_backward(x, weight, M_array, K_array, N_array)
@@ -416,7 +424,7 @@ class _GroupedGemmExperts(torch.autograd.Function):
     def backward(ctx, output_grad: torch.Tensor) -> tuple[torch.Tensor | None]:
         x, weight, M_array, K_array, N_array = ctx.saved_tensors
         _, N, K = weight.size()
-        x_grad = weight_grad = None
+        x_grad = weight_grad = bias_grad = None
 
         if ctx.needs_input_grad[0]:
             # dx_e = dy_e @ W_e : A = dy [sum(M), N], B = W_e stored [N, K] as a [K_gemm = N, N_gemm = K] matrix
@@ -432,7 +440,11 @@ class _GroupedGemmExperts(torch.autograd.Function):
                 is_A_transposed=True, is_B_transposed=False,
             )
 
-        return x_grad, weight_grad, None, None, None
+        if len(ctx.needs_input_grad) > 5 and ctx.needs_input_grad[5]:
+            bias_grad = torch.empty(weight.size(0), N, device=output_grad.device, dtype=output_grad.dtype)
+            expert_bias_grad_cuda(output_grad, M_array, bias_grad)
+
+        return (x_grad, weight_grad, None, None, None, bias_grad)[: len(ctx.needs_input_grad)]
 
 
 class _ExpertBias(torch.autograd.Function):
@@ -471,7 +483,7 @@ class _UpProjectionSwiglu(torch.autograd.Function):
     @ensure_contiguous
     def forward(
         ctx, x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor,
-        grad_enabled: bool,
+        grad_enabled: bool, bias: torch.Tensor | None = None,
     ) -> torch.Tensor:  # fmt: skip
         _, N, K = weight.size()
         assert N % 16 == 0
@@ -479,10 +491,10 @@ class _UpProjectionSwiglu(torch.autograd.Function):
         R = x.size(0)
         # needs_input_grad only says that an input requires grad; under no_grad / inference_mode no backward will
         # follow (grad mode is always off inside forward, so the caller passes what it was outside)
-        needs_backward = grad_enabled and any(ctx.needs_input_grad[:2])
+        needs_backward = grad_enabled and any(ctx.needs_input_grad)
         h = torch.empty(R, N, device=x.device, dtype=x.dtype) if needs_backward else None
         act = torch.empty(R, N // 2, device=x.device, dtype=x.dtype)
-        grouped_gemm_swiglu_cuda(x, weight, M_array, h, act)
+        grouped_gemm_swiglu_cuda(x, weight, M_array, h, act, bias)
         if needs_backward:
             ctx.save_for_backward(x, weight, h, M_array, K_array, N_array)
         return act
@@ -500,7 +512,7 @@ class _UpProjectionSwiglu(torch.autograd.Function):
             gate=gate, up=up, output_grad=act_grad, gate_grad=gate_grad, up_grad=up_grad, BLOCK_SIZE=1024
         )
         _, N, K = weight.size()
-        x_grad = weight_grad = None
+        x_grad = weight_grad = bias_grad = None
         if ctx.needs_input_grad[0]:
             x_grad = _expert_gemm(
                 h_grad, weight, M_array, K_array, N_array, x.size(), "M", 0, K, N,
@@ -511,7 +523,10 @@ class _UpProjectionSwiglu(torch.autograd.Function):
                 h_grad, x, N_array, K_array, M_array, weight.size(), "K", N, K, 0,
                 is_A_transposed=True, is_B_transposed=False,
             )
-        return x_grad, weight_grad, None, None, None, None
+        if len(ctx.needs_input_grad) > 6 and ctx.needs_input_grad[6]:
+            bias_grad = torch.empty(weight.size(0), N, device=h_grad.device, dtype=h_grad.dtype)
+            expert_bias_grad_cuda(h_grad, M_array, bias_grad)
+        return (x_grad, weight_grad, None, None, None, None, bias_grad)[: len(ctx.needs_input_grad)]
 
 
 # ---- the reference's padded grouping interface -------------------------------------------------------
@@ -668,12 +683,21 @@ def combine(o: torch.Tensor, gates: torch.Tensor, inv: torch.Tensor) -> torch.Te
 
 
 def grouped_gemm_experts(
-    x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor
-) -> torch.Tensor:
-    return _GroupedGemmExperts.apply(x, weight, M_array, N_array, K_array)
+    x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor,
+    bias: torch.Tensor | None = None,
+) -> torch.Tensor:  # fmt: skip
+    """y_e = x_e @ W_e^T + bias_e. The 16-bit kernel adds the bias in its epilogue (within its size limits); otherwise
+    it is a pass of its own over the fresh output."""
+    if bias is None:
+        return _GroupedGemmExperts.apply(x, weight, M_array, N_array, K_array)
+    _, N, K = weight.size()
+    if x.dtype in (torch.bfloat16, torch.float16) and bias.dtype == x.dtype and N < (1 << 23) and K < (1 << 21):
+        return _GroupedGemmExperts.apply(x, weight, M_array, N_array, K_array, bias)
+    return add_expert_bias(_GroupedGemmExperts.apply(x, weight, M_array, N_array, K_array), bias, M_array)
 
 
 def up_projection_swiglu_experts(
-    x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor
-) -> torch.Tensor:
-    return _UpProjectionSwiglu.apply(x, weight, M_array, N_array, K_array, torch.is_grad_enabled())
+    x: torch.Tensor, weight: torch.Tensor, M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor,
+    bias: torch.Tensor | None = None,
+) -> torch.Tensor:  # fmt: skip
+    return _UpProjectionSwiglu.apply(x, weight, M_array, N_array, K_array, torch.is_grad_enabled(), bias)

@@ -186,11 +186,15 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
  * fma_grouped_gemm with N_arr / K_arr (M_arr / N_arr) filled with those constants. Knowing them on the host lets the
  * kernel keep a third of the group table and run the operand loads as one stream across tile boundaries, which is
  * what the layer's GEMMs are launched through. dtype: FMA_BF16 or FMA_F16 (fp32 callers use fma_grouped_gemm).
+ * bias: NULL, or [E, N] of dtype (4-byte aligned, N even) added to every row of its group in the epilogue: the rounded
+ * product plus the bias in fp32, rounded once more, bit for bit what fma_expert_bias_add does to the output of the call
+ * without a bias. Only in the forward form (vary == FMA_VARY_M, trans_a == 0, trans_b != 0, alpha == 1).
  * Replaces the same grouped_gemm_cuda calls as fma_grouped_gemm, as _GroupedGemmExperts makes them with
  * N_array / K_array = full_like(M_array, N / K) (fma/modules/moe/__init__.py:82-83,
- * fma/modules/moe/cuda_implementation/__init__.py:28-78). */
-int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_t* sizes, int64_t E, int vary,
-                            int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, float alpha, int dtype,
+ * fma/modules/moe/cuda_implementation/__init__.py:28-78); with a bias, the per-expert F.linear(x_e, W[e], bias[e])
+ * of Experts.torch_forward (fma/modules/moe/__init__.py:98-105). */
+int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_t* sizes, const void* bias, int64_t E,
+                            int vary, int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, float alpha, int dtype,
                             void* stream);
 
 /* Up-projection with SwiGLU fused into the epilogue. For each expert e with M_e rows (rows of all experts
@@ -199,9 +203,11 @@ int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_
  *   act_e = h_e[:, :I] * silu(h_e[:, I:])         (first half "up", second half "gate")
  * computed from the ROUNDED h so the result equals fma_grouped_gemm followed by fma_swiglu_forward bit for
  * bit. W: [E, 2I, K] row-major; h: [R, 2I]; act: [R, I]; I % 8 == 0, K % 8 == 0, I < 2^22, K < 2^21.
+ * bias: NULL, or [E, 2I] of dtype (4-byte aligned), added to h as fma_expert_bias_add would (rounded product plus bias,
+ * rounded again) before the activation.
  * Fuses _GroupedGemmExperts.forward (fma/modules/moe/cuda_implementation/__init__.py:28-38) with
  * swiglu_packed (fma/ops/swiglu/__init__.py:133-164, up/gate = chunk(2, -1) at :153). */
-int fma_grouped_gemm_swiglu(const void* x, const void* W, void* h, void* act, const uint32_t* M_arr,
+int fma_grouped_gemm_swiglu(const void* x, const void* W, const void* bias, void* h, void* act, const uint32_t* M_arr,
                             int64_t E, int64_t I, int64_t K, int dtype, void* stream);
 
 /* ---- per-expert bias ------------------------------------------------------------------------ */

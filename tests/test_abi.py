@@ -27,7 +27,7 @@ def test_header_and_binding_agree():
 def test_library_exports_every_declared_symbol(lib):
     for name in _declared_symbols():
         assert hasattr(lib, name), f"libfma_hip.so does not export {name}"
-    assert lib.fma_abi_version() == 1
+    assert lib.fma_abi_version() == 2
 
 
 def test_workspace_queries(lib):
@@ -86,14 +86,14 @@ def test_swiglu_and_gemm_validation(lib):
     assert lib.fma_swiglu_backward(p, p, p, p, None, 4, 8, 8, 8, 8, 8, 8, 2, None) == -1
     assert lib.fma_grouped_gemm(p, p, p, p, p, p, 1025, 0, 1, 1.0, 2, None) == -4 and "1024" in _err(lib)
     assert lib.fma_grouped_gemm(p + 4, p, p, p, p, p, 4, 0, 1, 1.0, 0, None) == -6  # fp32 operands: same alignment rule
-    assert lib.fma_grouped_gemm_swiglu(p, p, p, p, p, 4, 16, 64, 0, None) == -8  # the fused epilogue is 16-bit only
+    assert lib.fma_grouped_gemm_swiglu(p, p, None, p, p, p, 4, 16, 64, 0, None) == -8  # the fused epilogue is 16-bit only
     assert lib.fma_grouped_gemm(p, p, p, p, p, p, 4, 0, 1, 1.0, 5, None) == -2
     assert lib.fma_grouped_gemm(p, p, p, None, p, p, 4, 0, 1, 1.0, 2, None) == -1
     assert lib.fma_grouped_gemm(p, p, p, p, p, p, 0, 0, 1, 1.0, 2, None) == 0
-    assert lib.fma_grouped_gemm_swiglu(p, p, p, p, p, 4, 12, 64, 2, None) == -3  # I % 8 != 0
-    assert lib.fma_grouped_gemm_swiglu(p, p, p, p, p, 4, 16, 60, 2, None) == -3  # K % 8 != 0
-    assert lib.fma_grouped_gemm_swiglu(p, p, p, p, p, 4, 1 << 22, 64, 2, None) == -3  # beyond the 32-bit tile offsets
-    assert lib.fma_grouped_gemm_swiglu(p, p, p, p, p, 4, 16, 1 << 21, 2, None) == -3
+    assert lib.fma_grouped_gemm_swiglu(p, p, None, p, p, p, 4, 12, 64, 2, None) == -3  # I % 8 != 0
+    assert lib.fma_grouped_gemm_swiglu(p, p, None, p, p, p, 4, 16, 60, 2, None) == -3  # K % 8 != 0
+    assert lib.fma_grouped_gemm_swiglu(p, p, None, p, p, p, 4, 1 << 22, 64, 2, None) == -3  # beyond the 32-bit tile offsets
+    assert lib.fma_grouped_gemm_swiglu(p, p, None, p, p, p, 4, 16, 1 << 21, 2, None) == -3
 
 
 def test_router_norm_and_bias_validation(lib):

@@ -6,7 +6,12 @@ import torch
 import torch.nn as nn
 
 from fma import KernelBackend, MoE, swiglu_packed
-from fma.modules.moe.cuda_implementation import expert_bias_add_cuda, expert_bias_grad_cuda
+from fma.modules.moe.cuda_implementation import (
+    expert_bias_add_cuda,
+    expert_bias_grad_cuda,
+    grouped_gemm_ragged_cuda,
+    grouped_gemm_swiglu_cuda,
+)
 from oracle import moe_oracle as O
 
 from gpu_util import DEV, rel_err
@@ -65,6 +70,74 @@ def test_bias_grad_is_the_segmented_column_sum(dtype, counts, N):
             assert float(got[e].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize(
+    "counts,N,K",
+    [
+        ([300, 1, 0, 4095, 17, 0, 256, 2], 4096, 512),  # thin groups, empty groups, 16 column tiles
+        ([2048 + 8 * (e % 7) for e in range(24)], 1024, 512),  # every workgroup streams through several tiles
+        ([40] * 64, 136, 192),  # half-width tiles, a last column tile of 8 columns, 3 K steps
+        ([1000, 520, 8], 264, 64),  # one K step per tile; columns end inside a tile
+        ([700, 0, 33], 512, 0),  # no reduction at all: the output is the bias
+    ],
+)
+def test_bias_in_the_gemm_epilogue_equals_gemm_then_bias_add(dtype, counts, N, K):
+    torch.manual_seed(N + K)
+    R, E = sum(counts), len(counts)
+    x = torch.randn(R, K, device=DEV).to(dtype)
+    w = (torch.randn(E, N, K, device=DEV) * 0.2).to(dtype)
+    bias = torch.randn(E, N, device=DEV).to(dtype)
+    M = _counts_tensor(counts)
+    two_pass = torch.full((R, N), 7.0, dtype=dtype, device=DEV)
+    grouped_gemm_ragged_cuda(x, w, two_pass, M, False, 0, N, K, False, True)
+    expert_bias_add_cuda(two_pass, bias, M)
+    fused = torch.full((R, N), 7.0, dtype=dtype, device=DEV)
+    grouped_gemm_ragged_cuda(x, w, fused, M, False, 0, N, K, False, True, bias)
+    assert torch.equal(fused, two_pass)
+    # and against the definition: per-expert linear in fp64, rounded, plus the bias, rounded
+    off = 0
+    for e, c in enumerate(counts):
+        if c and c <= 1000:
+            y = (x[off:off + c].double() @ w[e].double().T).to(dtype)
+            expect = (y.float() + bias[e].float()).to(dtype)
+            # (the fp32-accumulated product may round to the neighbour of the fp64 one: one step of the product's size)
+            eps = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
+            bad = (fused[off:off + c].float() - expect.float()).abs() > eps * (y.float().abs() + expect.float().abs()) + 1e-3
+            assert int(bad.sum()) == 0
+        off += c
+
+
+@pytest.mark.parametrize("counts,I,K", [([100, 0, 300, 1], 128, 64), ([40] * 16, 72, 520), ([3000, 0, 5000, 1, 4999], 1408, 520)])
+def test_bias_in_the_fused_swiglu_epilogue(counts, I, K):
+    torch.manual_seed(I + K)
+    R, E = sum(counts), len(counts)
+    x = torch.randn(R, K, device=DEV).bfloat16()
+    w = (torch.randn(E, 2 * I, K, device=DEV) * 0.1).bfloat16()
+    bias = torch.randn(E, 2 * I, device=DEV).bfloat16()
+    M = _counts_tensor(counts)
+    h_ref = torch.empty(R, 2 * I, dtype=torch.bfloat16, device=DEV)
+    grouped_gemm_ragged_cuda(x, w, h_ref, M, False, 0, 2 * I, K, False, True)
+    expert_bias_add_cuda(h_ref, bias, M)
+    h = torch.empty_like(h_ref)
+    act = torch.empty(R, I, dtype=torch.bfloat16, device=DEV)
+    grouped_gemm_swiglu_cuda(x, w, M, h, act, bias)
+    assert torch.equal(h, h_ref)
+    assert torch.equal(act, swiglu_packed(h_ref))
+    act_only = torch.empty_like(act)
+    grouped_gemm_swiglu_cuda(x, w, M, None, act_only, bias)
+    assert torch.equal(act_only, act)
+
+
+def test_bias_in_the_epilogue_is_refused_outside_the_forward_form():
+    x = torch.zeros(64, 64, device=DEV, dtype=torch.bfloat16)
+    out = torch.zeros(64, 64, device=DEV, dtype=torch.bfloat16)
+    bias = torch.zeros(1, 64, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="forward form"):
+        grouped_gemm_ragged_cuda(x, x, out, _counts_tensor([64]), False, 0, 64, 64, False, False, bias)
+    with pytest.raises(RuntimeError, match="forward form"):
+        grouped_gemm_ragged_cuda(x, x, out, _counts_tensor([64]), True, 64, 64, 0, False, True, bias)
+
+
 def _glu(x):
     a, b = x.chunk(2, dim=-1)
     return a * torch.sigmoid(b)
@@ -78,7 +151,7 @@ def test_moe_layer_with_bias(act_name, E, k, H, I, T):
     act = {"swiglu": swiglu_packed, "glu": nn.GLU(), "gelu": nn.GELU(approximate="tanh")}[act_name]
     oracle_act = {"swiglu": O.swiglu_packed, "glu": _glu, "gelu": nn.GELU(approximate="tanh")}[act_name]
     moe = MoE(E, k, H, I, act, is_glu, True, 0.02).to(torch.bfloat16).to(DEV)
-    assert not moe.fuse_swiglu  # the fused epilogue has no bias term
+    assert moe.fuse_swiglu == (act_name == "swiglu")  # the fused epilogue adds the bias before the activation
     with torch.no_grad():  # reset_parameters zeroes the biases (fma/modules/moe/__init__.py:121-122)
         moe.c_fc.bias.normal_(0, 0.5)
         moe.c_proj.bias.normal_(0, 0.5)

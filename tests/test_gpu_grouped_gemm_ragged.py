@@ -18,13 +18,13 @@ def _u32(values):
     return torch.tensor(values, dtype=torch.int64).to(torch.uint32).to(DEV)
 
 
-def _ragged(A, B, sizes, vary_k, M, N, K, tA, tB, out_elems, alpha=1.0):
+def _ragged(A, B, sizes, vary_k, M, N, K, tA, tB, out_elems, alpha=1.0, bias=None):
     lib = _lib.load()
     out = torch.full((max(out_elems, 1),), 7.0, dtype=A.dtype, device=DEV)
     s = _u32(sizes)
     rc = lib.fma_grouped_gemm_ragged(
-        A.data_ptr(), B.data_ptr(), out.data_ptr(), s.data_ptr(), len(sizes), _lib.FMA_VARY_K if vary_k else _lib.FMA_VARY_M,
-        M, N, K, int(tA), int(tB), alpha, _lib.dtype_code(A.dtype), torch.cuda.current_stream().cuda_stream,
+        A.data_ptr(), B.data_ptr(), out.data_ptr(), s.data_ptr(), _lib.ptr(bias), len(sizes),
+        _lib.FMA_VARY_K if vary_k else _lib.FMA_VARY_M, M, N, K, int(tA), int(tB), alpha, _lib.dtype_code(A.dtype), torch.cuda.current_stream().cuda_stream,
     )
     assert rc == 0, lib.fma_last_error_string()
     torch.cuda.synchronize()
@@ -120,9 +120,9 @@ def test_argument_validation():
     lib = _lib.load()
     p = torch.zeros(64, dtype=torch.bfloat16, device=DEV).data_ptr()
     s = _u32([8]).data_ptr()
-    assert lib.fma_grouped_gemm_ragged(p, p, p, s, 1, 2, 8, 8, 8, 0, 1, 1.0, _lib.FMA_BF16, None) == -3  # vary
-    assert lib.fma_grouped_gemm_ragged(p, p, p, s, 1, 0, 8, 8, 8, 0, 1, 1.0, _lib.FMA_F32, None) != 0  # fp32: other entry
-    assert lib.fma_grouped_gemm_ragged(p, p, p, s, 1025, 0, 8, 8, 8, 0, 1, 1.0, _lib.FMA_BF16, None) == -4
-    assert lib.fma_grouped_gemm_ragged(p, p, None, s, 1, 0, 8, 8, 8, 0, 1, 1.0, _lib.FMA_BF16, None) == -1
-    assert lib.fma_grouped_gemm_ragged(p, p + 2, p, s, 1, 0, 8, 8, 8, 0, 1, 1.0, _lib.FMA_BF16, None) == -6
-    assert lib.fma_grouped_gemm_ragged(p, p, p, s, 0, 0, 8, 8, 8, 0, 1, 1.0, _lib.FMA_BF16, None) == 0  # no groups
+    assert lib.fma_grouped_gemm_ragged(p, p, p, s, None, 1, 2, 8, 8, 8, 0, 1, 1.0, _lib.FMA_BF16, None) == -3  # vary
+    assert lib.fma_grouped_gemm_ragged(p, p, p, s, None, 1, 0, 8, 8, 8, 0, 1, 1.0, _lib.FMA_F32, None) != 0  # fp32: other entry
+    assert lib.fma_grouped_gemm_ragged(p, p, p, s, None, 1025, 0, 8, 8, 8, 0, 1, 1.0, _lib.FMA_BF16, None) == -4
+    assert lib.fma_grouped_gemm_ragged(p, p, None, s, None, 1, 0, 8, 8, 8, 0, 1, 1.0, _lib.FMA_BF16, None) == -1
+    assert lib.fma_grouped_gemm_ragged(p, p + 2, p, s, None, 1, 0, 8, 8, 8, 0, 1, 1.0, _lib.FMA_BF16, None) == -6
+    assert lib.fma_grouped_gemm_ragged(p, p, p, s, None, 0, 0, 8, 8, 8, 0, 1, 1.0, _lib.FMA_BF16, None) == 0  # no groups

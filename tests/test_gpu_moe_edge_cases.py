@@ -129,9 +129,9 @@ def test_evaluation_with_trainable_weights_does_not_store_the_preactivation(mode
     seen = []
     real = ci.grouped_gemm_swiglu_cuda
 
-    def spy(x_, weight, M_array, h, act):
+    def spy(x_, weight, M_array, h, act, bias=None):
         seen.append(h is not None)
-        return real(x_, weight, M_array, h, act)
+        return real(x_, weight, M_array, h, act, bias)
 
     monkeypatch.setattr(ci, "grouped_gemm_swiglu_cuda", spy)
     y_train, _ = moe(x.clone().requires_grad_(), kernel_backend=KernelBackend.cuda)

@@ -137,9 +137,9 @@ def test_router_and_bias_host_logic():
     assert logits.shape == (5, 8) and weights.shape == selected.shape == (5, 2) and selected.dtype == torch.int64
     assert torch.allclose(weights.sum(-1), torch.ones(5), atol=1e-6)
     assert bool((logits.gather(1, selected)[:, 0] >= logits.gather(1, selected)[:, 1]).all())
-    # a layer with biases keeps them as parameters of the reference's shapes and runs the up-projection unfused
+    # a layer with biases keeps them as parameters of the reference's shapes (the fused up-projection adds its own)
     biased = MoE(8, 2, 64, 128, swiglu_packed, True, True, 0.02)
-    assert biased.c_fc.bias.shape == (8, 256) and biased.c_proj.bias.shape == (8, 64) and not biased.fuse_swiglu
+    assert biased.c_fc.bias.shape == (8, 256) and biased.c_proj.bias.shape == (8, 64) and biased.fuse_swiglu
     assert float(biased.c_fc.bias.abs().max()) == 0.0  # reset_parameters zeroes them (fma/modules/moe/__init__.py:121-122)
     top1 = MoE(4, 1, 64, 128, swiglu_packed, True, False, 0.02)
     _, w1, s1 = top1._compute_routing_weights(torch.randn(5, 64))
