@@ -345,12 +345,14 @@ def measure_workload(name, args, full):
         rw = torch.empty(T, k, **bf)
         sel32 = torch.empty(T, k, dtype=torch.int32, device=dev)
         cnt = torch.empty(E, dtype=torch.uint32, device=dev)
-        # as the MoE module calls it: without the optional histogram (which costs one more small launch)
-        hbm("router_topk", T * H * s + E * H * s + T * E * s + T * k * (s + 4),
+        tbh = torch.empty((T + 15) // 16, E, dtype=torch.uint32, device=dev)
+        # as the MoE module calls it: with the histogram per block of 16 tokens that the index build starts from
+        hbm("router_topk", T * H * s + E * H * s + T * E * s + T * k * (s + 4) + tbh.numel() * 4,
             lambda i: ok(lib.fma_router_topk(xs3[i % 3].data_ptr(), wg.data_ptr(), T, H, E, k, lg.data_ptr(),
-                                             rw.data_ptr(), sel32.data_ptr(), None, BF16, stream)))
+                                             rw.data_ptr(), sel32.data_ptr(), None, tbh.data_ptr(), BF16, stream)))
+        assert int(tbh.view(torch.int32).sum()) == T * k, "router block histogram does not sum to T * top_k"
         ok(lib.fma_router_topk(x.data_ptr(), wg.data_ptr(), T, H, E, k, lg.data_ptr(), rw.data_ptr(),
-                               sel32.data_ptr(), cnt.data_ptr(), BF16, stream))
+                               sel32.data_ptr(), cnt.data_ptr(), None, BF16, stream))
         assert int(cnt.view(torch.int32).sum()) == T * k, "router histogram does not sum to T * top_k"
 
         def aten_router(i):  # the same results from library calls: gate linear, top-k, fp32 softmax, cast
@@ -417,6 +419,22 @@ def measure_workload(name, args, full):
                                                           inv.data_ptr(), ws_idx.data_ptr(), ws_idx.numel() * 4, stream)),
                      20, blocker=blocker)
         kernels["build_routing_index(3 launches)"] = {"ms": t[0], "ms_mean": t[1]}
+        # as the layer runs it behind the fused router: int32 choices and their histogram per block of 16 tokens (here
+        # made with torch; the call overwrites it, so every launch gets a copy of its own)
+        ids32 = selected_d.reshape(-1).to(torch.int32)
+        key = (torch.arange(R, device=dev) // (16 * k)) * E + ids32
+        hist0 = torch.bincount(key, minlength=((T + 15) // 16) * E).to(torch.int32)
+        n_idx = 20
+        hists = [hist0.clone() for _ in range(n_idx + 3)]
+        calls = iter(range(n_idx + 3))
+        want_perm = perm.clone()
+        t = time_gpu(lambda i: ok(lib.fma_moe_build_index_from_hist(ids32.data_ptr(), R, E, k, hists[next(calls)].data_ptr(),
+                                                                    counts.data_ptr(), offsets.data_ptr(), perm.data_ptr(),
+                                                                    eid.data_ptr(), inv.data_ptr(), stream)),
+                     n_idx, blocker=blocker)
+        assert torch.equal(perm, want_perm), "index build from the router's histogram differs"
+        kernels["build_routing_index_from_router_histogram(2 launches)"] = {"ms": t[0], "ms_mean": t[1]}
+        del hists
 
     # continuous_count on 16 Mi int32 ids in [0, 64): five distinct 64 MiB buffers (320 MiB > the 256 MiB
     # last-level cache) so that every launch reads from HBM. The figure covers both launches of one call

@@ -231,8 +231,10 @@ __global__ __launch_bounds__(kIdxThreads) void index_hist_kernel(const id_t* __r
     }
 }
 
-// counts, inclusive offsets, and hist[c][e] <- first output position of chunk c's slots of expert e
-__global__ __launch_bounds__(kScanThreads) void index_scan_kernel(uint32_t E, uint32_t nchunks, uint32_t* hist,
+// counts, inclusive offsets, and hist[c * rows][e] <- first output position of chunk c's slots of expert e.
+// A chunk's histogram is the sum of `rows` consecutive rows of hist (the last chunk may have fewer: nrows in all).
+__global__ __launch_bounds__(kScanThreads) void index_scan_kernel(uint32_t E, uint32_t nchunks, uint32_t rows,
+                                                                  uint32_t nrows, uint32_t* hist,
                                                                   uint32_t* __restrict__ counts,
                                                                   uint32_t* __restrict__ offsets) {
     __shared__ uint32_t s_seg[kScanThreads];  // [part][e]
@@ -251,7 +253,10 @@ __global__ __launch_bounds__(kScanThreads) void index_scan_kernel(uint32_t E, ui
 
     uint32_t s = 0;
     if (active) {
-        for (uint32_t c = c_lo; c < c_hi; ++c) s += hist[(uint64_t)c * E + e];
+        const uint32_t r_lo = c_lo * rows;
+        uint32_t r_hi = c_hi * rows;
+        if (r_hi > nrows) r_hi = nrows;
+        for (uint32_t r = r_lo; r < r_hi; ++r) s += hist[(uint64_t)r * E + e];
         s_seg[part * E + e] = s;
     }
     __syncthreads();
@@ -287,9 +292,12 @@ __global__ __launch_bounds__(kScanThreads) void index_scan_kernel(uint32_t E, ui
     if (active) {
         uint32_t running = s_start[e] + s_seg[part * E + e];
         for (uint32_t c = c_lo; c < c_hi; ++c) {
-            const uint64_t i = (uint64_t)c * E + e;
-            const uint32_t v = hist[i];
-            hist[i] = running;
+            const uint32_t r0 = c * rows;
+            uint32_t r1 = r0 + rows;
+            if (r1 > nrows) r1 = nrows;
+            uint32_t v = 0;
+            for (uint32_t r = r0; r < r1; ++r) v += hist[(uint64_t)r * E + e];
+            hist[(uint64_t)r0 * E + e] = running;
             running += v;
         }
     }
@@ -297,9 +305,11 @@ __global__ __launch_bounds__(kScanThreads) void index_scan_kernel(uint32_t E, ui
 
 // One wavefront per chunk walks its slots in order; lanes with the same expert id find each other with
 // ballots, the lowest of them advances the expert's cursor, each takes cursor + its rank in the group.
-template <typename id_t>
+// A chunk is chunk_slots <= STEPS * 64 consecutive slots; its cursors start at base[c * base_stride + e].
+template <typename id_t, int STEPS>
 __global__ __launch_bounds__(kIdxThreads) void index_place_kernel(const id_t* __restrict__ ids, int64_t R, uint32_t E,
-                                                                  uint32_t nbits, uint32_t nchunks,
+                                                                  uint32_t nbits, uint32_t nchunks, uint32_t chunk_slots,
+                                                                  uint64_t base_stride,
                                                                   const uint32_t* __restrict__ base,
                                                                   int32_t* __restrict__ perm, int32_t* __restrict__ eid,
                                                                   int32_t* __restrict__ inv) {
@@ -310,19 +320,21 @@ __global__ __launch_bounds__(kIdxThreads) void index_place_kernel(const id_t* __
     const uint32_t c = blockIdx.x * kIdxWaves + wave;
     const bool live = c < nchunks;
     if (live) {
-        for (uint32_t e = lane; e < E; e += kWave) cur[e] = base[(uint64_t)c * E + e];
+        for (uint32_t e = lane; e < E; e += kWave) cur[e] = base[(uint64_t)c * base_stride + e];
     }
     __syncthreads();
     if (!live) return;
 
-    const int64_t first = (int64_t)c * kIdxChunk;
-    int32_t id[kIdxSteps];
+    const int64_t first = (int64_t)c * chunk_slots;
+    const int64_t end = first + chunk_slots < R ? first + chunk_slots : R;  // slots past the chunk read as "no id"
+    int32_t id[STEPS];
 #pragma unroll
-    for (int s = 0; s < kIdxSteps; ++s) id[s] = load_id<id_t>(ids, first + s * kWave + lane, R, E);
+    for (int s = 0; s < STEPS; ++s) id[s] = load_id<id_t>(ids, first + s * kWave + lane, end, E);
 
     const uint64_t below = (1ull << lane) - 1ull;
 #pragma unroll
-    for (int s = 0; s < kIdxSteps; ++s) {
+    for (int s = 0; s < STEPS; ++s) {
+        if (s * kWave >= (int)chunk_slots) break;
         const bool valid = id[s] >= 0;
         uint64_t mask = __ballot(valid);
         for (uint32_t b = 0; b < nbits; ++b) {
@@ -379,20 +391,50 @@ int launch_build_index(const void* ids, int id_bytes, int64_t R, int64_t E, uint
         int rc = launch_status("moe_build_index(hist)");
         if (rc) return rc;
     }
-    hipLaunchKernelGGL(index_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, (uint32_t)E, nchunks, hist, counts,
-                       offsets);
+    hipLaunchKernelGGL(index_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, (uint32_t)E, nchunks, 1u, nchunks, hist,
+                       counts, offsets);
     int rc = launch_status("moe_build_index(scan)");
     if (rc) return rc;
     if (nchunks > 0) {
         if (id_bytes == 4)
-            hipLaunchKernelGGL(index_place_kernel<int32_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
-                               (const int32_t*)ids, R, (uint32_t)E, nbits, nchunks, hist, perm, eid, inv);
+            hipLaunchKernelGGL((index_place_kernel<int32_t, kIdxSteps>), dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
+                               (const int32_t*)ids, R, (uint32_t)E, nbits, nchunks, (uint32_t)kIdxChunk, (uint64_t)E,
+                               hist, perm, eid, inv);
         else
-            hipLaunchKernelGGL(index_place_kernel<int64_t>, dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
-                               (const int64_t*)ids, R, (uint32_t)E, nbits, nchunks, hist, perm, eid, inv);
+            hipLaunchKernelGGL((index_place_kernel<int64_t, kIdxSteps>), dim3(blocks), dim3(kIdxThreads), lds_bytes, st,
+                               (const int64_t*)ids, R, (uint32_t)E, nbits, nchunks, (uint32_t)kIdxChunk, (uint64_t)E,
+                               hist, perm, eid, inv);
         rc = launch_status("moe_build_index(place)");
     }
     return rc;
+}
+
+// The same sort from histograms the caller already has: hist[r][e] = number of slots of the r-th block of
+// 16 * top_k consecutive slots (16 tokens) that go to expert e. Two launches: scan and placement. A chunk of the
+// placement is `rows` consecutive blocks, about 512 slots.
+int launch_build_index_from_hist(const int32_t* ids, int64_t R, int64_t E, int64_t top_k, uint32_t* counts,
+                                 uint32_t* offsets, int32_t* perm, int32_t* eid, int32_t* inv, uint32_t* hist,
+                                 hipStream_t st) {
+    const int64_t block_slots = 16 * top_k;
+    const uint32_t nrows = (uint32_t)((R + block_slots - 1) / block_slots);
+    const uint32_t rows = (uint32_t)(block_slots >= kIdxChunk ? 1 : kIdxChunk / block_slots);
+    const uint32_t chunk_slots = (uint32_t)(rows * block_slots);  // <= 1024 (top_k <= 64)
+    const uint32_t nchunks = (nrows + rows - 1) / rows;
+    const uint32_t blocks = (nchunks + kIdxWaves - 1) / kIdxWaves;
+    const size_t lds_bytes = (size_t)kIdxWaves * E * 4;
+    uint32_t nbits = 0;
+    while ((1ll << nbits) < E) ++nbits;
+    hipLaunchKernelGGL(index_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, (uint32_t)E, nchunks, rows, nrows, hist,
+                       counts, offsets);
+    int rc = launch_status("moe_build_index_from_hist(scan)");
+    if (rc || nchunks == 0) return rc;
+    if (chunk_slots <= kIdxSteps * kWave)
+        hipLaunchKernelGGL((index_place_kernel<int32_t, kIdxSteps>), dim3(blocks), dim3(kIdxThreads), lds_bytes, st, ids, R,
+                           (uint32_t)E, nbits, nchunks, chunk_slots, (uint64_t)rows * (uint64_t)E, hist, perm, eid, inv);
+    else
+        hipLaunchKernelGGL((index_place_kernel<int32_t, 2 * kIdxSteps>), dim3(blocks), dim3(kIdxThreads), lds_bytes, st, ids,
+                           R, (uint32_t)E, nbits, nchunks, chunk_slots, (uint64_t)rows * (uint64_t)E, hist, perm, eid, inv);
+    return launch_status("moe_build_index_from_hist(place)");
 }
 
 // Address of `scratch` on the current device, looked up once per device (each GPU holds its own copy of the array at
@@ -494,6 +536,20 @@ int fma_moe_build_index(const void* ids, int id_bytes, int64_t R, int64_t E, uin
                 (long long)need);
     return launch_build_index(ids, id_bytes, R, E, counts, offsets, perm, eid, inv, (uint32_t*)workspace,
                               (hipStream_t)stream);
+}
+
+int fma_moe_build_index_from_hist(const int32_t* ids, int64_t R, int64_t E, int64_t top_k, uint32_t* token_block_hist,
+                                  uint32_t* counts, uint32_t* offsets, int32_t* perm, int32_t* eid, int32_t* inv,
+                                  void* stream) {
+    using namespace fmahip;
+    int rc = check_build_index(ids, 4, R, E, counts, offsets, perm, eid, inv);
+    if (rc) return rc;
+    FMA_REQUIRE(top_k >= 1 && top_k <= 64 && R % top_k == 0, FMA_ERR_BAD_SIZE,
+                "moe_build_index_from_hist: top_k must lie in [1, 64] and divide R (top_k=%lld, R=%lld)",
+                (long long)top_k, (long long)R);
+    FMA_REQUIRE(R == 0 || token_block_hist, FMA_ERR_NULL_POINTER, "moe_build_index_from_hist: the histogram is NULL");
+    return launch_build_index_from_hist(ids, R, E, top_k, counts, offsets, perm, eid, inv, token_block_hist,
+                                        (hipStream_t)stream);
 }
 
 int64_t fma_moe_build_index_static_max_words(void) { return FMA_STATIC_INDEX_WORDS; }

@@ -55,6 +55,7 @@ struct RouterArgs {
     uint16_t* weights;       // [T, k]
     int32_t* selected;       // [T, k]
     uint32_t* counts;        // [E] or null
+    uint32_t* hist;          // [ceil(T / 16), E] or null: choices per expert among each 16 consecutive tokens
     int64_t T;
     int32_t H, E, k;
 };
@@ -121,7 +122,7 @@ __global__ __launch_bounds__(kRouterThreads) void fill_u32_kernel(uint32_t* p, i
 // j % 16, so that after the k rounds every lane turns its own choices into weights and writes them.
 template <typename EL, int NR>
 __device__ __forceinline__ void topk_softmax_tokens(uint32_t* const (&keys)[NR], int c, const int64_t (&token)[NR],
-                                                    const RouterArgs& a, uint32_t* s_hist) {
+                                                    const int64_t tok0, const RouterArgs& a, uint32_t* s_hist) {
     const int E = a.E, k = a.k;
     uint32_t mine[NR][kMaxTopK / 16];
     uint32_t first[NR];
@@ -169,19 +170,35 @@ __device__ __forceinline__ void topk_softmax_tokens(uint32_t* const (&keys)[NR],
                     const int col = key_column(mine[t][i]);
                     a.selected[token[t] * k + j] = col;
                     a.weights[token[t] * k + j] = EL::bits(e[i] / sum);
-                    if (a.counts) atomicAdd(&s_hist[col], 1u);
+                    if (a.counts || a.hist) atomicAdd(&s_hist[(int)((token[t] - tok0) >> 4) * E + col], 1u);
                 }
             }
         }
     }
 }
 
-__device__ __forceinline__ void flush_histogram(const RouterArgs& a, const uint32_t* s_hist, int tid, int nthreads) {
-    if (!a.counts) return;
+// s_hist: [groups][E], one row per 16 consecutive tokens of the workgroup (its first token tok0 is a multiple of 16)
+__device__ __forceinline__ void clear_histogram(const RouterArgs& a, uint32_t* s_hist, int groups, int tid, int nthreads) {
+    if (a.counts || a.hist)
+        for (int n = tid; n < groups * a.E; n += nthreads) s_hist[n] = 0;
+}
+__device__ __forceinline__ void flush_histogram(const RouterArgs& a, const uint32_t* s_hist, int groups, int64_t tok0,
+                                                int tid, int nthreads) {
+    if (!a.counts && !a.hist) return;
     __syncthreads();
-    for (int n = tid; n < a.E; n += nthreads) {
-        const uint32_t h = s_hist[n];
-        if (h) atomicAdd(a.counts + n, h);
+    if (a.hist) {
+        // every row of 16 tokens belongs to one workgroup: plain stores, nothing to clear beforehand
+        const int64_t row0 = tok0 >> 4, nrows = (a.T + 15) >> 4;
+        for (int g = 0; g < groups; ++g)
+            if (row0 + g < nrows)
+                for (int n = tid; n < a.E; n += nthreads) a.hist[(row0 + g) * a.E + n] = s_hist[g * a.E + n];
+    }
+    if (a.counts) {
+        for (int n = tid; n < a.E; n += nthreads) {
+            uint32_t h = 0;
+            for (int g = 0; g < groups; ++g) h += s_hist[g * a.E + n];
+            if (h) atomicAdd(a.counts + n, h);
+        }
     }
 }
 
@@ -193,15 +210,14 @@ __global__ __launch_bounds__(kRouterThreads) void router_topk_kernel(const Route
     constexpr int kCols = NBLK * 16, kToks = RB * kTok;
     __shared__ float s_part[kRouterWaves][kToks][kCols];
     __shared__ uint32_t s_key[kToks][EMAX + kRowPad];
-    __shared__ uint32_t s_hist[EMAX];
+    __shared__ uint32_t s_hist[RB * EMAX];
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
     const int H = a.H, E = a.E;
     const int64_t tok0 = (int64_t)blockIdx.x * kToks;
 
-    if (a.counts)
-        for (int n = tid; n < E; n += kRouterThreads) s_hist[n] = 0;
+    clear_histogram(a, s_hist, RB, tid, kRouterThreads);
 
     // ---- logits: 16 RB tokens x E, this wavefront's share of the reduction dimension -------------------------------
     const uint16_t* xa[RB];
@@ -321,9 +337,9 @@ __global__ __launch_bounds__(kRouterThreads) void router_topk_kernel(const Route
             rows[rb] = s_key[rb * kTok + (tid >> 4)];
             tokens[rb] = tok0 + rb * kTok + (tid >> 4);
         }
-        topk_softmax_tokens<EL, RB>(rows, tid & 15, tokens, a, s_hist);
+        topk_softmax_tokens<EL, RB>(rows, tid & 15, tokens, tok0, a, s_hist);
     }
-    flush_histogram(a, s_hist, tid, kRouterThreads);
+    flush_histogram(a, s_hist, RB, tok0, tid, kRouterThreads);
 }
 
 // ---- the same for more than 16 experts -------------------------------------------------------------------------------
@@ -346,15 +362,14 @@ __global__ __launch_bounds__(W * kWave) void router_topk_wide_kernel(const Route
     constexpr int kCols = NBLK * 16, kToks = W * kTok;
     __shared__ __attribute__((aligned(16))) uint8_t s_tile[2][kCols * kTileRowBytes];
     __shared__ uint32_t s_key[kToks][EMAX + kRowPad];
-    __shared__ uint32_t s_hist[EMAX];
+    __shared__ uint32_t s_hist[W * EMAX];
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
     const int H = a.H, E = a.E;
     const int64_t tok0 = (int64_t)blockIdx.x * kToks;
 
-    if (a.counts)
-        for (int n = tid; n < E; n += kThreadsW) s_hist[n] = 0;
+    clear_histogram(a, s_hist, W, tid, kThreadsW);
 
     const int64_t t_mine = tok0 + wave * kTok + r;
     const uint16_t* xa = a.x + (t_mine < a.T ? t_mine : a.T - 1) * H + q * 32;  // past the end: the last token again
@@ -491,9 +506,9 @@ __global__ __launch_bounds__(W * kWave) void router_topk_wide_kernel(const Route
             rows[round] = s_key[round * (W * 4) + (tid >> 4)];
             tokens[round] = tok0 + round * (W * 4) + (tid >> 4);
         }
-        topk_softmax_tokens<EL, 4>(rows, tid & 15, tokens, a, s_hist);
+        topk_softmax_tokens<EL, 4>(rows, tid & 15, tokens, tok0, a, s_hist);
     }
-    flush_histogram(a, s_hist, tid, kThreadsW);
+    flush_histogram(a, s_hist, W, tok0, tid, kThreadsW);
 }
 
 template <typename EL, int NBLK, int EMAX>
@@ -646,7 +661,8 @@ int check_router(const char* what, int dtype, int64_t T, int64_t E, int64_t k) {
 extern "C" {
 
 int fma_router_topk(const void* x, const void* gate_weight, int64_t T, int64_t H, int64_t E, int64_t top_k,
-                    void* logits, void* weights, int32_t* selected, uint32_t* counts, int dtype, void* stream) {
+                    void* logits, void* weights, int32_t* selected, uint32_t* counts, uint32_t* token_block_hist,
+                    int dtype, void* stream) {
     using namespace fmahip;
     static_assert(kMaxTopK == FMA_MAX_ROUTER_TOP_K, "header and kernel disagree on the top_k limit");
     int rc = check_router("router_topk", dtype, T, E, top_k);
@@ -671,6 +687,7 @@ int fma_router_topk(const void* x, const void* gate_weight, int64_t T, int64_t H
     a.weights = (uint16_t*)weights;
     a.selected = selected;
     a.counts = counts;
+    a.hist = token_block_hist;
     a.T = T;
     a.H = (int32_t)H;
     a.E = (int32_t)E;

@@ -50,7 +50,8 @@ SIGNATURES = {
     "fma_expert_bias_add": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "fma_expert_bias_grad_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "fma_expert_bias_grad": (_i32, [_p, _p, _i64, _i64, _i64, _p, _p, _i64, _i32, _p]),
-    "fma_router_topk": (_i32, [_p, _p, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _i32, _p]),
+    "fma_router_topk": (_i32, [_p, _p, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p, _i32, _p]),
+    "fma_moe_build_index_from_hist": (_i32, [_p, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _p]),
     "fma_router_topk_bwd": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _p, _i32, _p]),
     "fma_fused_residual_add_rmsnorm_fwd": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _i64, _f32, _f32, _i32, _p]),
     "fma_fused_residual_add_rmsnorm_bwd_workspace_bytes": (_i64, [_i64, _i64]),

@@ -18,6 +18,7 @@ from .cuda_implementation import (
     build_routing_index,
     combine,
     fused_router,
+    fused_router_with_histogram,
     gather_rows,
     grouped_gemm_experts,
     up_projection_swiglu_experts,
@@ -132,11 +133,22 @@ class MoE(nn.Module):
 
         # hidden_states -> (total_q, hidden_size)
         hidden_states = hidden_states.view(-1, self.hidden_size)
-        router_logits, router_weights, selected_experts = self._compute_routing_weights(hidden_states)
+        token_block_histogram = None
+        if self._router_is_fusable(hidden_states):
+            # the router kernel counts its choices as it makes them; the index build starts from those counts
+            router_logits, router_weights, selected_experts, token_block_histogram = fused_router_with_histogram(
+                hidden_states, self.gate.weight, self.top_k
+            )
+        else:
+            router_logits, router_weights, selected_experts = self._compute_routing_weights(hidden_states)
 
         # router_logits -> (total_q, num_experts); router_weights, selected_experts -> (total_q, top_k)
         hidden_states = self._compute_experts(
-            hidden_states, router_weights, selected_experts, kernel_backend=kernel_backend
+            hidden_states,
+            router_weights,
+            selected_experts,
+            kernel_backend=kernel_backend,
+            token_block_histogram=token_block_histogram,
         )
 
         hidden_states = hidden_states.view(original_shape)
@@ -180,12 +192,15 @@ class MoE(nn.Module):
         router_weights: torch.Tensor,
         selected_experts: torch.Tensor,
         kernel_backend: KernelBackend,
+        token_block_histogram: torch.Tensor | None = None,
     ) -> torch.Tensor:
         if not is_hip_kernel_backend(kernel_backend):
             raise ValueError(f"unexpected kernel_backend ({kernel_backend})")
 
         # counts, offsets and the stable expert-major order of the (token, choice) slots, with its inverse
-        expert_frequency, _, sorted_scattered_idxs, _, inverse = build_routing_index(selected_experts, self.num_experts)
+        expert_frequency, _, sorted_scattered_idxs, _, inverse = build_routing_index(
+            selected_experts, self.num_experts, token_block_histogram
+        )
 
         # rows of every expert back to back: x[slot // top_k]
         hidden_states = gather_rows(hidden_states, sorted_scattered_idxs, inverse, self.top_k)

@@ -49,6 +49,38 @@ def moe_build_index_cuda(
     _lib.check(rc, "moe_build_index_cuda")
 
 
+@custom_op(
+    f"{LIBRARY_NAME}::moe_build_index_from_hist_cuda",
+    mutates_args={"token_block_hist", "counts", "offsets", "perm", "eid", "inv"},
+)
+def moe_build_index_from_hist_cuda(
+    ids: torch.Tensor,
+    top_k: int,
+    token_block_hist: torch.Tensor,
+    counts: torch.Tensor,
+    offsets: torch.Tensor,
+    perm: torch.Tensor,
+    eid: torch.Tensor,
+    inv: torch.Tensor,
+) -> None:
+    """moe_build_index_cuda for choices the fused router has already counted per block of 16 tokens: scan and
+    placement only. The histogram serves as scratch memory and is overwritten."""
+    _lib.require_gpu(ids, token_block_hist, counts, offsets, perm, eid, inv)
+    assert ids.dtype == torch.int32 and ids.is_contiguous()
+    assert counts.dtype == torch.uint32 and offsets.dtype == torch.uint32
+    assert perm.dtype == eid.dtype == inv.dtype == torch.int32
+    R, E = ids.numel(), counts.numel()
+    assert perm.numel() == eid.numel() == inv.numel() == R and offsets.numel() == E and R % top_k == 0
+    assert token_block_hist.dtype == torch.uint32 and token_block_hist.is_contiguous()
+    assert token_block_hist.shape == ((R // top_k + 15) // 16, E)
+    with torch.cuda.device(ids.device):
+        rc = _lib.load().fma_moe_build_index_from_hist(
+            ids.data_ptr(), R, E, top_k, _lib.ptr(token_block_hist), counts.data_ptr(), offsets.data_ptr(),
+            perm.data_ptr(), eid.data_ptr(), inv.data_ptr(), _lib.current_stream(ids.device),
+        )
+    _lib.check(rc, "moe_build_index_from_hist_cuda")
+
+
 @custom_op(f"{LIBRARY_NAME}::gather_rows_cuda", mutates_args={"output"})
 def gather_rows_cuda(x: torch.Tensor, idx: torch.Tensor, divisor: int, output: torch.Tensor) -> None:
     _lib.require_gpu(x, idx, output)
@@ -231,7 +263,9 @@ def expert_bias_grad_cuda(output_grad: torch.Tensor, M_array: torch.Tensor, bias
     _lib.check(rc, "expert_bias_grad_cuda")
 
 
-@custom_op(f"{LIBRARY_NAME}::router_topk_cuda", mutates_args={"logits", "weights", "selected", "counts"})
+@custom_op(
+    f"{LIBRARY_NAME}::router_topk_cuda", mutates_args={"logits", "weights", "selected", "counts", "token_block_hist"}
+)
 def router_topk_cuda(
     x: torch.Tensor,
     gate_weight: torch.Tensor,
@@ -240,20 +274,25 @@ def router_topk_cuda(
     weights: torch.Tensor,
     selected: torch.Tensor,
     counts: torch.Tensor | None,
+    token_block_hist: torch.Tensor | None,
 ) -> None:
-    _lib.require_gpu(x, gate_weight, logits, weights, selected, counts)
+    _lib.require_gpu(x, gate_weight, logits, weights, selected, counts, token_block_hist)
     T, H = x.shape
     E = gate_weight.size(0)
     assert gate_weight.shape == (E, H) and logits.shape == (T, E)
     assert weights.shape == (T, top_k) and selected.shape == (T, top_k)
     assert x.dtype == gate_weight.dtype == logits.dtype == weights.dtype and selected.dtype == torch.int32
     assert counts is None or (counts.dtype == torch.uint32 and counts.numel() == E)
-    for t in (x, gate_weight, logits, weights, selected, counts):
+    assert token_block_hist is None or (
+        token_block_hist.dtype == torch.uint32 and token_block_hist.shape == ((T + 15) // 16, E)
+    )
+    for t in (x, gate_weight, logits, weights, selected, counts, token_block_hist):
         assert t is None or t.is_contiguous()
     with torch.cuda.device(x.device):
         rc = _lib.load().fma_router_topk(
             x.data_ptr(), gate_weight.data_ptr(), T, H, E, top_k, logits.data_ptr(), weights.data_ptr(),
-            selected.data_ptr(), _lib.ptr(counts), _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
+            selected.data_ptr(), _lib.ptr(counts), _lib.ptr(token_block_hist), _lib.dtype_code(x.dtype),
+            _lib.current_stream(x.device),
         )
     _lib.check(rc, "router_topk_cuda")
 
@@ -288,9 +327,12 @@ def router_topk_backward_cuda(
 
 @torch.no_grad()
 def build_routing_index(
-    selected_experts: torch.Tensor, num_experts: int
+    selected_experts: torch.Tensor, num_experts: int, token_block_histogram: torch.Tensor | None = None
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """Stable counting sort of the flattened (token, choice) slots by expert.
+
+    token_block_histogram: what the fused router counted while choosing (per block of 16 tokens); with it the sort is a
+    scan and a placement pass, without it the choices are counted first. It is overwritten.
 
     Returns (expert_frequency uint32[E], expert_offsets uint32[E] (inclusive), sorted_scattered_idxs int32[R],
     sorted_expert_idxs int32[R], inverse int32[R]); the first four are what the reference obtains from
@@ -305,7 +347,12 @@ def build_routing_index(
     perm = torch.empty(R, dtype=torch.int32, device=device)
     eid = torch.empty(R, dtype=torch.int32, device=device)
     inv = torch.empty(R, dtype=torch.int32, device=device)
-    moe_build_index_cuda(ids, counts, offsets, perm, eid, inv)
+    if token_block_histogram is not None and ids.dtype == torch.int32 and selected_experts.dim() == 2:
+        moe_build_index_from_hist_cuda(
+            ids, selected_experts.size(1), token_block_histogram, counts, offsets, perm, eid, inv
+        )
+    else:
+        moe_build_index_cuda(ids, counts, offsets, perm, eid, inv)
     return counts, offsets, perm, eid, inv
 
 
@@ -325,15 +372,17 @@ class _FusedRouter(torch.autograd.Function):
         logits = torch.empty(T, E, device=x.device, dtype=x.dtype)
         weights = torch.empty(T, top_k, device=x.device, dtype=x.dtype)
         selected = torch.empty(T, top_k, device=x.device, dtype=torch.int32)
-        router_topk_cuda(x, gate_weight, top_k, logits, weights, selected, None)
+        # the choices counted per block of 16 tokens, for the index build that follows
+        token_block_hist = torch.empty((T + 15) // 16, E, device=x.device, dtype=torch.uint32)
+        router_topk_cuda(x, gate_weight, top_k, logits, weights, selected, None, token_block_hist)
         ctx.save_for_backward(x, gate_weight, logits, selected)
-        ctx.mark_non_differentiable(selected)
+        ctx.mark_non_differentiable(selected, token_block_hist)
         ctx.set_materialize_grads(False)
-        return logits, weights, selected
+        return logits, weights, selected, token_block_hist
 
     @staticmethod
     @ensure_contiguous
-    def backward(ctx, logits_output_grad, weights_grad, _):
+    def backward(ctx, logits_output_grad, weights_grad, _, __):
         x, gate_weight, logits, selected = ctx.saved_tensors
         if logits_output_grad is None and weights_grad is None:
             return None, None, None
@@ -345,6 +394,13 @@ class _FusedRouter(torch.autograd.Function):
 
 
 def fused_router(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int):
+    """(router_logits, router_weights, selected_experts)"""
+    return _FusedRouter.apply(x, gate_weight, top_k)[:3]
+
+
+def fused_router_with_histogram(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int):
+    """fused_router plus the uint32 [ceil(T / 16), E] histogram of the choices per block of 16 tokens, which
+    build_routing_index takes (and overwrites)"""
     return _FusedRouter.apply(x, gate_weight, top_k)
 
 

@@ -94,6 +94,16 @@ int fma_moe_build_index(const void* ids, int id_bytes, int64_t R, int64_t E, uin
                         uint32_t* offsets, int32_t* perm, int32_t* eid, int32_t* inv, void* workspace,
                         int64_t workspace_bytes, void* stream);
 
+/* fma_moe_build_index for ids that come from fma_router_topk, which has already counted them: token_block_hist
+ * ([ceil(T / 16), E] uint32, T = R / top_k) holds, per block of 16 consecutive tokens, the number of choices of every
+ * expert, as that call writes it. Two launches (prefix scan, placement) instead of three, no workspace: the histogram
+ * itself is the scratch memory and is OVERWRITTEN. ids: int32 [R], every id in [0, E); top_k <= 64 divides R. Same
+ * outputs, bit for bit, as fma_moe_build_index. Replaces the same reference lines, for the case that the choice and
+ * its histogram come out of one kernel (fma/modules/moe/__init__.py:191-217). */
+int fma_moe_build_index_from_hist(const int32_t* ids, int64_t R, int64_t E, int64_t top_k, uint32_t* token_block_hist,
+                                  uint32_t* counts, uint32_t* offsets, int32_t* perm, int32_t* eid, int32_t* inv,
+                                  void* stream);
+
 /* Words (uint32) of the built-in scratch array of fma_moe_build_index_static: it serves calls with
  * fma_moe_build_index_workspace_bytes(R, E) <= 4 * this value. */
 int64_t fma_moe_build_index_static_max_words(void);
@@ -237,6 +247,8 @@ int fma_expert_bias_grad(const void* dy, const uint32_t* M_arr, int64_t E, int64
  *                    in ascending column order; NaN ranks above every number                     (int32 [T, top_k])
  *   weights[t, :] = softmax of those top_k logits, computed in fp32, rounded to dtype           ([T, top_k])
  *   counts[e]     = #{(t, j) : selected[t, j] == e}   (uint32 [E]; fully overwritten; may be NULL)
+ *   token_block_hist[b, e] = #{(t, j) : 16 b <= t < 16 b + 16, selected[t, j] == e}
+ *                    (uint32 [ceil(T / 16), E]; fully overwritten; may be NULL): what fma_moe_build_index_from_hist takes
  * gate_weight: [E, H] row-major. dtype: FMA_BF16 or FMA_F16. H % 8 == 0, E <= FMA_MAX_GROUPS,
  * top_k <= min(E, FMA_MAX_ROUTER_TOP_K). x and gate_weight 16-byte aligned.
  * Replaces MoE._compute_routing_weights and MoE._get_topk (fma/modules/moe/__init__.py:191-204, 292-298:
@@ -244,7 +256,8 @@ int fma_expert_bias_grad(const void* dy, const uint32_t* M_arr, int64_t E, int64
  * counts it also yields what continuous_count(sorted_expert_idxs, num_experts) returns at :215-217. torch.topk
  * leaves the order of equal values open; the order here is one of the orders it may return. */
 int fma_router_topk(const void* x, const void* gate_weight, int64_t T, int64_t H, int64_t E, int64_t top_k,
-                    void* logits, void* weights, int32_t* selected, uint32_t* counts, int dtype, void* stream);
+                    void* logits, void* weights, int32_t* selected, uint32_t* counts, uint32_t* token_block_hist,
+                    int dtype, void* stream);
 
 /* Backward of the top-k + softmax part of fma_router_topk: the gradient with respect to the logits.
  *   d_out[t, :] = d_logits[t, :]                          (zeros if d_logits == NULL)

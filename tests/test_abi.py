@@ -100,14 +100,14 @@ def test_router_norm_and_bias_validation(lib):
     buf = ctypes.create_string_buffer(4096 + 16)
     p = (ctypes.addressof(buf) + 15) & ~15
     # router: T, H, E, top_k
-    assert lib.fma_router_topk(p, p, 4, 64, 8, 9, p, p, p, None, 2, None) == -3 and "top_k" in _err(lib)
-    assert lib.fma_router_topk(p, p, 4, 64, 8, 65, p, p, p, None, 2, None) == -3
-    assert lib.fma_router_topk(p, p, 4, 60, 8, 2, p, p, p, None, 2, None) == -3 and "multiple of 8" in _err(lib)
-    assert lib.fma_router_topk(p, p, 4, 64, 1025, 2, p, p, p, None, 2, None) == -4
-    assert lib.fma_router_topk(p, p, 4, 64, 8, 2, p, p, p, None, 0, None) == -2  # 16-bit dtypes only
-    assert lib.fma_router_topk(p, p, 4, 64, 8, 2, None, p, p, None, 2, None) == -1
-    assert lib.fma_router_topk(p + 2, p, 4, 64, 8, 2, p, p, p, None, 2, None) == -6
-    assert lib.fma_router_topk(p, p, 0, 64, 8, 2, p, p, p, None, 2, None) == 0
+    assert lib.fma_router_topk(p, p, 4, 64, 8, 9, p, p, p, None, None, 2, None) == -3 and "top_k" in _err(lib)
+    assert lib.fma_router_topk(p, p, 4, 64, 8, 65, p, p, p, None, None, 2, None) == -3
+    assert lib.fma_router_topk(p, p, 4, 60, 8, 2, p, p, p, None, None, 2, None) == -3 and "multiple of 8" in _err(lib)
+    assert lib.fma_router_topk(p, p, 4, 64, 1025, 2, p, p, p, None, None, 2, None) == -4
+    assert lib.fma_router_topk(p, p, 4, 64, 8, 2, p, p, p, None, None, 0, None) == -2  # 16-bit dtypes only
+    assert lib.fma_router_topk(p, p, 4, 64, 8, 2, None, p, p, None, None, 2, None) == -1
+    assert lib.fma_router_topk(p + 2, p, 4, 64, 8, 2, p, p, p, None, None, 2, None) == -6
+    assert lib.fma_router_topk(p, p, 0, 64, 8, 2, p, p, p, None, None, 2, None) == 0
     assert lib.fma_router_topk_bwd(p, p, None, None, 4, 8, 9, p, 2, None) == -3
     assert lib.fma_router_topk_bwd(p, None, None, None, 4, 8, 2, p, 2, None) == -1
     # residual add + RMSNorm: B, H

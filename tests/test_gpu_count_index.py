@@ -96,6 +96,35 @@ def test_routing_index(T, E, k, kind, empty, dtype):
         assert (to_np(counts)[-empty:] == 0).all()
 
 
+@pytest.mark.parametrize(
+    "T,E,k,kind,empty",
+    [
+        (7, 8, 2, "uniform", 0),
+        (1, 4, 4, "uniform", 0),
+        (333, 5, 3, "uniform", 0),  # 48 slots per block of 16 tokens: chunks of 10 blocks, the last one short
+        (16384, 8, 2, "uniform", 0),  # Mixtral shape
+        (16384, 64, 6, "zipf", 4),  # fine-grained: 96 slots per block, chunks of 5 blocks
+        (32768, 64, 8, "zipf", 4),
+        (8192, 128, 8, "uniform", 0),
+        (1000, 1024, 8, "zipf", 100),
+        (100, 64, 64, "uniform", 0),  # 1024 slots per block: the placement's long chunk
+        (530, 80, 40, "uniform", 0),  # 640 slots per block
+    ],
+)
+def test_routing_index_from_token_block_histogram(T, E, k, kind, empty):
+    # the two-launch build that starts from per-16-token histograms (as the router kernel writes them, here counted
+    # with numpy): the same five arrays as the oracle's, and the histogram may be consumed
+    selected, _ = make_routing(T, E, k, kind, seed=T + E, empty_tail=empty)
+    expect = c_oracle.routing_index(selected.numpy(), E)
+    hist = np.zeros(((T + 15) // 16, E), dtype=np.int32)
+    np.add.at(hist, (np.repeat(np.arange(T) // 16, k), selected.numpy().reshape(-1)), 1)
+    got = build_routing_index(
+        selected.to(torch.int32).to(DEV), E, token_block_histogram=torch.from_numpy(hist).to(DEV).view(torch.uint32)
+    )
+    for a, key in zip(got, ("counts", "offsets", "perm", "eid", "inv")):
+        assert np.array_equal(to_np(a), expect[key]), key
+
+
 def test_routing_index_fixture():
     # tests/golden/routing_index_4096.npz: 4096 skewed ids, three empty experts, answers from numpy
     import os

@@ -12,7 +12,12 @@ import torch
 import torch.nn.functional as F
 
 from fma import KernelBackend, MoE, swiglu_packed
-from fma.modules.moe.cuda_implementation import fused_router, router_topk_backward_cuda, router_topk_cuda
+from fma.modules.moe.cuda_implementation import (
+    build_routing_index,
+    fused_router,
+    router_topk_backward_cuda,
+    router_topk_cuda,
+)
 from oracle import moe_oracle as O
 
 from gpu_util import DEV, rel_err, to_np
@@ -41,15 +46,19 @@ SHAPES = [
 ]
 
 
-def _run_forward(x, w, k, with_counts=True):
+def _run_forward(x, w, k, with_counts=True, block_hist=None):
     T, E = x.size(0), w.size(0)
     logits = torch.full((T, E), float("nan"), device=DEV, dtype=x.dtype)
     weights = torch.full((T, k), float("nan"), device=DEV, dtype=x.dtype)
     selected = torch.full((T, k), -1, device=DEV, dtype=torch.int32)
     counts = torch.full((E,), 12345, device=DEV, dtype=torch.int32).view(torch.uint32) if with_counts else None
-    router_topk_cuda(x, w, k, logits, weights, selected, counts)
+    router_topk_cuda(x, w, k, logits, weights, selected, counts, block_hist)
     torch.cuda.synchronize()
     return logits, weights, selected, counts
+
+
+def _block_hist_buffer(T, E):
+    return torch.full(((T + 15) // 16, E), 12345, device=DEV, dtype=torch.int32).view(torch.uint32)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -83,6 +92,22 @@ def test_router_forward(dtype, T, H, E, k):
     # and without the optional histogram the other outputs are the same bits
     l2, w2, s2, _ = _run_forward(x.to(DEV), w.to(DEV), k, with_counts=False)
     assert torch.equal(l2.cpu(), logits) and torch.equal(w2.cpu(), weights) and torch.equal(s2.cpu(), selected)
+
+    # the histogram per block of 16 tokens (with and without the total beside it), and the index built from it:
+    # the same five arrays as from the ids alone
+    for with_counts in (False, True):
+        hist = _block_hist_buffer(T, E)
+        l3, w3, s3, c3 = _run_forward(x.to(DEV), w.to(DEV), k, with_counts=with_counts, block_hist=hist)
+        assert torch.equal(l3.cpu(), logits) and torch.equal(w3.cpu(), weights) and torch.equal(s3.cpu(), selected)
+        expect_hist = np.zeros(((T + 15) // 16, E), dtype=np.int64)
+        np.add.at(expect_hist, (np.repeat(np.arange(T) // 16, k), selected.numpy().reshape(-1)), 1)
+        assert np.array_equal(to_np(hist).astype(np.int64), expect_hist)
+        if with_counts:
+            assert np.array_equal(to_np(c3), to_np(counts))
+    plain = build_routing_index(s3, E)
+    from_hist = build_routing_index(s3, E, token_block_histogram=hist)
+    for a, b, name in zip(from_hist, plain, ("counts", "offsets", "perm", "eid", "inv")):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32)), name
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -222,7 +247,7 @@ def test_router_rejects_bad_arguments():
         T, E = x.size(0), w.size(0)
         router_topk_cuda(
             x, w, k, torch.empty(T, E, device=DEV, dtype=x.dtype), torch.empty(T, k, device=DEV, dtype=x.dtype),
-            torch.empty(T, k, device=DEV, dtype=torch.int32), None,
+            torch.empty(T, k, device=DEV, dtype=torch.int32), None, None,
         )
 
     with pytest.raises(RuntimeError, match="top_k"):
