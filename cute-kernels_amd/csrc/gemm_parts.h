@@ -85,6 +85,24 @@ __device__ __forceinline__ void buffer_load_lds_quiet_b32(u32x4 rsrc, uint32_t v
                  : "=&s"(saved_m0)
                  : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr));
 }
+// LDS words at addr, addr + 256, addr + 512 and addr + 768 bytes, read in assembly and waited for here: for a table that
+// only direct-to-LDS loads written in assembly fill, which the compiler therefore knows nothing about
+__device__ __forceinline__ void lds_read4_stride64_quiet(uint32_t addr, uint32_t (&v)[4]) {
+    uint2 a, b;
+    asm volatile("ds_read2st64_b32 %0, %2 offset1:1\n\tds_read2st64_b32 %1, %2 offset0:2 offset1:3\n\t"
+                 "s_waitcnt lgkmcnt(0)"
+                 : "=&v"(a), "=&v"(b)
+                 : "v"(addr));
+    v[0] = a.x;
+    v[1] = a.y;
+    v[2] = b.x;
+    v[3] = b.y;
+}
+__device__ __forceinline__ uint32_t lds_read1_quiet(uint32_t addr) {
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr));
+    return v;
+}
 __device__ __forceinline__ uint32_t lds_address(const uint8_t* p) {
     return (uint32_t)(uintptr_t)(lds_void*)const_cast<uint8_t*>(p);
 }

@@ -44,6 +44,9 @@ struct Args {
     uint16_t* ACT;          // swiglu only: activation output
     const uint32_t* sizes;  // E values of the varying dimension
     const uint16_t* bias;   // BIAS kernels: [E, n] added to the rounded product before anything else
+    // GATHER kernels: row i of the packed A operand is row row_index[i] / divisor of A, which has a_rows rows
+    const int32_t* row_index;
+    uint32_t divisor, a_rows;
     uint32_t E;
     uint32_t m, n, k;  // the dimensions all groups share (the varying one is ignored)
     float alpha;
@@ -69,10 +72,11 @@ __device__ unsigned long long fma_prof[1024 * 8 * 8];
 #define PROF_STAMP(t) asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t))
 #endif
 
-template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K, bool BIAS>
+template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K, bool BIAS, bool GATHER>
 __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     static_assert(EPI == EPI_PLAIN || (A_KC && B_KC && !VARY_K), "the SwiGLU epilogue exists for the NT layout only");
     static_assert(!BIAS || (A_KC && B_KC && !VARY_K), "the bias term exists for the forward (NT) layout only");
+    static_assert(!GATHER || (A_KC && B_KC && !VARY_K), "rows are gathered in the forward (NT) layout only");
 
     // one array per stage and operand: distinct LDS objects let the compiler see that a direct-to-LDS load
     // into one stage cannot alias the fragment reads of the other, so it does not wait for the load first
@@ -82,9 +86,12 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     __shared__ __attribute__((aligned(1024))) uint8_t s_b1[kTileBytes];
     __shared__ __attribute__((aligned(1024))) uint8_t s_stage[NW * kStageBytes];
     __shared__ uint32_t s_pf[64];  // where the dwords fetched by the L2 prefetch end up (never read)
-    // BIAS: per wavefront, the bias values of the tile's 256 columns (plain) or 128 "up" | 128 "gate" columns
-    constexpr int kBiasBytes = 512;
+    // BIAS: per wavefront, the bias values of its own 64 columns (plain) or 32 "up" | 32 "gate" columns
+    constexpr int kBiasBytes = 128;
     __shared__ __attribute__((aligned(256))) uint8_t s_bias[BIAS ? NW * kBiasBytes : 16];
+    // GATHER: the row_index entries of the 256 rows of a tile, for the tile of round r in half r % 2. Filled by
+    // direct-to-LDS loads and read in assembly: the compiler never sees an access to it.
+    __shared__ __attribute__((aligned(256))) uint32_t s_rows[GATHER ? 512 : 4];
     // The group table, one LDS object: first tile of the group at position p of the tile sequence, exclusive prefix of the
     // varying dimension over the groups, and which group is at position p.
     __shared__ uint32_t s_table[2 * (FMA_MAX_GROUPS + 1) + FMA_MAX_GROUPS / 2];
@@ -236,6 +243,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         bool valid, fast;
         uint32_t Me, Ke, m0, n0, n_lim;  // n_lim: first column past the tile (kTileN columns wide, or half of that)
         uint32_t e;                      // the group
+        uint32_t row0;                   // rows vary: first packed row of the group
         uint64_t off_a, off_b, off_d;
         uint32_t pf_r, pf_c;  // position of the tile in its XCD's 8 x 4 block of tiles (row, column)
     };
@@ -279,6 +287,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             t.off_b = before * Ne;
             t.off_d = (uint64_t)e * args.m * Ne;
         } else {
+            t.row0 = (uint32_t)before;
             t.off_a = before * args.k;
             t.off_b = (uint64_t)e * Ne * args.k;
             t.off_d = before * Ne;
@@ -298,6 +307,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     // a tile whose first two K steps can be fetched by the tile before it, and which can fetch the next tile's
     auto streams = [&](const Tile& t) { return t.valid && t.fast && t.Ke > 0 && !is_thin(t); };
 
+    uint32_t round = 0;  // tiles this workgroup has finished
+
     // ---- loaders: `cur` feeds the tile being computed, `nxt` the tile after it ----
     LoaderK<NW, false> lk_a;
     LoaderK<NW, EPI != EPI_PLAIN> lk_b;
@@ -307,6 +318,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     uint32_t va_cur = 0, va_nxt = 0, vb_cur = 0, vb_nxt = 0;  // the loaders' per-lane offsets (they depend on the pitch)
     // sets a loader object up for tile t and keeps what is specific to the tile
     auto setup_a = [&](const Tile& t, Feed<A_KC>& f, uint32_t& v) {
+        if constexpr (GATHER) return;  // nothing per tile: the rows come from the table in s_rows
         const uint16_t* Ae = args.A + t.off_a;
         if constexpr (A_KC) {
             lk_a.setup(Ae + (uint64_t)t.m0 * t.Ke, nullptr, t.Me - t.m0 < (uint32_t)BM ? t.Me - t.m0 : (uint32_t)BM, t.Ke, wave, lane);
@@ -337,6 +349,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     };
     // points a loader object at a feed (what depends on lane and wavefront only stays as the last setup left it)
     auto aim_a = [&](const Feed<A_KC>& f, uint32_t v) {
+        if constexpr (GATHER) return;
         if constexpr (A_KC) { lk_a.base0 = f.base0; lk_a.bytes = f.extent; lk_a.ldb = f.ldb; lk_a.kdim = f.ldb / 2u; lk_a.voff = v; }
         else { lt_a.base = f.base0; lt_a.kdim = f.extent; lt_a.ldb = f.ldb; lt_a.col_bytes = f.col_bytes; lt_a.voff = v; }
     };
@@ -344,6 +357,55 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         if constexpr (B_KC) { lk_b.base0 = f.base0; lk_b.base1 = f.base1; lk_b.bytes = f.extent; lk_b.ldb = f.ldb; lk_b.kdim = f.ldb / 2u; lk_b.voff = v; }
         else { lt_b.base = f.base0; lt_b.kdim = f.extent; lt_b.ldb = f.ldb; lt_b.col_bytes = f.col_bytes; lt_b.voff = v; }
     };
+
+    // ---- GATHER: the A operand's rows are rows of args.A picked through args.row_index ----
+    // The tile of round r keeps the row_index entries of its 256 rows in half r % 2 of s_rows. A wavefront's four load
+    // instructions of a K step fetch tile rows g_row, g_row + 64, + 128, + 192 of this lane: four table entries, divided by
+    // the divisor, times the row pitch. Entries past the group's rows read as zero (row 0 of A: rows never stored).
+    const uint32_t g_full = GATHER ? args.a_rows * args.k * 2u : 0u;  // bytes of A (below 2^31)
+    const uint32_t g_ldb = args.k * 2u;
+    const uint32_t g_row = logical_row(wave * 8u + (lane >> 3));
+    const uint32_t g_chunk = (lane & 7u) ^ (g_row & 7u);
+    // n / divisor for n < 2^31: the high word of n * ceil(2^32 / divisor) is the quotient or one more
+    const uint32_t g_magic = (GATHER && args.divisor > 1u) ? (uint32_t)((0x100000000ull + args.divisor - 1u) / args.divisor) : 0u;
+    auto g_source_row = [&](uint32_t n) -> uint32_t {
+        if (args.divisor == 1u) return n;
+        uint32_t q = __umulhi(n, g_magic);
+        if (q * args.divisor > n) --q;
+        return q;
+    };
+    uint32_t g_bytes_nxt = 0;  // bytes of A the loads for the next tile may read: all of it, or nothing when nothing follows
+    // per-lane offsets of the four loads of a K step of the tile in table half `half` (the step's k0 goes into the
+    // instruction's scalar offset)
+    auto g_tile_offsets = [&](uint32_t half, uint32_t (&v)[4]) {
+        uint32_t n[4];
+        lds_read4_stride64_quiet(lds_address(reinterpret_cast<const uint8_t*>(s_rows)) + half * 1024u + g_row * 4u, n);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = g_source_row(n[i]) * g_ldb + g_chunk * 16u;
+    };
+    // last, partial K step: chunks past the end of K are pushed out of range, which zero-fills them
+    auto g_clip = [&](uint32_t k0, uint32_t (&v)[4]) {
+        const bool past = k0 + (uint32_t)BK > args.k && k0 + g_chunk * 8u >= args.k;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = past ? kOutOfRange : v[i];
+    };
+    auto g_offsets = [&](uint32_t half, uint32_t k0, uint32_t (&v)[4]) {
+        g_tile_offsets(half, v);
+        g_clip(k0, v);
+    };
+    uint32_t g_kept[4] = {0u, 0u, 0u, 0u};  // g_tile_offsets of the tile the full-tile K loop is loading from
+    // the table of tile t into half `half`: 32 entries per wavefront, in assembly (one load per wavefront)
+    auto g_issue_table = [&](const Tile& t, uint32_t half) {
+        if constexpr (GATHER) {
+            const bool real = t.valid && t.Me > t.m0;
+            const uint32_t rows = real ? (t.Me - t.m0 < (uint32_t)BM ? t.Me - t.m0 : (uint32_t)BM) : 0u;
+            const u32x4 rs = make_rsrc_words(reinterpret_cast<const uint16_t*>(args.row_index + (real ? (uint64_t)t.row0 + t.m0 : 0u)),
+                                             rows * 4u);
+            const uint32_t to = lds_address(reinterpret_cast<const uint8_t*>(s_rows)) + half * 1024u + wave * 128u;
+            if (lane < 32u) buffer_load_lds_quiet_b32(rs, (wave * 32u + lane) * 4u, 0u, to);
+        }
+    };
+    static_assert(!GATHER || 32 / NW == 4, "four load instructions per wavefront and K step");
 
     // ---- L2 prefetch by designated workgroups (grouped_gemm.hip): one 4-byte load per shared line, kPfDist steps ahead ----
     constexpr bool kPrefetch = A_KC == B_KC;
@@ -358,7 +420,12 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         pf_steps = k_steps(t);
         if (!pf_is_b) {
             const uint32_t i = p * 16u + lane;
-            if constexpr (A_KC) {
+            if constexpr (GATHER) {
+                const uint32_t n = lds_read1_quiet(lds_address(reinterpret_cast<const uint8_t*>(s_rows)) + (round & 1u) * 1024u +
+                                                   (lane < 16u ? 4u * i + t.pf_c : 0u) * 4u);
+                pf_base = args.A; pf_bytes = g_full;
+                pf_voff = lane < 16u ? g_source_row(n) * g_ldb : kOutOfRange;
+            } else if constexpr (A_KC) {
                 pf_base = fa_cur.base0; pf_bytes = fa_cur.extent;
                 pf_voff = lane < 16u ? (4u * i + t.pf_c) * (t.Ke * 2u) : kOutOfRange;
             } else {
@@ -402,13 +469,37 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         if constexpr (A_KC) lk_a.template issue_range<0, kLoads>(stage ? s_a1 : s_a0, k0);
         else lt_a.template issue_range<0, kLoads>(stage ? s_a1 : s_a0, k0);
     };
+    // GATHER: the same four loads through the row table in half `half`; `bytes`: how much of A they may read
+    // kept: take the offsets from g_kept (the caller has set it for that tile) instead of reading the table
+    auto issue_a_gathered = [&](int stage, uint32_t k0, uint32_t half, uint32_t bytes, bool kept) {
+        uint32_t v[4];
+        if (kept) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = g_kept[i];
+            g_clip(k0, v);
+        } else {
+            g_offsets(half, k0, v);
+        }
+        const __amdgpu_buffer_rsrc_t r = make_rsrc(args.A, bytes);
+        uint8_t* tile = stage ? s_a1 : s_a0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(tile + (i * NW + wave) * 1024), 16, v[i], k0 * 2u, 0, 0);
+    };
     auto issue_b = [&](int stage, uint32_t k0) {
         if constexpr (B_KC) lk_b.template issue_range<0, kLoads>(stage ? s_b1 : s_b0, k0);
         else lt_b.template issue_range<0, kLoads>(stage ? s_b1 : s_b0, k0);
     };
     // ... and written in assembly, for a cold start
     auto issue_quiet = [&](int stage, uint32_t k0) {
-        if constexpr (A_KC) lk_a.issue_quiet(stage ? s_a1 : s_a0, k0);
+        if constexpr (GATHER) {
+            uint32_t v[4];
+            g_offsets(round & 1u, k0, v);
+            const u32x4 r = make_rsrc_words(args.A, g_full);
+            const uint32_t lds0 = lds_address(stage ? s_a1 : s_a0) + wave * 1024u;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) buffer_load_lds_quiet(r, v[i], k0 * 2u, lds0 + (uint32_t)(i * NW) * 1024u);
+        } else if constexpr (A_KC) lk_a.issue_quiet(stage ? s_a1 : s_a0, k0);
         else lt_a.issue_quiet(stage ? s_a1 : s_a0, k0);
         if constexpr (B_KC) lk_b.issue_quiet(stage ? s_b1 : s_b0, k0);
         else lt_b.issue_quiet(stage ? s_b1 : s_b0, k0);
@@ -418,8 +509,10 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     uint64_t p_start, p_t0 = 0, p_t1 = 0, p_seg[6] = {0, 0, 0, 0, 0, 0}, p_tiles = 0;
     PROF_STAMP(p_start);
 #endif
-    uint32_t round = 0;
     Tile cur = lookup(0), nxt = lookup(1);
+    // GATHER: the second tile's rows (the first tile fetches its own in its cold start; from then on every tile
+    // fetches those of the tile after next, before its epilogue)
+    g_issue_table(nxt, 1u);
     bool streamed = false;  // the first two K steps of `cur` were fetched by the tile before it
     while (cur.valid) {
         const uint32_t Me = cur.Me, Ke = cur.Ke, m0 = cur.m0, n0 = cur.n0, n_lim = cur.n_lim;
@@ -439,6 +532,13 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             setup_a(cur, fa_cur, va_cur);
             setup_b(cur, fb_cur, vb_cur);
         }
+        if (GATHER && !streamed) {
+            // a tile that starts cold fetches its own rows and waits for them (and for everything else in flight)
+            g_issue_table(cur, round & 1u);
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, false));
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        }
         setup_prefetch(cur);
         const uint32_t KT = (Ke + BK - 1) / BK;
         const uint32_t KT2 = (KT + 1u) & ~1u;  // steps of the K loop: an odd count gets a step of zeros
@@ -450,13 +550,16 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             setup_b(nxt, fb_nxt, vb_nxt);
         } else {
             // a feed that fetches nothing: every load of it zero-fills
-            fa_nxt = fa_cur;
+            if constexpr (!GATHER) {
+                fa_nxt = fa_cur;
+                fa_nxt.extent = 0u;
+                va_nxt = va_cur;
+            }
             fb_nxt = fb_cur;
-            fa_nxt.extent = 0u;
             fb_nxt.extent = 0u;
-            va_nxt = va_cur;
             vb_nxt = vb_cur;
         }
+        g_bytes_nxt = stream_next ? g_full : 0u;
         // (the set-ups above left the loader objects aimed at the last tile set up)
         aim_a(fa_cur, va_cur);
         aim_b(fb_cur, vb_cur);
@@ -529,15 +632,21 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             } else {
                 const bool of_next = kt + 2u >= KT2;
                 k0 = (of_next ? kt + 2u - KT2 : kt + 2u) * (uint32_t)BK;
-                aim_a(Feed<A_KC>{of_next ? fa_nxt.base0 : fa_cur.base0, nullptr, of_next ? fa_nxt.extent : fa_cur.extent,
-                                 of_next ? fa_nxt.ldb : fa_cur.ldb, of_next ? fa_nxt.col_bytes : fa_cur.col_bytes},
-                      of_next ? va_nxt : va_cur);
+                if constexpr (!GATHER)
+                    aim_a(Feed<A_KC>{of_next ? fa_nxt.base0 : fa_cur.base0, nullptr, of_next ? fa_nxt.extent : fa_cur.extent,
+                                     of_next ? fa_nxt.ldb : fa_cur.ldb, of_next ? fa_nxt.col_bytes : fa_cur.col_bytes},
+                          of_next ? va_nxt : va_cur);
                 aim_b(Feed<B_KC>{of_next ? fb_nxt.base0 : fb_cur.base0, of_next ? fb_nxt.base1 : fb_cur.base1,
                                  of_next ? fb_nxt.extent : fb_cur.extent, of_next ? fb_nxt.ldb : fb_cur.ldb,
                                  of_next ? fb_nxt.col_bytes : fb_cur.col_bytes},
                       of_next ? vb_nxt : vb_cur);
             }
-            issue_a(stage, k0);
+            if constexpr (GATHER) {
+                const bool of_next = SRC == 1 || (SRC == 2 && kt + 2u >= KT2);
+                issue_a_gathered(stage, k0, (of_next ? round + 1u : round) & 1u, of_next ? g_bytes_nxt : g_full, SRC != 2);
+            } else {
+                issue_a(stage, k0);
+            }
             issue_b(stage, k0);
             // the prefetch goes out behind this step's loads (the empty statement orders it: the wait of the next step
             // counts on it being the newest load)
@@ -554,18 +663,20 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         // stores of the previous epilogue (or the cold start's stand-ins) and the two loads of the bias tile are newer
         // than the loads waited for as well
         using WaitStep = std::integral_constant<int, waitcnt_imm(kPrefetch ? 1 : 0, true)>;
-        using WaitFirst = std::integral_constant<int, waitcnt_imm((int)kTileStores + (kPrefetch ? 1 : 0) + (BIAS ? 2 : 0), true)>;
+        using WaitFirst = std::integral_constant<int, waitcnt_imm((int)kTileStores + (kPrefetch ? 1 : 0) + (BIAS ? 1 : 0), true)>;
 
-        // BIAS: this tile's bias values into this wavefront's 512 bytes of LDS: two 256-byte loads, complete (loads and
-        // stores complete in issue order) long before the epilogue reads them. Columns past the end zero-fill.
+        // BIAS: the bias values of this wavefront's columns of the tile into its 128 bytes of LDS: one load by 32 lanes
+        // (every wavefront issues it, so that all count the same loads), complete (loads and stores complete in issue
+        // order) long before the epilogue reads them. Columns past the end zero-fill.
         auto issue_bias = [&]() {
             if constexpr (BIAS) {
                 const uint16_t* row = args.bias + (uint64_t)cur.e * Ne;
                 const u32x4 rs = make_rsrc_words(row, Ne * 2u);
                 const uint32_t to = lds_address(s_bias) + wave * (uint32_t)kBiasBytes;
-                const uint32_t second = EPI != EPI_PLAIN ? n_span * 2u : 256u;  // byte offset of the second 128 columns
-                buffer_load_lds_quiet_b32(rs, n0 * 2u + lane * 4u, 0u, to);
-                buffer_load_lds_quiet_b32(rs, n0 * 2u + second + lane * 4u, 0u, to + 256u);
+                // plain: columns n0 + wn*64 + 2*lane; swiglu: lanes 0..15 the 32 "up" columns, lanes 16..31 the "gate" ones
+                const uint32_t col = EPI == EPI_PLAIN ? n0 + wn * WN + 2u * lane
+                                                      : n0 + wn * (WN / 2) + 2u * (lane & 15u) + (lane >= 16u ? n_span : 0u);
+                if (lane < 32u) buffer_load_lds_quiet_b32(rs, col * 2u, 0u, to);
             }
         };
         Tile nn{};  // the tile after next
@@ -581,7 +692,11 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             const uint8_t* const b_lo[3] = {s_b0, s_b1, s_a0 + 16384};
             const uint8_t* const b_hi[3] = {s_b0 + 16384, s_b1 + 16384, s_a1 + 16384};
             auto issue_thin = [&](int st, uint32_t k0) {
-                if constexpr (A_KC) lk_a.issue_quiet_first_rows(lds_address(a_at[st]), k0);
+                if constexpr (GATHER) {
+                    uint32_t v[4];
+                    g_offsets(round & 1u, k0, v);
+                    buffer_load_lds_quiet(make_rsrc_words(args.A, g_full), v[0], k0 * 2u, lds_address(a_at[st]) + wave * 1024u);
+                } else if constexpr (A_KC) lk_a.issue_quiet_first_rows(lds_address(a_at[st]), k0);
                 if constexpr (B_KC) lk_b.issue_quiet_halves(lds_address(b_lo[st]), lds_address(b_hi[st]), k0);
                 else lt_b.issue_quiet_halves(lds_address(b_lo[st]), lds_address(b_hi[st]), k0);
             };
@@ -678,6 +793,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                     if (KT2 > 2u) {
                         aim_a(fa_cur, va_cur);
                         aim_b(fb_cur, vb_cur);
+                        if constexpr (GATHER) g_tile_offsets(round & 1u, g_kept);
                         uint32_t kt = 2;
                         for (; kt + 2u < KT2; kt += 2) {  // two steps per iteration without a branch between them
                             step(fa_c, WaitStep{}, SrcCur{}, 0, kt);
@@ -685,6 +801,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                         }
                         aim_a(fa_nxt, va_nxt);
                         aim_b(fb_nxt, vb_nxt);
+                        if constexpr (GATHER) g_tile_offsets((round + 1u) & 1u, g_kept);
                         step(fa_c, WaitStep{}, SrcNext{}, 0, kt);
                         step(fa_c, WaitStep{}, SrcNext{}, 1, kt + 1);
                     }
@@ -722,6 +839,9 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         }
         // the tile after next is looked up here: scalar work beside an epilogue that is bound by the store path
         nn = lookup(round + 2);
+        // GATHER: its rows go where this tile's were (no load of this tile is left to be issued). The load is older than
+        // this tile's stores, so the first wait of the next tile covers it.
+        g_issue_table(nn, round & 1u);
 #ifdef FMA_PROF
         PROF_STAMP(p_t1);
         p_seg[1] += p_t1 - p_t0;  // look-up
@@ -753,8 +873,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             for (int j = 0; j < FN; ++j)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    // plain: column wn*64 + j*32 + ...; swiglu: "up" (j = 0) in the first 256 bytes, "gate" in the second
-                    const uint32_t c = (EPI == EPI_PLAIN ? wn * WN + j * 32 : j * 128 + wn * (WN / 2)) + q * 8 + (el >> 5) * 4;
+                    // plain: 64 columns; swiglu: 32 "up" columns (j = 0), then 32 "gate" columns
+                    const uint32_t c = j * 32 + q * 8 + (el >> 5) * 4;
                     at[j * 4 + q] = mine + c * 2u;
                 }
             lds_read8x8_quiet(at, raw);
@@ -866,9 +986,11 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         // ---- on to the next tile ----
         streamed = stream_next;
         if (stream_next) {
-            fa_cur = fa_nxt;
+            if constexpr (!GATHER) {
+                fa_cur = fa_nxt;
+                va_cur = va_nxt;
+            }
             fb_cur = fb_nxt;
-            va_cur = va_nxt;
             vb_cur = vb_nxt;
         }
         cur = nxt;
@@ -891,29 +1013,46 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
 
 // every instantiation the entry points launch (explicit, so that host stub and device code are both emitted)
 #define FMA_RAGGED_INSTANTIATE(EL)                                                                          \
-    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, false, false>(const Args);           \
-    template __global__ void ragged_gemm_kernel<EL, true, false, EPI_PLAIN, false, false>(const Args);          \
-    template __global__ void ragged_gemm_kernel<EL, false, true, EPI_PLAIN, false, false>(const Args);          \
-    template __global__ void ragged_gemm_kernel<EL, false, false, EPI_PLAIN, false, false>(const Args);         \
-    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, true, false>(const Args);            \
-    template __global__ void ragged_gemm_kernel<EL, true, false, EPI_PLAIN, true, false>(const Args);           \
-    template __global__ void ragged_gemm_kernel<EL, false, true, EPI_PLAIN, true, false>(const Args);           \
-    template __global__ void ragged_gemm_kernel<EL, false, false, EPI_PLAIN, true, false>(const Args);          \
-    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU, false, false>(const Args);          \
-    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false, false>(const Args);      \
-    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, false, true>(const Args);            \
-    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU, false, true>(const Args);           \
-    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false, true>(const Args);
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, false, false, false>(const Args);    \
+    template __global__ void ragged_gemm_kernel<EL, true, false, EPI_PLAIN, false, false, false>(const Args);   \
+    template __global__ void ragged_gemm_kernel<EL, false, true, EPI_PLAIN, false, false, false>(const Args);   \
+    template __global__ void ragged_gemm_kernel<EL, false, false, EPI_PLAIN, false, false, false>(const Args);  \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, true, false, false>(const Args);     \
+    template __global__ void ragged_gemm_kernel<EL, true, false, EPI_PLAIN, true, false, false>(const Args);    \
+    template __global__ void ragged_gemm_kernel<EL, false, true, EPI_PLAIN, true, false, false>(const Args);    \
+    template __global__ void ragged_gemm_kernel<EL, false, false, EPI_PLAIN, true, false, false>(const Args);   \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU, false, false, false>(const Args);   \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false, false, false>(const Args); \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, false, true, false>(const Args);     \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU, false, true, false>(const Args);    \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false, true, false>(const Args); \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, false, false, true>(const Args);     \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU, false, false, true>(const Args);    \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false, false, true>(const Args); \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, false, true, true>(const Args);      \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU, false, true, true>(const Args);     \
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false, true, true>(const Args);
 FMA_RAGGED_INSTANTIATE(ElemBf16)
 FMA_RAGGED_INSTANTIATE(ElemF16)
 #undef FMA_RAGGED_INSTANTIATE
 
-template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K, bool BIAS = false>
+template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K, bool BIAS = false, bool GATHER = false>
 int launch(const Args& args, hipStream_t st) {
     int cus = num_compute_units();
     if (cus <= 0) cus = 256;
-    hipLaunchKernelGGL((ragged_gemm_kernel<EL, A_KC, B_KC, EPI, VARY_K, BIAS>), dim3((uint32_t)cus), dim3(NT), 0, st, args);
+    hipLaunchKernelGGL((ragged_gemm_kernel<EL, A_KC, B_KC, EPI, VARY_K, BIAS, GATHER>), dim3((uint32_t)cus), dim3(NT), 0, st,
+                       args);
     return launch_status("grouped_gemm_ragged");
+}
+
+// the forward (NT) kernels by epilogue, bias and gather
+template <typename EL, int EPI>
+int launch_forward(const Args& args, hipStream_t st) {
+    const bool bias = args.bias != nullptr, gather = args.row_index != nullptr;
+    if (bias && gather) return launch<EL, true, true, EPI, false, true, true>(args, st);
+    if (bias) return launch<EL, true, true, EPI, false, true, false>(args, st);
+    if (gather) return launch<EL, true, true, EPI, false, false, true>(args, st);
+    return launch<EL, true, true, EPI, false, false, false>(args, st);
 }
 
 template <typename EL, bool VARY_K>
@@ -922,6 +1061,54 @@ int launch_plain(const Args& args, bool a_kc, bool b_kc, hipStream_t st) {
     if (a_kc && !b_kc) return launch<EL, true, false, EPI_PLAIN, VARY_K>(args, st);
     if (!a_kc && b_kc) return launch<EL, false, true, EPI_PLAIN, VARY_K>(args, st);
     return launch<EL, false, false, EPI_PLAIN, VARY_K>(args, st);
+}
+
+// The forward product of an expert projection, out_e = x_e W_e^T (+ bias_e), with the rows of x_e packed (row_index
+// NULL) or picked through row_index; swiglu: N = 2 I, out is the pre-activation (may be NULL) and act its activation.
+int up_projection(const char* who, const void* x, int64_t x_rows, const int32_t* row_index, int32_t divisor, const void* W,
+                  const void* bias, void* out, void* act, const uint32_t* M_arr, int64_t E, int64_t N, int64_t K, int swiglu,
+                  int dtype, hipStream_t st) {
+    FMA_REQUIRE(dtype == FMA_BF16 || dtype == FMA_F16, dtype_bytes(dtype) ? FMA_ERR_UNSUPPORTED : FMA_ERR_BAD_DTYPE,
+                "%s: bf16 and fp16 operands are implemented (dtype code %d)", who, dtype);
+    FMA_REQUIRE(E >= 0, FMA_ERR_BAD_SIZE, "%s: negative group count %lld", who, (long long)E);
+    FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "%s: E=%lld exceeds the limit %d", who, (long long)E,
+                FMA_MAX_GROUPS);
+    // the upper bounds are those of the kernel's 32-bit tile offsets; these entry points have no scalar path beyond them
+    if (swiglu) {
+        FMA_REQUIRE(N >= 16 && N % 16 == 0 && N < (1ll << 23), FMA_ERR_BAD_SIZE,
+                    "%s: intermediate size %lld must be a positive multiple of 8 below 2^22", who, (long long)(N / 2));
+    } else {
+        FMA_REQUIRE(N >= 8 && N % 8 == 0 && N < (1ll << 23), FMA_ERR_BAD_SIZE,
+                    "%s: N=%lld must be a positive multiple of 8 below 2^23", who, (long long)N);
+    }
+    FMA_REQUIRE(K >= 8 && K % 8 == 0 && K < (1ll << 21), FMA_ERR_BAD_SIZE,
+                "%s: K=%lld must be a positive multiple of 8 below 2^21", who, (long long)K);
+    if (E == 0) return FMA_OK;
+    FMA_REQUIRE(x && W && M_arr && (swiglu ? act != nullptr : out != nullptr), FMA_ERR_NULL_POINTER, "%s: NULL pointer", who);
+    FMA_REQUIRE(aligned16(x) && aligned16(W) && aligned16(act) && aligned16(out), FMA_ERR_MISALIGNED,
+                "%s: x, W and the outputs must be 16-byte aligned", who);
+    FMA_REQUIRE((reinterpret_cast<uintptr_t>(bias) & 3u) == 0 && (reinterpret_cast<uintptr_t>(row_index) & 3u) == 0,
+                FMA_ERR_MISALIGNED, "%s: bias and row_index must be 4-byte aligned", who);
+    Args args{};
+    args.A = (const uint16_t*)x;
+    args.B = (const uint16_t*)W;
+    args.D = (uint16_t*)out;
+    args.ACT = swiglu ? (uint16_t*)act : nullptr;
+    args.sizes = M_arr;
+    args.bias = (const uint16_t*)bias;
+    args.row_index = row_index;
+    args.divisor = (uint32_t)divisor;
+    args.a_rows = (uint32_t)x_rows;
+    args.E = (uint32_t)E;
+    args.m = 0;
+    args.n = (uint32_t)N;
+    args.k = (uint32_t)K;
+    args.alpha = 1.0f;
+    // whether the pre-activation is stored is a compile-time property of the kernel: the epilogue is then one
+    // straight-line block
+    if (!swiglu) return dtype == FMA_BF16 ? launch_forward<ElemBf16, EPI_PLAIN>(args, st) : launch_forward<ElemF16, EPI_PLAIN>(args, st);
+    if (out) return dtype == FMA_BF16 ? launch_forward<ElemBf16, EPI_SWIGLU>(args, st) : launch_forward<ElemF16, EPI_SWIGLU>(args, st);
+    return dtype == FMA_BF16 ? launch_forward<ElemBf16, EPI_SWIGLU_ACT>(args, st) : launch_forward<ElemF16, EPI_SWIGLU_ACT>(args, st);
 }
 
 }  // namespace ragged
@@ -981,8 +1168,8 @@ int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_
     args.k = (uint32_t)K;
     args.alpha = alpha;
     if (bias)
-        return dtype == FMA_BF16 ? ragged::launch<ElemBf16, true, true, EPI_PLAIN, false, true>(args, st)
-                                 : ragged::launch<ElemF16, true, true, EPI_PLAIN, false, true>(args, st);
+        return dtype == FMA_BF16 ? ragged::launch_forward<ElemBf16, EPI_PLAIN>(args, st)
+                                 : ragged::launch_forward<ElemF16, EPI_PLAIN>(args, st);
     if (vary == FMA_VARY_K)
         return dtype == FMA_BF16 ? ragged::launch_plain<ElemBf16, true>(args, a_kc, b_kc, st)
                                  : ragged::launch_plain<ElemF16, true>(args, a_kc, b_kc, st);
@@ -992,50 +1179,24 @@ int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_
 
 int fma_grouped_gemm_swiglu(const void* x, const void* W, const void* bias, void* h, void* act, const uint32_t* M_arr,
                             int64_t E, int64_t I, int64_t K, int dtype, void* stream) {
+    return fmahip::gemm::ragged::up_projection("grouped_gemm_swiglu", x, 0, nullptr, 1, W, bias, h, act, M_arr, E, 2 * I, K,
+                                               1, dtype, (hipStream_t)stream);
+}
+
+int fma_grouped_gemm_gathered(const void* x, int64_t x_rows, const int32_t* row_index, int32_t divisor, const void* W,
+                              const void* bias, void* out, void* act, const uint32_t* M_arr, int64_t E, int64_t N,
+                              int64_t K, int swiglu, int dtype, void* stream) {
     using namespace fmahip;
-    using namespace fmahip::gemm;
-    FMA_REQUIRE(dtype == FMA_BF16 || dtype == FMA_F16, dtype_bytes(dtype) ? FMA_ERR_UNSUPPORTED : FMA_ERR_BAD_DTYPE,
-                "grouped_gemm_swiglu: bf16 and fp16 operands are implemented (dtype code %d)", dtype);
-    FMA_REQUIRE(E >= 0, FMA_ERR_BAD_SIZE, "grouped_gemm_swiglu: negative group count %lld", (long long)E);
-    FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "grouped_gemm_swiglu: E=%lld exceeds the limit %d",
-                (long long)E, FMA_MAX_GROUPS);
-    // the upper bounds are those of the kernel's 32-bit tile offsets; this entry point has no scalar path beyond them
-    FMA_REQUIRE(I >= 8 && I % 8 == 0 && 2 * I < (1ll << 23), FMA_ERR_BAD_SIZE,
-                "grouped_gemm_swiglu: intermediate size %lld must be a positive multiple of 8 below 2^22", (long long)I);
-    FMA_REQUIRE(K >= 8 && K % 8 == 0 && K < (1ll << 21), FMA_ERR_BAD_SIZE,
-                "grouped_gemm_swiglu: K=%lld must be a positive multiple of 8 below 2^21", (long long)K);
-    if (E == 0) return FMA_OK;
-    FMA_REQUIRE(x && W && act && M_arr, FMA_ERR_NULL_POINTER, "grouped_gemm_swiglu: NULL pointer");
-    FMA_REQUIRE(aligned16(x) && aligned16(W) && aligned16(act) && aligned16(h), FMA_ERR_MISALIGNED,
-                "grouped_gemm_swiglu: x, W, h and act must be 16-byte aligned");
-    FMA_REQUIRE((reinterpret_cast<uintptr_t>(bias) & 3u) == 0, FMA_ERR_MISALIGNED,
-                "grouped_gemm_swiglu: the bias must be 4-byte aligned");
-    ragged::Args args{};
-    args.bias = (const uint16_t*)bias;
-    args.A = (const uint16_t*)x;
-    args.B = (const uint16_t*)W;
-    args.D = (uint16_t*)h;
-    args.ACT = (uint16_t*)act;
-    args.sizes = M_arr;
-    args.E = (uint32_t)E;
-    args.m = 0;
-    args.n = (uint32_t)(2 * I);
-    args.k = (uint32_t)K;
-    args.alpha = 1.0f;
-    hipStream_t st = (hipStream_t)stream;
-    // whether h is stored is a compile-time property of the kernel: the epilogue is then one straight-line block
-    if (bias) {
-        if (h)
-            return dtype == FMA_BF16 ? ragged::launch<ElemBf16, true, true, EPI_SWIGLU, false, true>(args, st)
-                                     : ragged::launch<ElemF16, true, true, EPI_SWIGLU, false, true>(args, st);
-        return dtype == FMA_BF16 ? ragged::launch<ElemBf16, true, true, EPI_SWIGLU_ACT, false, true>(args, st)
-                                 : ragged::launch<ElemF16, true, true, EPI_SWIGLU_ACT, false, true>(args, st);
-    }
-    if (h)
-        return dtype == FMA_BF16 ? ragged::launch<ElemBf16, true, true, EPI_SWIGLU, false>(args, st)
-                                 : ragged::launch<ElemF16, true, true, EPI_SWIGLU, false>(args, st);
-    return dtype == FMA_BF16 ? ragged::launch<ElemBf16, true, true, EPI_SWIGLU_ACT, false>(args, st)
-                             : ragged::launch<ElemF16, true, true, EPI_SWIGLU_ACT, false>(args, st);
+    FMA_REQUIRE(row_index != nullptr || E == 0, FMA_ERR_NULL_POINTER, "grouped_gemm_gathered: row_index is NULL");
+    FMA_REQUIRE(divisor >= 1 && divisor <= 65536, FMA_ERR_BAD_SIZE,
+                "grouped_gemm_gathered: divisor must lie in [1, 65536] (got %d)", divisor);
+    FMA_REQUIRE(x_rows >= 1 || E == 0, FMA_ERR_BAD_SIZE, "grouped_gemm_gathered: x has no rows (%lld)", (long long)x_rows);
+    // the loads address x with 32-bit byte offsets below 2^31
+    FMA_REQUIRE(K <= 0 || x_rows <= ((1ll << 31) - 1) / (2 * K), FMA_ERR_UNSUPPORTED,
+                "grouped_gemm_gathered: x must be smaller than 2 GiB (%lld rows of %lld elements)", (long long)x_rows,
+                (long long)K);
+    return gemm::ragged::up_projection("grouped_gemm_gathered", x, x_rows, row_index, divisor, W, bias, out, act, M_arr, E,
+                                       N, K, swiglu, dtype, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -19,6 +19,8 @@ from .cuda_implementation import (
     combine,
     fused_router,
     fused_router_with_histogram,
+    gathered_up_projection_experts,
+    can_gather_inside_gemm,
     gather_rows,
     grouped_gemm_experts,
     up_projection_swiglu_experts,
@@ -107,6 +109,9 @@ class MoE(nn.Module):
             add_bias=add_bias,
             std=std,
         )
+
+        # None: decided per call (see _gathers_inside_gemm); True / False: always / never
+        self.gather_in_gemm: bool | None = None
 
         self.act = activation_function
         # swiglu_packed as the activation of a GLU layer is computed inside the up-projection's epilogue (a kernel for
@@ -202,6 +207,18 @@ class MoE(nn.Module):
             selected_experts, self.num_experts, token_block_histogram
         )
 
+        if self._gathers_inside_gemm(hidden_states):
+            # the first projection reads its rows x[slot // top_k] through the routing order: no grouped copy of x
+            fused = self.fuse_swiglu
+            hidden_states = gathered_up_projection_experts(
+                hidden_states, self.c_fc.weight, self.c_fc.bias, sorted_scattered_idxs, inverse, expert_frequency,
+                self.c_fc.N_array, self.c_fc.K_array, self.top_k, fused,
+            )  # fmt: skip
+            if not fused:
+                hidden_states = self.act(hidden_states)
+            hidden_states = self.c_proj.cuda_forward(input=hidden_states, expert_frequency=expert_frequency)
+            return combine(hidden_states, router_weights, inverse)
+
         # rows of every expert back to back: x[slot // top_k]
         hidden_states = gather_rows(hidden_states, sorted_scattered_idxs, inverse, self.top_k)
 
@@ -217,6 +234,18 @@ class MoE(nn.Module):
         hidden_states = combine(hidden_states, router_weights, inverse)
 
         return hidden_states
+
+    def _gathers_inside_gemm(self, hidden_states: torch.Tensor) -> bool:
+        """Whether the first projection gathers its rows itself instead of reading a grouped copy of the tokens.
+        gather_in_gemm None: when no backward will follow (which would need the grouped copy for the weight gradient
+        anyway) and the projection is narrow enough for the saved row-movement pass to outweigh the slower operand
+        fetch of scattered rows; True / False force it (True trades one more row-movement pass in the backward for not
+        keeping the grouped copy alive between forward and backward)."""
+        if self.gather_in_gemm is False or not can_gather_inside_gemm(hidden_states, self.c_fc.weight, self.c_fc.bias):
+            return False
+        if self.gather_in_gemm:
+            return True
+        return not torch.is_grad_enabled() and self.c_fc.out_features <= 6144
 
     def _get_topk(self, x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
         if self.top_k == 1:

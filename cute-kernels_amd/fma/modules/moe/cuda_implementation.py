@@ -229,6 +229,43 @@ def grouped_gemm_swiglu_cuda(
     _lib.check(rc, "grouped_gemm_swiglu_cuda")
 
 
+@custom_op(f"{LIBRARY_NAME}::grouped_gemm_gathered_cuda", mutates_args={"out", "act"})
+def grouped_gemm_gathered_cuda(
+    x: torch.Tensor,
+    row_index: torch.Tensor,
+    divisor: int,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None,
+    M_array: torch.Tensor,
+    out: torch.Tensor | None,
+    act: torch.Tensor | None,
+) -> None:
+    """The forward product of an expert projection on the rows x[row_index[i] // divisor] (i over the packed rows of all
+    experts), gathered inside the operand load. act None: out [R, N] = rows @ W^T (+ bias). Otherwise N = 2 I, act [R, I]
+    is swiglu_packed of the pre-activation, which is also written to out unless that is None (fma_grouped_gemm_gathered).
+    """
+    _lib.require_gpu(x, row_index, weight, bias, M_array, out, act)
+    E, N, K = weight.shape
+    R = row_index.numel()
+    assert x.dim() == 2 and x.size(1) == K and x.dtype == weight.dtype and x.dtype in (torch.bfloat16, torch.float16)
+    assert row_index.dtype == torch.int32 and M_array.dtype == torch.uint32 and M_array.numel() == E
+    assert out is None or (out.shape == (R, N) and out.dtype == x.dtype)
+    assert act is None or (N % 2 == 0 and act.shape == (R, N // 2) and act.dtype == x.dtype)
+    assert out is not None or act is not None
+    assert bias is None or (bias.shape == (E, N) and bias.dtype == x.dtype)
+    for t in (x, row_index, weight, bias, M_array, out, act):
+        assert t is None or t.is_contiguous()
+    if R == 0 or N == 0:
+        return
+    with torch.cuda.device(x.device):
+        rc = _lib.load().fma_grouped_gemm_gathered(
+            x.data_ptr(), x.size(0), row_index.data_ptr(), divisor, weight.data_ptr(), _lib.ptr(bias), _lib.ptr(out),
+            _lib.ptr(act), M_array.data_ptr(), E, N, K, int(act is not None), _lib.dtype_code(x.dtype),
+            _lib.current_stream(x.device),
+        )
+    _lib.check(rc, "grouped_gemm_gathered_cuda")
+
+
 @custom_op(f"{LIBRARY_NAME}::expert_bias_add_cuda", mutates_args={"y"})
 def expert_bias_add_cuda(y: torch.Tensor, bias: torch.Tensor, M_array: torch.Tensor) -> None:
     _lib.require_gpu(y, bias, M_array)
@@ -583,6 +620,98 @@ class _UpProjectionSwiglu(torch.autograd.Function):
             bias_grad = torch.empty(weight.size(0), N, device=h_grad.device, dtype=h_grad.dtype)
             expert_bias_grad_cuda(h_grad, M_array, bias_grad)
         return (x_grad, weight_grad, None, None, None, None, bias_grad)[: len(ctx.needs_input_grad)]
+
+
+class _GatheredUpProjection(torch.autograd.Function):
+    """The first expert projection on tokens instead of grouped rows: y_i = x[perm[i] // top_k] @ W_e^T (+ bias_e), with
+    swiglu_packed applied in the epilogue if `swiglu`. The rows are gathered inside the GEMM's operand load, so the
+    [T * top_k, H] buffer of grouped rows is neither written in the forward nor kept for the backward, which rebuilds it
+    (one row-movement pass) for the weight gradient and returns the gradient per token."""
+
+    @staticmethod
+    @ensure_contiguous
+    def forward(
+        ctx, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, perm: torch.Tensor, inv: torch.Tensor,
+        M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor, top_k: int, swiglu: bool, grad_enabled: bool,
+    ) -> torch.Tensor:  # fmt: skip
+        _, N, K = weight.size()
+        assert N % (16 if swiglu else 8) == 0 and K % 8 == 0
+        R = perm.numel()
+        needs_backward = grad_enabled and any(ctx.needs_input_grad[:3])
+        if swiglu:
+            h = torch.empty(R, N, device=x.device, dtype=x.dtype) if needs_backward else None
+            output = torch.empty(R, N // 2, device=x.device, dtype=x.dtype)
+            grouped_gemm_gathered_cuda(x, perm, top_k, weight, bias, M_array, h, output)
+        else:
+            h = None
+            output = torch.empty(R, N, device=x.device, dtype=x.dtype)
+            grouped_gemm_gathered_cuda(x, perm, top_k, weight, bias, M_array, output, None)
+        if needs_backward:
+            ctx.save_for_backward(x, weight, h, inv, M_array, K_array, N_array)
+        ctx.top_k = top_k
+        ctx.has_bias = bias is not None
+        return output
+
+    @staticmethod
+    @ensure_contiguous
+    def backward(ctx, output_grad: torch.Tensor) -> tuple[torch.Tensor | None]:
+        from ...ops.swiglu.cuda_implementation import swiglu_backward_cuda
+
+        x, weight, h, inv, M_array, K_array, N_array = ctx.saved_tensors
+        _, N, K = weight.size()
+        if h is not None:
+            h_grad = torch.empty_like(h)
+            up, gate = h.chunk(2, dim=-1)
+            up_grad, gate_grad = h_grad.chunk(2, dim=-1)
+            swiglu_backward_cuda(
+                gate=gate, up=up, output_grad=output_grad, gate_grad=gate_grad, up_grad=up_grad, BLOCK_SIZE=1024
+            )
+        else:
+            h_grad = output_grad
+        x_grad = weight_grad = bias_grad = None
+        if ctx.needs_input_grad[0]:
+            grouped_grad = _expert_gemm(
+                h_grad, weight, M_array, K_array, N_array, (h_grad.size(0), K), "M", 0, K, N,
+                is_A_transposed=False, is_B_transposed=False,
+            )
+            x_grad = torch.empty_like(x)
+            combine_cuda(grouped_grad, inv, None, ctx.top_k, x_grad)
+        if ctx.needs_input_grad[1]:
+            grouped = torch.empty(h_grad.size(0), K, device=x.device, dtype=x.dtype)
+            dispatch_rows_cuda(x, inv, ctx.top_k, grouped)
+            weight_grad = _expert_gemm(
+                h_grad, grouped, N_array, K_array, M_array, weight.size(), "K", N, K, 0,
+                is_A_transposed=True, is_B_transposed=False,
+            )
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            bias_grad = torch.empty(weight.size(0), N, device=h_grad.device, dtype=h_grad.dtype)
+            expert_bias_grad_cuda(h_grad, M_array, bias_grad)
+        return x_grad, weight_grad, bias_grad, None, None, None, None, None, None, None, None
+
+
+def gathered_up_projection_experts(
+    x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, perm: torch.Tensor, inv: torch.Tensor,
+    M_array: torch.Tensor, N_array: torch.Tensor, K_array: torch.Tensor, top_k: int, swiglu: bool,
+) -> torch.Tensor:  # fmt: skip
+    return _GatheredUpProjection.apply(
+        x, weight, bias, perm, inv, M_array, N_array, K_array, top_k, swiglu, torch.is_grad_enabled()
+    )
+
+
+def can_gather_inside_gemm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None) -> bool:
+    """the size and type limits of fma_grouped_gemm_gathered"""
+    _, N, K = weight.size()
+    return (
+        x.is_cuda
+        and x.dtype in (torch.bfloat16, torch.float16)
+        and weight.dtype == x.dtype
+        and (bias is None or bias.dtype == x.dtype)
+        and N % 16 == 0
+        and K % 8 == 0
+        and N < (1 << 23)
+        and K < (1 << 21)
+        and 0 < x.size(0) * K * 2 < (1 << 31)
+    )
 
 
 # ---- the reference's padded grouping interface -------------------------------------------------------

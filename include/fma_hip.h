@@ -220,6 +220,22 @@ int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_
 int fma_grouped_gemm_swiglu(const void* x, const void* W, const void* bias, void* h, void* act, const uint32_t* M_arr,
                             int64_t E, int64_t I, int64_t K, int dtype, void* stream);
 
+/* The forward product of an expert projection with the gather of the routed rows inside the operand load: for each
+ * expert e with M_e rows (packed rows i of all experts back to back, R = sum M_e)
+ *   out[i, :] = x[row_index[i] / divisor, :] * W_e[N, K]^T (+ bias_e)
+ * i.e. fma_grouped_gemm_ragged (swiglu == 0: out [R, N], act ignored) or fma_grouped_gemm_swiglu (swiglu != 0:
+ * N = 2 I, out = the pre-activation h [R, 2 I] or NULL, act [R, I]) applied to the output of
+ * fma_gather_rows(x, row_index, R, K, divisor), bit for bit, without that [R, K] buffer ever being written.
+ * x: [x_rows, K] with x_rows * K * 2 < 2^31 bytes; every row_index[i] / divisor < x_rows; divisor in [1, 65536]
+ * (top_k with row_index = the stable routing order perm of fma_moe_build_index; 1 for a plain row index).
+ * N % 8 == 0 (16 for swiglu), K % 8 == 0, N < 2^23, K < 2^21; dtype FMA_BF16 or FMA_F16.
+ * Replaces the gather inside the reference's fused Triton expert kernel (fma/modules/moe/triton_implementation/
+ * scatter_kernel.py:55-135: rows addressed through the sorted index while the product is formed) for the grouped-GEMM
+ * path, where the reference materialises them (fma/modules/moe/__init__.py:269, cuda_implementation/__init__.py:28-38). */
+int fma_grouped_gemm_gathered(const void* x, int64_t x_rows, const int32_t* row_index, int32_t divisor, const void* W,
+                              const void* bias, void* out, void* act, const uint32_t* M_arr, int64_t E, int64_t N,
+                              int64_t K, int swiglu, int dtype, void* stream);
+
 /* ---- per-expert bias ------------------------------------------------------------------------ */
 
 /* y[i, :] += bias[e, :] for every row i of expert e, rows packed expert by expert with M_arr[e] rows each (device

@@ -127,13 +127,18 @@ def test_evaluation_with_trainable_weights_does_not_store_the_preactivation(mode
     assert moe.fuse_swiglu and all(p.requires_grad for p in moe.parameters())
     x = torch.randn(300, 256, device=DEV).bfloat16()
     seen = []
-    real = ci.grouped_gemm_swiglu_cuda
+    real, real_gathered = ci.grouped_gemm_swiglu_cuda, ci.grouped_gemm_gathered_cuda
 
     def spy(x_, weight, M_array, h, act, bias=None):
         seen.append(h is not None)
         return real(x_, weight, M_array, h, act, bias)
 
+    def spy_gathered(x_, row_index, divisor, weight, bias, M_array, out, act):  # the evaluation call gathers by itself
+        seen.append(out is not None)
+        return real_gathered(x_, row_index, divisor, weight, bias, M_array, out, act)
+
     monkeypatch.setattr(ci, "grouped_gemm_swiglu_cuda", spy)
+    monkeypatch.setattr(ci, "grouped_gemm_gathered_cuda", spy_gathered)
     y_train, _ = moe(x.clone().requires_grad_(), kernel_backend=KernelBackend.cuda)
     assert seen == [True]
     with torch.no_grad() if mode == "no_grad" else torch.inference_mode():
