@@ -38,7 +38,7 @@ WORKLOADS = {
 # (FETCH_SIZE 7.5011e6 KiB, WRITE_SIZE 2.7678e6 KiB per dispatch; other pairs of runs read 6.78e6 and 7.06e6 KiB fetched) scaled by what the same counters read for a 1 GiB
 # device copy (FETCH_SIZE 0.50, WRITE_SIZE 1.00 of the true bytes); profiles/grouped_gemm_mixtral_counters.txt holds
 # the runs. Measured for the mixtral workload only; a constant from those profile runs, not measured by this script.
-MEASURED_TRAFFIC_BYTES = {"mixtral": (2 * 7.5011e6 + 2.7678e6) * 1024}
+MEASURED_TRAFFIC_BYTES = {"mixtral": (2 * 7.5383e6 + 2.7531e6) * 1024}
 TRAFFIC_SOURCE = "profiles/grouped_gemm_mixtral_counters.txt (two rocprofv3 --pmc runs of this script; not measured in this run)"
 
 
@@ -55,6 +55,9 @@ def parse_args():
                    help="1 / 0: compute SwiGLU inside / after the up-projection kernel; -1: the module's default")
     p.add_argument("--permute-experts", action="store_true",
                    help="relabel the experts by a fixed random permutation (skewed routing no longer sorted by expert id)")
+    p.add_argument("--zero-operands", action="store_true",
+                   help="diagnostic: tokens, weights and gradients all zero in the per-kernel section (same instructions, no "
+                        "bits toggling: separates the power limit on the clock from the kernels' schedule)")
     p.add_argument("--only", default="", help="comma-separated substrings: measure only the kernels whose name matches")
     p.add_argument("--no-extra-workloads", action="store_true",
                    help="skip the layer step and GEMMs of the other two benchmark shapes")
@@ -157,6 +160,23 @@ def measure_workload(name, args, full):
         torch.cuda.synchronize()
         ms_with_router = (time.perf_counter() - t1) * 1e3 / steps
 
+    # the forward alone with autograd off (evaluation / serving): with the first projection gathering its rows through the
+    # routing order, and with the grouped copy of the tokens written first (what the training step above does)
+    ms_forward = {}
+    if steps:
+        for label, gather in (("gather_in_gemm", True), ("grouped_copy", False)):
+            moe.gather_in_gemm = gather
+            with torch.no_grad():
+                for _ in range(max(1, warmup)):
+                    moe._compute_experts(x, weights_d, selected_d, KernelBackend.cuda)
+                torch.cuda.synchronize()
+                t2 = time.perf_counter()
+                for _ in range(steps):
+                    moe._compute_experts(x, weights_d, selected_d, KernelBackend.cuda)
+                torch.cuda.synchronize()
+                ms_forward[label] = (time.perf_counter() - t2) * 1e3 / steps
+        moe.gather_in_gemm = None
+
     layer = {
         "workload": f"{name}: MoE layer fwd+bwd, T={T} tokens, hidden={H}, SwiGLU intermediate={I}, "
         f"E={E}, top-k={k}, {c['kind']} routing" + (f", {c['empty']} experts empty" if c["empty"] else ""),
@@ -167,6 +187,7 @@ def measure_workload(name, args, full):
         "tokens_per_s": tokens_per_s,
         "ms_per_step_with_router": ms_with_router,
         "tokens_per_s_with_router": None if ms_with_router is None else T / (ms_with_router * 1e-3),
+        "ms_forward_no_grad": ms_forward or None,
         "layer_gemm_tflops": gemm_flops_step / (ms_per_step * 1e-3) / 1e12,
         "layer_gemm_frac_of_peak": gemm_flops_step / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
     }
@@ -195,6 +216,10 @@ def measure_workload(name, args, full):
     dw1 = torch.empty(E, 2 * I, H, **bf)
     dw2 = torch.empty(E, H, I, **bf)
     dgates = torch.empty(T, k, **bf)
+    if args.zero_operands:
+        with torch.no_grad():
+            for t in (x, w1, w2, o, dh, d_o):
+                t.zero_()
     blk = torch.randn(8192, 8192, device=dev).bfloat16()
 
     def blocker():  # ~10 ms of queued GPU work, so the host runs ahead of the GPU
@@ -251,6 +276,12 @@ def measure_workload(name, args, full):
          lambda i: ok(lib.fma_grouped_gemm_swiglu(xg.data_ptr(), w1.data_ptr(), None, None, a.data_ptr(),
                                                   counts.data_ptr(), E, I, H, BF16, stream)),
          nbytes=R * H * s + w1_b + R * I * s)
+    # the same with the gather of the routed rows inside the operand load (x read through perm; no xg), as the layer
+    # runs its forward when no backward follows; the flops are the same, the time replaces dispatch_rows + the launch above
+    mfma("up_projection_swiglu_fwd_inference_gathered(NT, rows gathered in the operand load)", 2.0 * R * 2 * I * H,
+         lambda i: ok(lib.fma_grouped_gemm_gathered(x.data_ptr(), T, perm.data_ptr(), k, w1.data_ptr(), None, None,
+                                                    a.data_ptr(), counts.data_ptr(), E, 2 * I, H, 1, BF16, stream)),
+         nbytes=T * H * s + R * 4 + w1_b + R * I * s)
     # the unfused pair the fused kernel above replaces (same bits): plain up-projection, then swiglu_forward below
     mfma("up_projection_plain_fwd(NT)", 2.0 * R * 2 * I * H, lambda i: gemm(xg, w1, h, counts, VARY_M, 0, 2 * I, H, 0, 1),
          nbytes=R * H * s + w1_b + R * 2 * I * s)
@@ -586,7 +617,7 @@ def main():
         result["kernels"] = kernels
         dominant = kernels.get("up_projection_swiglu_fwd(NT)") or next(iter(kernels.values()))
         result["roofline"] = {
-            "kernel": "grouped_gemm_kernel<NT, SwiGLU epilogue> (up-projection forward)",
+            "kernel": "ragged_gemm_kernel<NT, SwiGLU epilogue> (up-projection forward)",
             "bound": "mfma",
             "achieved": dominant["achieved"],
             "peak": PEAK_BF16_TFLOPS,
