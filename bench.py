@@ -609,6 +609,7 @@ def main():
             "router": "excluded (routing computed once, outside the timed region); ms_per_step_with_router includes it",
         },
         "ms_per_step_with_router": layer["ms_per_step_with_router"],
+        "ms_forward_no_grad": layer["ms_forward_no_grad"],
         "tokens_per_s_with_router": layer["tokens_per_s_with_router"],
         "layer_gemm_tflops": layer["layer_gemm_tflops"],
         "layer_gemm_frac_of_peak": layer["layer_gemm_frac_of_peak"],
@@ -641,7 +642,7 @@ def main():
         layer, kernels, context = measure_workload(name, args, full=False)
         del context
         entry = {key: layer[key] for key in ("workload", "ms_per_step", "tokens_per_s", "ms_per_step_with_router",
-                                             "layer_gemm_tflops", "layer_gemm_frac_of_peak")}
+                                             "ms_forward_no_grad", "layer_gemm_tflops", "layer_gemm_frac_of_peak")}
         entry["kernels"] = kernels
         result["workloads"][name] = entry
         torch.cuda.empty_cache()
