@@ -117,6 +117,18 @@ __device__ __forceinline__ float sigmoid_for(float x) {
     else return sigmoid_clamped_fast(x);
 }
 
+// SwiGLU y = up * gate * sigmoid(gate) and its gradients, in fp32, for an op whose tensors have type T
+template <typename T>
+__device__ __forceinline__ float swiglu_f(float g, float u) {
+    return u * g * sigmoid_for<T>(g);
+}
+template <typename T>
+__device__ __forceinline__ void swiglu_b(float g, float u, float dy, float& dg, float& du) {
+    const float s = sigmoid_for<T>(g);
+    dg = dy * u * (s + g * s * (1.0f - s));
+    du = dy * g * s;
+}
+
 // inclusive prefix sum across the 64 lanes of a wavefront
 template <typename T>
 __device__ __forceinline__ T wave_inclusive_scan(T v) {

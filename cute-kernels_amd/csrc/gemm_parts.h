@@ -24,6 +24,9 @@ typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 constexpr int EPI_PLAIN = 0;
 constexpr int EPI_SWIGLU = 1;      // stores the rounded pre-activation h and the activation
 constexpr int EPI_SWIGLU_ACT = 2;  // the activation only (a forward pass that no backward follows)
+// the product is the gradient of a SwiGLU activation: the gradient of the packed pre-activation h is written instead
+// (columns c and I + c of a row from column c of the product), with h read in the epilogue
+constexpr int EPI_SWIGLU_BWD = 3;
 
 // ---- the two 16-bit element types: conversions and the matrix instruction ------------------------------------------
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;

@@ -30,7 +30,10 @@ namespace ragged {
 #ifndef FMA_PF_DIST
 #define FMA_PF_DIST 4
 #endif
-constexpr uint32_t kPfDist = FMA_PF_DIST;  // K steps between a line's prefetch and the step that loads it
+constexpr uint32_t kPfDist = FMA_PF_DIST;
+#ifndef FMA_BWD_AHEAD
+#define FMA_BWD_AHEAD 2  // passes of the SwiGLU-gradient epilogue whose h values are requested ahead
+#endif  // K steps between a line's prefetch and the step that loads it
 
 constexpr int NWM = 2, NWN = 4, NW = NWM * NWN, NT = NW * 64;
 constexpr int WM = BM / NWM, WN = BN / NWN;  // 128 x 64 per wavefront
@@ -44,6 +47,7 @@ struct Args {
     uint16_t* ACT;          // swiglu only: activation output
     const uint32_t* sizes;  // E values of the varying dimension
     const uint16_t* bias;   // BIAS kernels: [E, n] added to the rounded product before anything else
+    const uint16_t* h_in;   // EPI_SWIGLU_BWD: the packed pre-activation [rows, 2 n] whose gradient goes to D
     // GATHER kernels: row i of the packed A operand is row row_index[i] / divisor of A, which has a_rows rows
     const int32_t* row_index;
     uint32_t divisor, a_rows;
@@ -74,7 +78,11 @@ __device__ unsigned long long fma_prof[1024 * 8 * 8];
 
 template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K, bool BIAS, bool GATHER>
 __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
-    static_assert(EPI == EPI_PLAIN || (A_KC && B_KC && !VARY_K), "the SwiGLU epilogue exists for the NT layout only");
+    // kGlu: a forward SwiGLU epilogue (the tile holds 128 "up" and 128 "gate" columns of the product)
+    constexpr bool kGlu = EPI == EPI_SWIGLU || EPI == EPI_SWIGLU_ACT;
+    static_assert(!kGlu || (A_KC && B_KC && !VARY_K), "the SwiGLU epilogue exists for the NT layout only");
+    static_assert(EPI != EPI_SWIGLU_BWD || (A_KC && !B_KC && !VARY_K && !BIAS && !GATHER),
+                  "the SwiGLU-gradient epilogue exists for the input-gradient (NN) layout only");
     static_assert(!BIAS || (A_KC && B_KC && !VARY_K), "the bias term exists for the forward (NT) layout only");
     static_assert(!GATHER || (A_KC && B_KC && !VARY_K), "rows are gathered in the forward (NT) layout only");
 
@@ -125,8 +133,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     auto group_k = [&](uint32_t e) { return VARY_K ? sizes[e] : args.k; };
     const uint32_t Ne = args.n;
     constexpr bool kCanNarrow = A_KC && B_KC;
-    constexpr uint32_t kTileN = EPI != EPI_PLAIN ? BN / 2 : BN;  // columns of the tile grid one tile covers
-    const uint32_t n_span = EPI != EPI_PLAIN ? Ne / 2 : Ne;      // columns the tile grid runs over
+    constexpr uint32_t kTileN = kGlu ? BN / 2 : BN;  // columns of the tile grid one tile covers
+    const uint32_t n_span = kGlu ? Ne / 2 : Ne;      // columns the tile grid runs over
     bool narrow = false;
     auto tiles_of = [&](uint32_t m) -> uint32_t {
         if (m == 0 || Ne == 0) return 0;
@@ -211,7 +219,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
 
     // first tile row of B fragment j of this wavefront
     auto b_frag_row = [&](int j) -> uint32_t {
-        if constexpr (EPI != EPI_PLAIN) {
+        if constexpr (kGlu) {
             return j < FN / 2 ? wn * (WN / 2) + j * 32 : BN / 2 + wn * (WN / 2) + (j - FN / 2) * 32;
         } else {
             return wn * WN + j * 32;
@@ -297,7 +305,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         bool fast = (Ne % 8u == 0) && (Ne < (1u << 23)) && (t.off_a % 8u == 0) && (t.off_b % 8u == 0) && (t.off_d % 8u == 0);
         if (A_KC || B_KC) fast = fast && (t.Ke % 8u == 0) && (t.Ke < (1u << 21));
         if (!A_KC) fast = fast && (t.Me % 8u == 0) && (t.Me < (1u << 23));
-        if (EPI != EPI_PLAIN) fast = fast && (n_span % 8u == 0);
+        if (kGlu) fast = fast && (n_span % 8u == 0);
         t.fast = fast;
         return t;
     };
@@ -311,7 +319,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
 
     // ---- loaders: `cur` feeds the tile being computed, `nxt` the tile after it ----
     LoaderK<NW, false> lk_a;
-    LoaderK<NW, EPI != EPI_PLAIN> lk_b;
+    LoaderK<NW, kGlu> lk_b;
     LoaderT<NW> lt_a, lt_b;
     Feed<A_KC> fa_cur{}, fa_nxt{};
     Feed<B_KC> fb_cur{}, fb_nxt{};
@@ -333,7 +341,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     auto setup_b = [&](const Tile& t, Feed<B_KC>& f, uint32_t& v) {
         const uint16_t* Be = args.B + t.off_b;
         if constexpr (B_KC) {
-            if constexpr (EPI != EPI_PLAIN) {
+            if constexpr (kGlu) {
                 // tile rows 0..127: "up" rows n0.. of the weight; rows 128..255: "gate" rows I + n0..
                 lk_b.setup(Be + (uint64_t)t.n0 * t.Ke, Be + (uint64_t)(n_span + t.n0) * t.Ke, t.n_lim - t.n0, t.Ke, wave, lane);
             } else {
@@ -435,7 +443,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         } else {
             if constexpr (B_KC) {
                 pf_bytes = fb_cur.extent;
-                if constexpr (EPI != EPI_PLAIN) {
+                if constexpr (kGlu) {
                     pf_base = (p >> 1) ? fb_cur.base1 : fb_cur.base0;
                     pf_voff = lane < 8u ? (8u * ((p & 1u) * 8u + lane) + t.pf_r) * (t.Ke * 2u) : kOutOfRange;
                 } else {
@@ -462,7 +470,9 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     constexpr int kLoads = 32 / NW;                // load instructions per wavefront, operand and K step
     constexpr uint32_t kStepLoads = 2 * kLoads;    // per wavefront and K step
     // store instructions per wavefront and tile (the epilogue issues a fixed number)
-    constexpr uint32_t kTileStores = EPI == EPI_PLAIN ? WM * WN * 2 / 1024 : (EPI == EPI_SWIGLU ? WM * WN * 2 / 1024 : 0) + WM * WN / 1024;
+    constexpr uint32_t kTileStores = EPI == EPI_PLAIN        ? WM * WN * 2 / 1024
+                                     : EPI == EPI_SWIGLU_BWD ? 2 * (WM * WN * 2 / 1024)  // two columns written per column
+                                                             : (EPI == EPI_SWIGLU ? WM * WN * 2 / 1024 : 0) + WM * WN / 1024;
 
     // loads of one K step of the CURRENT loaders' aim into `stage` (compiler-visible: placed by the scheduling hints)
     auto issue_a = [&](int stage, uint32_t k0) {
@@ -682,7 +692,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         Tile nn{};  // the tile after next
         const uint32_t tile_rows = Me - m0 < (uint32_t)BM ? Me - m0 : (uint32_t)BM;
         const uint32_t wave_rows = tile_rows > wm * WM ? tile_rows - wm * WM : 0u;
-        const bool has_columns = n0 + wn * (EPI != EPI_PLAIN ? WN / 2 : WN) < n_lim;
+        const bool has_columns = n0 + wn * (kGlu ? WN / 2 : WN) < n_lim;
         const uint32_t row_blocks = has_columns ? uniform((wave_rows + 31u) / 32u) : 0u;
         if (thin) {
             // three LDS stages in the space a tile of at most 64 rows leaves unused (grouped_gemm.hip); cold start
@@ -895,6 +905,67 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             if constexpr (BIAS) return EL::round(product) + bias_f[j][q][x];
             else return product;
         };
+        // EPI_SWIGLU_BWD: the h values of the eight passes (16 rows each) of this wavefront's sub-tile: [pass][row 0/1][up, gate]
+        u32x4 bwd_h[EPI == EPI_SWIGLU_BWD ? 2 * FM : 1][2][2];
+        // byte offset of this lane's piece of row `r` (0 or 1: rows lane / 8 and 8 + lane / 8 of the pass) from the pass's
+        // first row and the wavefront's first column, or out of range
+        auto bwd_offset = [&](int r, uint32_t cols_valid) -> uint32_t {
+            const uint32_t c16 = el & 7u;
+            const uint32_t row = (uint32_t)r * 8u + (el >> 3);
+            return c16 * 8u < cols_valid ? row * (Ne * 4u) + c16 * 16u : kOutOfRange;
+        };
+        auto bwd_rows = [&](int pass) -> uint32_t {  // rows of the pass inside the group
+            const uint32_t r0 = m0 + wm * WM + (uint32_t)pass * 16u;
+            return r0 < Me ? (Me - r0 < 16u ? Me - r0 : 16u) : 0u;
+        };
+        auto bwd_origin = [&](int pass, uint32_t col0) -> uint64_t {  // element offset of the pass's first row and column
+            return ((uint64_t)cur.row0 + m0 + wm * WM + (uint32_t)pass * 16u) * (2ull * Ne) + col0;
+        };
+        auto bwd_request = [&](int pass, uint32_t col0, uint32_t cols_valid) {
+            if constexpr (EPI == EPI_SWIGLU_BWD) {
+                const __amdgpu_buffer_rsrc_t rs = make_rsrc(args.h_in + bwd_origin(pass, col0), bwd_rows(pass) * (Ne * 4u));
+#pragma unroll
+                for (int r = 0; r < 2; ++r) {
+                    const uint32_t off = bwd_offset(r, cols_valid);
+                    bwd_h[pass][r][0] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, 0);
+                    bwd_h[pass][r][1] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, (int)(Ne * 2u), 0);
+                }
+            }
+        };
+        auto bwd_finish = [&](int pass, uint32_t col0, uint32_t cols_valid) {
+            if constexpr (EPI == EPI_SWIGLU_BWD) {
+                const uint32_t c16 = el & 7u;
+                u32x4 dy[2];
+                stage_get2_quiet(img, stage_off<WN * 2>(el >> 3, c16), stage_off<WN * 2>(8u + (el >> 3), c16), dy[0], dy[1]);
+                const __amdgpu_buffer_rsrc_t rs = make_rsrc(args.D + bwd_origin(pass, col0), bwd_rows(pass) * (Ne * 4u));
+#pragma unroll
+                for (int r = 0; r < 2; ++r) {
+                    u32x4 du, dg;
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        float gu[2], gg[2];
+#pragma unroll
+                        for (int hlf = 0; hlf < 2; ++hlf) {
+                            const int sh = hlf * 16;
+                            const float d = EL::from_bits((uint16_t)(dy[r][x] >> sh));
+                            const float u = EL::from_bits((uint16_t)(bwd_h[pass][r][0][x] >> sh));
+                            const float g = EL::from_bits((uint16_t)(bwd_h[pass][r][1][x] >> sh));
+                            swiglu_b<typename EL::act_t>(g, u, d, gg[hlf], gu[hlf]);
+                        }
+                        du[x] = EL::pack2(gu[0], gu[1]);
+                        dg[x] = EL::pack2(gg[0], gg[1]);
+                    }
+                    // The "gate" half's column offset goes into the per-lane offset, not into the instruction's scalar
+                    // offset: a 16-byte store with a scalar-register offset whose first data register the next VALU
+                    // instruction overwrites lost that dword in some lanes on this part, and the compiler leaves no wait state
+                    // there (it does for stores with a constant scalar offset, as every other store of this library has).
+                    const uint32_t off = bwd_offset(r, cols_valid);
+                    const uint32_t off_gate = off == kOutOfRange ? kOutOfRange : off + Ne * 2u;
+                    __builtin_amdgcn_raw_buffer_store_b128(du, rs, (int)off, 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(dg, rs, (int)off_gate, 0, 0);
+                }
+            }
+        };
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
             const uint32_t row0 = m0 + wm * WM + i * 32;  // first output row of this block
@@ -921,6 +992,38 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                     const uint32_t r0 = row0 + half * 16;
                     const uint32_t rows_valid = r0 < Me ? (Me - r0 < 16u ? Me - r0 : 16u) : 0u;
                     stage_flush_quiet<WN * 2, 16>(img, args.D + off_d + (uint64_t)r0 * Ne + col0, Ne, rows_valid, cols_valid, el);
+                }
+            } else if constexpr (EPI == EPI_SWIGLU_BWD) {
+                // The product (rounded) is the gradient of the activation; h and its gradient are [rows, 2 Ne] with "up" in
+                // columns 0.., "gate" in columns Ne... A pass is 16 rows x 64 columns: a lane takes 8 columns of two rows,
+                // fetches the 8 up and 8 gate values of each (requested two passes ahead), and stores both gradients.
+                const uint32_t col0 = n0 + wn * WN;
+                const uint32_t cols_valid = col0 < n_lim ? n_lim - col0 : 0u;
+                uint2 w[FN][4];
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const f32x16& c = acc[i][j];
+                        w[j][q].x = EL::pack2(c[q * 4 + 0], c[q * 4 + 1]);
+                        w[j][q].y = EL::pack2(c[q * 4 + 2], c[q * 4 + 3]);
+                    }
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    constexpr int kAhead = FMA_BWD_AHEAD;
+                    const int pass = i * 2 + half;
+                    if (pass == 0) {
+#pragma unroll
+                        for (int a = 0; a < kAhead; ++a) bwd_request(a, col0, cols_valid);
+                    }
+                    if (upper == (half == 1)) {
+#pragma unroll
+                        for (int j = 0; j < FN; ++j)
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) stage_put_quiet<WN * 2>(img, el & 15u, j * 32 + q * 8 + (el >> 5) * 4, w[j][q]);
+                    }
+                    bwd_finish(pass, col0, cols_valid);
+                    if (pass + kAhead < 2 * FM) bwd_request(pass + kAhead, col0, cols_valid);
                 }
             } else {
                 // first the rounded pre-activation (32 "up" columns | 32 "gate" columns per row), then the activation
@@ -1026,6 +1129,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, false, true, false>(const Args);     \
     template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU, false, true, false>(const Args);    \
     template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false, true, false>(const Args); \
+    template __global__ void ragged_gemm_kernel<EL, true, false, EPI_SWIGLU_BWD, false, false, false>(const Args); \
     template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, false, false, true>(const Args);     \
     template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU, false, false, true>(const Args);    \
     template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false, false, true>(const Args); \
@@ -1181,6 +1285,40 @@ int fma_grouped_gemm_swiglu(const void* x, const void* W, const void* bias, void
                             int64_t E, int64_t I, int64_t K, int dtype, void* stream) {
     return fmahip::gemm::ragged::up_projection("grouped_gemm_swiglu", x, 0, nullptr, 1, W, bias, h, act, M_arr, E, 2 * I, K,
                                                1, dtype, (hipStream_t)stream);
+}
+
+int fma_grouped_gemm_swiglu_bwd(const void* dy, const void* W, const void* h, void* dh, const uint32_t* M_arr, int64_t E,
+                                int64_t I, int64_t K, int dtype, void* stream) {
+    using namespace fmahip;
+    using namespace fmahip::gemm;
+    FMA_REQUIRE(dtype == FMA_BF16 || dtype == FMA_F16, dtype_bytes(dtype) ? FMA_ERR_UNSUPPORTED : FMA_ERR_BAD_DTYPE,
+                "grouped_gemm_swiglu_bwd: bf16 and fp16 operands are implemented (dtype code %d)", dtype);
+    FMA_REQUIRE(E >= 0, FMA_ERR_BAD_SIZE, "grouped_gemm_swiglu_bwd: negative group count %lld", (long long)E);
+    FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "grouped_gemm_swiglu_bwd: E=%lld exceeds the limit %d",
+                (long long)E, FMA_MAX_GROUPS);
+    // (with these sizes every tile takes the matrix-instruction path, the only one with this epilogue)
+    FMA_REQUIRE(I >= 8 && I % 8 == 0 && I < (1ll << 22), FMA_ERR_BAD_SIZE,
+                "grouped_gemm_swiglu_bwd: intermediate size %lld must be a positive multiple of 8 below 2^22", (long long)I);
+    FMA_REQUIRE(K >= 8 && K % 8 == 0 && K < (1ll << 21), FMA_ERR_BAD_SIZE,
+                "grouped_gemm_swiglu_bwd: K=%lld must be a positive multiple of 8 below 2^21", (long long)K);
+    if (E == 0) return FMA_OK;
+    FMA_REQUIRE(dy && W && h && dh && M_arr, FMA_ERR_NULL_POINTER, "grouped_gemm_swiglu_bwd: NULL pointer");
+    FMA_REQUIRE(aligned16(dy) && aligned16(W) && aligned16(h) && aligned16(dh), FMA_ERR_MISALIGNED,
+                "grouped_gemm_swiglu_bwd: dy, W, h and dh must be 16-byte aligned");
+    ragged::Args args{};
+    args.A = (const uint16_t*)dy;
+    args.B = (const uint16_t*)W;
+    args.D = (uint16_t*)dh;
+    args.h_in = (const uint16_t*)h;
+    args.sizes = M_arr;
+    args.E = (uint32_t)E;
+    args.m = 0;
+    args.n = (uint32_t)I;
+    args.k = (uint32_t)K;
+    args.alpha = 1.0f;
+    hipStream_t st = (hipStream_t)stream;
+    return dtype == FMA_BF16 ? ragged::launch<ElemBf16, true, false, EPI_SWIGLU_BWD, false>(args, st)
+                             : ragged::launch<ElemF16, true, false, EPI_SWIGLU_BWD, false>(args, st);
 }
 
 int fma_grouped_gemm_gathered(const void* x, int64_t x_rows, const int32_t* row_index, int32_t divisor, const void* W,

@@ -9,17 +9,7 @@ namespace {
 
 constexpr int kSwThreads = 256;
 
-template <typename T>
-__device__ __forceinline__ float swiglu_f(float g, float u) {
-    return u * g * sigmoid_for<T>(g);
-}
-
-template <typename T>
-__device__ __forceinline__ void swiglu_b(float g, float u, float dy, float& dg, float& du) {
-    const float s = sigmoid_for<T>(g);
-    dg = dy * u * (s + g * s * (1.0f - s));
-    du = dy * g * s;
-}
+// (the arithmetic itself, swiglu_f / swiglu_b, is shared with the GEMM epilogues: common.h)
 
 struct Strides2 {
     int64_t gate, up, out;

@@ -46,6 +46,7 @@ SIGNATURES = {
     "fma_swiglu_backward": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _p]),
     "fma_grouped_gemm": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _i32, _i32, _f32, _i32, _p]),
     "fma_grouped_gemm_ragged": (_i32, [_p, _p, _p, _p, _p, _i64, _i32, _i64, _i64, _i64, _i32, _i32, _f32, _i32, _p]),
+    "fma_grouped_gemm_swiglu_bwd": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "fma_grouped_gemm_gathered": (_i32, [_p, _i64, _p, _i32, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i32, _i32, _p]),
     "fma_grouped_gemm_swiglu": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "fma_expert_bias_add": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),

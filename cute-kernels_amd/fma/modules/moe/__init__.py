@@ -20,6 +20,7 @@ from .cuda_implementation import (
     fused_router,
     fused_router_with_histogram,
     gathered_up_projection_experts,
+    swiglu_experts,
     can_gather_inside_gemm,
     gather_rows,
     grouped_gemm_experts,
@@ -112,6 +113,8 @@ class MoE(nn.Module):
 
         # None: decided per call (see _gathers_inside_gemm); True / False: always / never
         self.gather_in_gemm: bool | None = None
+        # the activation's backward inside the second projection's input-gradient GEMM (see _runs_swiglu_experts_as_one_node)
+        self.fuse_swiglu_backward = True
 
         self.act = activation_function
         # swiglu_packed as the activation of a GLU layer is computed inside the up-projection's epilogue (a kernel for
@@ -222,6 +225,14 @@ class MoE(nn.Module):
         # rows of every expert back to back: x[slot // top_k]
         hidden_states = gather_rows(hidden_states, sorted_scattered_idxs, inverse, self.top_k)
 
+        if self._runs_swiglu_experts_as_one_node(hidden_states):
+            # both projections in one autograd node: its backward forms the pre-activation's gradient in one kernel
+            hidden_states = swiglu_experts(
+                hidden_states, self.c_fc.weight, self.c_fc.bias, self.c_proj.weight, self.c_proj.bias, expert_frequency,
+                self.c_fc.N_array, self.c_fc.K_array, self.c_proj.N_array, self.c_proj.K_array,
+            )  # fmt: skip
+            return combine(hidden_states, router_weights, inverse)
+
         if self.fuse_swiglu and hidden_states.dtype in (torch.bfloat16, torch.float16):
             hidden_states = self.c_fc.cuda_forward_swiglu(input=hidden_states, expert_frequency=expert_frequency)
         else:
@@ -234,6 +245,21 @@ class MoE(nn.Module):
         hidden_states = combine(hidden_states, router_weights, inverse)
 
         return hidden_states
+
+    def _runs_swiglu_experts_as_one_node(self, hidden_states: torch.Tensor) -> bool:
+        """fuse_swiglu_backward: with the fused SwiGLU up-projection, run the second projection in the same autograd node
+        so that its input gradient and the activation's backward are one kernel (16-bit types; the sizes that kernel takes)"""
+        return (
+            self.fuse_swiglu
+            and self.fuse_swiglu_backward
+            and hidden_states.dtype in (torch.bfloat16, torch.float16)
+            and self.c_proj.weight.dtype == hidden_states.dtype
+            and self.c_fc.weight.dtype == hidden_states.dtype
+            and (self.c_fc.bias is None or self.c_fc.bias.dtype == hidden_states.dtype)
+            and (self.c_proj.bias is None or self.c_proj.bias.dtype == hidden_states.dtype)
+            and self.intermediate_size < (1 << 22)
+            and self.hidden_size < (1 << 21)
+        )
 
     def _gathers_inside_gemm(self, hidden_states: torch.Tensor) -> bool:
         """Whether the first projection gathers its rows itself instead of reading a grouped copy of the tokens.

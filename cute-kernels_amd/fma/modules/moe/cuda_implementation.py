@@ -229,6 +229,31 @@ def grouped_gemm_swiglu_cuda(
     _lib.check(rc, "grouped_gemm_swiglu_cuda")
 
 
+@custom_op(f"{LIBRARY_NAME}::grouped_gemm_swiglu_bwd_cuda", mutates_args={"h_grad"})
+def grouped_gemm_swiglu_bwd_cuda(
+    output_grad: torch.Tensor, weight: torch.Tensor, h: torch.Tensor, M_array: torch.Tensor, h_grad: torch.Tensor
+) -> None:
+    """h_grad = backward of swiglu_packed at h applied to (output_grad_e @ W_e), W_e the second projection's [out, in]
+    weight: the input gradient of that projection with the activation's backward in its epilogue
+    (fma_grouped_gemm_swiglu_bwd)."""
+    _lib.require_gpu(output_grad, weight, h, M_array, h_grad)
+    E, K, inter = weight.shape
+    R = output_grad.size(0)
+    assert output_grad.shape == (R, K) and h.shape == (R, 2 * inter) and h_grad.shape == h.shape
+    assert output_grad.dtype == weight.dtype == h.dtype == h_grad.dtype and h.dtype in (torch.bfloat16, torch.float16)
+    assert M_array.dtype == torch.uint32 and M_array.numel() == E
+    for t in (output_grad, weight, h, M_array, h_grad):
+        assert t.is_contiguous()
+    if R == 0 or inter == 0:
+        return
+    with torch.cuda.device(h.device):
+        rc = _lib.load().fma_grouped_gemm_swiglu_bwd(
+            output_grad.data_ptr(), weight.data_ptr(), h.data_ptr(), h_grad.data_ptr(), M_array.data_ptr(), E, inter, K,
+            _lib.dtype_code(h.dtype), _lib.current_stream(h.device),
+        )
+    _lib.check(rc, "grouped_gemm_swiglu_bwd_cuda")
+
+
 @custom_op(f"{LIBRARY_NAME}::grouped_gemm_gathered_cuda", mutates_args={"out", "act"})
 def grouped_gemm_gathered_cuda(
     x: torch.Tensor,
@@ -620,6 +645,80 @@ class _UpProjectionSwiglu(torch.autograd.Function):
             bias_grad = torch.empty(weight.size(0), N, device=h_grad.device, dtype=h_grad.dtype)
             expert_bias_grad_cuda(h_grad, M_array, bias_grad)
         return (x_grad, weight_grad, None, None, None, None, bias_grad)[: len(ctx.needs_input_grad)]
+
+
+class _SwigluExperts(torch.autograd.Function):
+    """Both projections of a SwiGLU expert layer on grouped rows, o_e = swiglu_packed(x_e @ W1_e^T + b1_e) @ W2_e^T + b2_e,
+    as one autograd node, so that the backward can keep the activation's gradient inside the second projection's input
+    gradient: d_h comes out of one kernel (fma_grouped_gemm_swiglu_bwd) instead of a GEMM that writes d_a and an
+    element-wise pass that reads it back. Same values, bit for bit, as _UpProjectionSwiglu followed by _GroupedGemmExperts."""
+
+    @staticmethod
+    @ensure_contiguous
+    def forward(
+        ctx, x: torch.Tensor, weight1: torch.Tensor, bias1: torch.Tensor | None, weight2: torch.Tensor,
+        bias2: torch.Tensor | None, M_array: torch.Tensor, N1_array: torch.Tensor, K1_array: torch.Tensor,
+        N2_array: torch.Tensor, K2_array: torch.Tensor, grad_enabled: bool,
+    ) -> torch.Tensor:  # fmt: skip
+        _, N1, K1 = weight1.size()
+        _, N2, K2 = weight2.size()
+        assert N1 % 16 == 0 and K1 % 8 == 0 and N2 % 8 == 0 and K2 == N1 // 2
+        R = x.size(0)
+        needs_backward = grad_enabled and any(ctx.needs_input_grad[:5])
+        h = torch.empty(R, N1, device=x.device, dtype=x.dtype) if needs_backward else None
+        act = torch.empty(R, K2, device=x.device, dtype=x.dtype)
+        grouped_gemm_swiglu_cuda(x, weight1, M_array, h, act, bias1)
+        output = _expert_gemm(
+            act, weight2, M_array, N2_array, K2_array, (R, N2), "M", 0, N2, K2, is_A_transposed=False, is_B_transposed=True,
+            bias=bias2,
+        )
+        if needs_backward:
+            ctx.save_for_backward(x, weight1, weight2, h, act, M_array, N1_array, K1_array, N2_array, K2_array)
+        ctx.has_bias = (bias1 is not None, bias2 is not None)
+        return output
+
+    @staticmethod
+    @ensure_contiguous
+    def backward(ctx, output_grad: torch.Tensor) -> tuple[torch.Tensor | None]:
+        x, weight1, weight2, h, act, M_array, N1_array, K1_array, N2_array, K2_array = ctx.saved_tensors
+        _, N1, K1 = weight1.size()
+        _, N2, K2 = weight2.size()
+        x_grad = weight1_grad = bias1_grad = weight2_grad = bias2_grad = None
+        if ctx.needs_input_grad[3]:
+            weight2_grad = _expert_gemm(
+                output_grad, act, N2_array, K2_array, M_array, weight2.size(), "K", N2, K2, 0,
+                is_A_transposed=True, is_B_transposed=False,
+            )
+        if ctx.has_bias[1] and ctx.needs_input_grad[4]:
+            bias2_grad = torch.empty(weight2.size(0), N2, device=output_grad.device, dtype=output_grad.dtype)
+            expert_bias_grad_cuda(output_grad, M_array, bias2_grad)
+        if any(ctx.needs_input_grad[:3]):
+            # d_h = backward of the activation at h applied to output_grad_e @ W2_e, in the GEMM's epilogue
+            h_grad = torch.empty_like(h)
+            grouped_gemm_swiglu_bwd_cuda(output_grad, weight2, h, M_array, h_grad)
+            if ctx.needs_input_grad[0]:
+                x_grad = _expert_gemm(
+                    h_grad, weight1, M_array, K1_array, N1_array, x.size(), "M", 0, K1, N1,
+                    is_A_transposed=False, is_B_transposed=False,
+                )
+            if ctx.needs_input_grad[1]:
+                weight1_grad = _expert_gemm(
+                    h_grad, x, N1_array, K1_array, M_array, weight1.size(), "K", N1, K1, 0,
+                    is_A_transposed=True, is_B_transposed=False,
+                )
+            if ctx.has_bias[0] and ctx.needs_input_grad[2]:
+                bias1_grad = torch.empty(weight1.size(0), N1, device=h_grad.device, dtype=h_grad.dtype)
+                expert_bias_grad_cuda(h_grad, M_array, bias1_grad)
+        return x_grad, weight1_grad, bias1_grad, weight2_grad, bias2_grad, None, None, None, None, None, None
+
+
+def swiglu_experts(
+    x: torch.Tensor, weight1: torch.Tensor, bias1: torch.Tensor | None, weight2: torch.Tensor, bias2: torch.Tensor | None,
+    M_array: torch.Tensor, N1_array: torch.Tensor, K1_array: torch.Tensor, N2_array: torch.Tensor, K2_array: torch.Tensor,
+) -> torch.Tensor:  # fmt: skip
+    return _SwigluExperts.apply(
+        x, weight1, bias1, weight2, bias2, M_array, N1_array, K1_array, N2_array, K2_array, torch.is_grad_enabled()
+    )
 
 
 class _GatheredUpProjection(torch.autograd.Function):

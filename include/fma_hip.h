@@ -220,6 +220,18 @@ int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_
 int fma_grouped_gemm_swiglu(const void* x, const void* W, const void* bias, void* h, void* act, const uint32_t* M_arr,
                             int64_t E, int64_t I, int64_t K, int dtype, void* stream);
 
+/* Input gradient of the second projection with the backward of SwiGLU in its epilogue. For each expert e with M_e rows:
+ *   da_e = dy_e[M_e, K] * W_e[K, I]              (the gradient of the activation, rounded to dtype)
+ *   dh_e[:, :I] = da_e * gate * s                 dh_e[:, I:] = da_e * up * (s + gate * s * (1 - s)),  s = sigmoid(gate)
+ * with up = h_e[:, :I], gate = h_e[:, I:] of the packed pre-activation h [R, 2I]: what fma_grouped_gemm_ragged (rows vary,
+ * trans_a = 0, trans_b = 0, N = I) followed by fma_swiglu_backward on the two halves of h gives, bit for bit, without da
+ * ever being written. W: [E, K, I] row-major (the second projection's weight [E, out = K, in = I]); dh: [R, 2I].
+ * I % 8 == 0, K % 8 == 0, I < 2^22, K < 2^21; dtype FMA_BF16 or FMA_F16.
+ * Fuses _GroupedGemmExperts.backward (fma/modules/moe/cuda_implementation/__init__.py:40-60, the x_grad product) with the
+ * backward of swiglu_packed (fma/ops/swiglu/__init__.py:133-164; cuda_implementation/backward.cu:79-129). */
+int fma_grouped_gemm_swiglu_bwd(const void* dy, const void* W, const void* h, void* dh, const uint32_t* M_arr, int64_t E,
+                                int64_t I, int64_t K, int dtype, void* stream);
+
 /* The forward product of an expert projection with the gather of the routed rows inside the operand load: for each
  * expert e with M_e rows (packed rows i of all experts back to back, R = sum M_e)
  *   out[i, :] = x[row_index[i] / divisor, :] * W_e[N, K]^T (+ bias_e)
