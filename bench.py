@@ -289,6 +289,14 @@ def measure_workload(name, args, full):
          nbytes=R * I * s + w2_b + R * H * s)
     mfma("down_projection_dgrad(NN)", 2.0 * R * I * H, lambda i: gemm(d_o, w2, da, counts, VARY_M, 0, I, H, 0, 0),
          nbytes=R * H * s + w2_b + R * I * s)
+    # the same product with the backward of SwiGLU in its epilogue (h read, the gradient of h written instead of the
+    # gradient of the activation): what the layer's backward runs; it replaces the launch above plus swiglu_backward
+    dh_f = torch.empty(R, 2 * I, **bf)
+    mfma("down_projection_dgrad_swiglu_bwd(NN + SwiGLU backward)", 2.0 * R * I * H,
+         lambda i: ok(lib.fma_grouped_gemm_swiglu_bwd(d_o.data_ptr(), w2.data_ptr(), h.data_ptr(), dh_f.data_ptr(),
+                                                      counts.data_ptr(), E, I, H, BF16, stream)),
+         nbytes=R * H * s + w2_b + 2 * R * 2 * I * s)
+    del dh_f
     mfma("down_projection_wgrad(TN)", 2.0 * R * I * H, lambda i: gemm(d_o, a, dw2, counts, VARY_K, H, I, 0, 1, 0),
          nbytes=R * H * s + R * I * s + w2_b)
     mfma("up_projection_dgrad(NN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, w1, dxg, counts, VARY_M, 0, H, 2 * I, 0, 0),
