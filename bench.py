@@ -538,7 +538,7 @@ def cpu_baseline(context, name):
             progress(f"step {n}, {time.perf_counter() - t0:.1f} s")
         return (time.perf_counter() - t0) / n, n
 
-    # As BASELINE.md describes it: bf16 on the first T/16 tokens, as long as that fits the time box (about 30 s of CPU
+    # bf16 on the first T/16 tokens, as long as that fits the time box (about 30 s of CPU
     # work). A first bf16 step on T/64 tokens sizes it: if four times its duration is beyond the box the sample stays at
     # T/64 tokens, and if the host's bf16 kernels are so slow that even that step takes more than 10 s the leg runs in fp32.
     note = ""

@@ -71,10 +71,6 @@ struct Feed {
     uint32_t col_bytes;     // [k][out] tile: byte offset of the tile's first column inside a row
 };
 
-#ifdef FMA_PROF
-__device__ unsigned long long fma_prof[1024 * 8 * 8];
-#define PROF_STAMP(t) asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t))
-#endif
 
 template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K, bool BIAS, bool GATHER>
 __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
@@ -515,10 +511,6 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         else lt_b.issue_quiet(stage ? s_b1 : s_b0, k0);
     };
 
-#ifdef FMA_PROF
-    uint64_t p_start, p_t0 = 0, p_t1 = 0, p_seg[6] = {0, 0, 0, 0, 0, 0}, p_tiles = 0;
-    PROF_STAMP(p_start);
-#endif
     Tile cur = lookup(0), nxt = lookup(1);
     // GATHER: the second tile's rows (the first tile fetches its own in its cold start; from then on every tile
     // fetches those of the tile after next, before its epilogue)
@@ -779,11 +771,6 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             }
             issue_bias();
             issue_prefetch(kPfDist - 1);
-#ifdef FMA_PROF
-            PROF_STAMP(p_t1);
-            if (p_t0) p_seg[3] += p_t1 - p_t0;  // tile top: set-ups, accumulators cleared
-            p_t0 = p_t1;
-#endif
             using SrcCur = std::integral_constant<int, 0>;
             using SrcNext = std::integral_constant<int, 1>;
             using SrcEither = std::integral_constant<int, 2>;
@@ -792,11 +779,6 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 load_frags(fa_c, 0, 0, 0);
                 step(fa_c, WaitFirst{}, SrcEither{}, 0, 0);
                 step(fa_c, WaitStep{}, SrcEither{}, 1, 1);
-#ifdef FMA_PROF
-                PROF_STAMP(p_t1);
-                p_seg[4] += p_t1 - p_t0;  // the first two K steps
-                p_t0 = p_t1;
-#endif
                 if constexpr (FA == FM) {
                     // full tiles: the steps in the middle load from the current tile and the last two from the next, each
                     // with the loaders aimed once, so that the loop body carries no selects
@@ -836,13 +818,6 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             }
         }
 
-#ifdef FMA_PROF
-        PROF_STAMP(p_t1);
-        p_seg[0] += p_t1 - p_t0;  // rest of the K loop
-        p_t0 = p_t1;
-        p_seg[5] += KT2 > 2 ? KT2 - 2 : 0;
-        ++p_tiles;
-#endif
         if (BIAS && KT == 0) {  // a group without reduction: the result is the bias
             issue_bias();
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, false));
@@ -852,11 +827,6 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         // GATHER: its rows go where this tile's were (no load of this tile is left to be issued). The load is older than
         // this tile's stores, so the first wait of the next tile covers it.
         g_issue_table(nn, round & 1u);
-#ifdef FMA_PROF
-        PROF_STAMP(p_t1);
-        p_seg[1] += p_t1 - p_t0;  // look-up
-        p_t0 = p_t1;
-#endif
 
         // ---- epilogue: through this wavefront's 2 KB of the staging buffer, 16 rows of 128 bytes at a time ----
         // A lane holds row (lane & 31), columns q*8 + (lane >> 5)*4 + 0..3 of each 32x32 accumulator block.
@@ -1081,11 +1051,6 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             }
         }
 
-#ifdef FMA_PROF
-        PROF_STAMP(p_t1);
-        p_seg[2] += p_t1 - p_t0;  // epilogue
-        p_t0 = p_t1;
-#endif
         // ---- on to the next tile ----
         streamed = stream_next;
         if (stream_next) {
@@ -1100,18 +1065,6 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         nxt = nn;
         ++round;
     }
-#ifdef FMA_PROF
-    {
-        uint64_t t;
-        PROF_STAMP(t);
-        if (lane == 0) {
-            unsigned long long* o = fma_prof + ((size_t)blockIdx.x * 8 + wave) * 8;
-            for (int i = 0; i < 6; ++i) o[i] = p_seg[i];
-            o[6] = p_tiles;
-            o[7] = t - p_start;
-        }
-    }
-#endif
 }
 
 // every instantiation the entry points launch (explicit, so that host stub and device code are both emitted)
@@ -1221,11 +1174,6 @@ int up_projection(const char* who, const void* x, int64_t x_rows, const int32_t*
 
 extern "C" {
 
-#ifdef FMA_PROF
-int fma_debug_prof(void* host, int64_t bytes) {
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(fmahip::gemm::ragged::fma_prof), (size_t)bytes, 0, hipMemcpyDeviceToHost);
-}
-#endif
 
 int fma_grouped_gemm_ragged(const void* A, const void* B, void* D, const uint32_t* sizes, const void* bias, int64_t E,
                             int vary, int64_t M, int64_t N, int64_t K, int trans_a, int trans_b, float alpha, int dtype,
