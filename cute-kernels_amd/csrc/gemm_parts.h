@@ -247,9 +247,10 @@ __device__ __forceinline__ void stage_get2_quiet(uint32_t image, uint32_t off0, 
                  : "memory");
 }
 // stage_flush for images of exactly two store instructions (ROWS * ROWB == 2048)
+// stream (the same in every lane): store with the non-temporal hint
 template <int ROWB, int ROWS>
 __device__ __forceinline__ void stage_flush_quiet(uint32_t image, uint16_t* origin, uint32_t ld, uint32_t rows_valid,
-                                                  uint32_t cols_valid, uint32_t lane) {
+                                                  uint32_t cols_valid, uint32_t lane, bool stream = false) {
     constexpr uint32_t kChunks = ROWB / 16;
     constexpr uint32_t kRowsPerInst = 64 / kChunks;
     static_assert(ROWS == 2 * kRowsPerInst, "two store instructions per image");
@@ -260,8 +261,14 @@ __device__ __forceinline__ void stage_flush_quiet(uint32_t image, uint16_t* orig
     const uint32_t r0 = lane / kChunks, r1 = kRowsPerInst + lane / kChunks;
     u32x4 v0, v1;
     stage_get2_quiet(image, stage_off<ROWB>(r0, c16), stage_off<ROWB>(r1, c16), v0, v1);
-    store_tile16<false>(rsrc, col_ok ? r0 * ldb + c16 * 16u : kOutOfRange, __builtin_bit_cast(uint4, v0));
-    store_tile16<false>(rsrc, col_ok ? r1 * ldb + c16 * 16u : kOutOfRange, __builtin_bit_cast(uint4, v1));
+    const uint32_t off0 = col_ok ? r0 * ldb + c16 * 16u : kOutOfRange, off1 = col_ok ? r1 * ldb + c16 * 16u : kOutOfRange;
+    if (stream) {
+        store_tile16<true>(rsrc, off0, __builtin_bit_cast(uint4, v0));
+        store_tile16<true>(rsrc, off1, __builtin_bit_cast(uint4, v1));
+    } else {
+        store_tile16<false>(rsrc, off0, __builtin_bit_cast(uint4, v0));
+        store_tile16<false>(rsrc, off1, __builtin_bit_cast(uint4, v1));
+    }
 }
 template <int ROWB, int ROWS, int HALF>
 __device__ __forceinline__ void stage_flush_split_quiet(uint32_t image, uint16_t* origin, uint32_t ld, uint32_t rows_valid,

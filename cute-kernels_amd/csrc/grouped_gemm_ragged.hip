@@ -31,6 +31,9 @@ namespace ragged {
 #define FMA_PF_DIST 4
 #endif
 constexpr uint32_t kPfDist = FMA_PF_DIST;
+#ifndef FMA_STREAM_OUT_ALL_LAYOUTS
+#define FMA_STREAM_OUT_ALL_LAYOUTS 0
+#endif
 #ifndef FMA_BWD_AHEAD
 #define FMA_BWD_AHEAD 2  // passes of the SwiGLU-gradient epilogue whose h values are requested ahead
 #endif  // K steps between a line's prefetch and the step that loads it
@@ -843,6 +846,12 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 for (int j = 0; j < FN; ++j) acc[i][j] *= alpha;
         }
         const bool upper = ((el >> 4) & 1u) != 0;  // this lane's row lies in the second 16 rows of its 32-row block
+#ifndef FMA_STREAM_OUT_STEPS
+#define FMA_STREAM_OUT_STEPS 16
+#endif
+        // Tiles with a short reduction write much per flop (a weight gradient over ~500 rows: 8 K steps per 128 KB tile):
+        // their stores carry the non-temporal hint (+4 to 5 % there); for long reductions plain stores are faster by 0 to 1 %
+        const bool stream_out = FMA_STREAM_OUT_ALL_LAYOUTS ? KT <= FMA_STREAM_OUT_STEPS : (VARY_K && KT <= FMA_STREAM_OUT_STEPS);
         // BIAS: the eight groups of four columns this lane holds of every row block: [j][q], as fp32
         float bias_f[FN][4][4];
         if constexpr (BIAS) {
@@ -961,7 +970,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                     }
                     const uint32_t r0 = row0 + half * 16;
                     const uint32_t rows_valid = r0 < Me ? (Me - r0 < 16u ? Me - r0 : 16u) : 0u;
-                    stage_flush_quiet<WN * 2, 16>(img, args.D + off_d + (uint64_t)r0 * Ne + col0, Ne, rows_valid, cols_valid, el);
+                    stage_flush_quiet<WN * 2, 16>(img, args.D + off_d + (uint64_t)r0 * Ne + col0, Ne, rows_valid, cols_valid, el,
+                                                  stream_out);
                 }
             } else if constexpr (EPI == EPI_SWIGLU_BWD) {
                 // The product (rounded) is the gradient of the activation; h and its gradient are [rows, 2 Ne] with "up" in
