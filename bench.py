@@ -333,7 +333,14 @@ def measure_workload(name, args, full):
         src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()
         dst = torch.empty_like(src)
         hbm("hbm_copy_1GiB", 2 * src.numel() * s, lambda i: dst.copy_(src), n=30)
-        del src, dst
+        # what streams of other read : write mixes reach on this part with the runtime's own kernels, for reference beside
+        # the row kernels: write only (a fill), and one read for two writes (the mix of gather / dispatch
+        # at top-k 2: every input row goes to two output rows)
+        hbm("hbm_write_1GiB(fill)", dst.numel() * s, lambda i: dst.fill_(1.0), n=30)
+        half = src[: src.numel() // 2]
+        hbm("hbm_1read_2writes_1.5GiB(expanded copy)", 3 * half.numel() * s,
+            lambda i: dst.view(2, -1).copy_(half.unsqueeze(0).expand(2, -1)), n=30)
+        del src, dst, half
 
     # Row kernels: algorithmic bytes = each distinct input row once + each output row once + index / gate words.
     # Inputs and outputs rotate over several buffer sets whose footprint together exceeds 1 GiB (four times the
