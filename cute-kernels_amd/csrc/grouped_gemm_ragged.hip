@@ -665,7 +665,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             }
         };
         // waits of a step: all but the newest load when that is the previous step's prefetch; in a tile's first step the
-        // stores of the previous epilogue (or the cold start's stand-ins) and the two loads of the bias tile are newer
+        // stores of the previous epilogue (or the cold start's stand-ins) and the one load of the bias values are newer
         // than the loads waited for as well
         using WaitStep = std::integral_constant<int, waitcnt_imm(kPrefetch ? 1 : 0, true)>;
         using WaitFirst = std::integral_constant<int, waitcnt_imm((int)kTileStores + (kPrefetch ? 1 : 0) + (BIAS ? 1 : 0), true)>;
