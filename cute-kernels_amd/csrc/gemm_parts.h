@@ -12,6 +12,7 @@ namespace gemm {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
@@ -44,6 +45,11 @@ struct ElemBf16 {
     static __device__ __forceinline__ f32x16 mfma(frag a, frag b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
+    // 16x16 block over 32 k: at the same arithmetic rate the part sustains a higher clock on this shape (measured on
+    // N(0,1) operands, matrix instructions only: 0.79 against 0.70 of the peak rate)
+    static __device__ __forceinline__ f32x4 mfma16(frag a, frag b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
 };
 
 struct ElemF16 {
@@ -58,6 +64,9 @@ struct ElemF16 {
     static __device__ __forceinline__ f32x16 mfma(frag a, frag b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
+    static __device__ __forceinline__ f32x4 mfma16(frag a, frag b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
 };
 
 // ---- direct global -> LDS loaders ---------------------------------------------------------------------------------
@@ -69,6 +78,13 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const uint16_t* p, u
     // stride 0 (raw buffer), 32-bit data format
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, (int)bytes, 0x00020000);
 }
+// States that a value is the same in every lane (a no-op for a value the compiler already keeps in scalar registers).
+// The assembly below needs its scalar operands in scalar registers whatever the compiler has decided about the
+// computation that feeds them.
+__device__ __forceinline__ uint32_t uniform(uint32_t x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ u32x4 uniform(u32x4 x) {
+    return u32x4{uniform(x[0]), uniform(x[1]), uniform(x[2]), uniform(x[3])};
+}
 // The same load written in assembly, with its M0 set-up (M0 holds the LDS address the wavefront's 1 KB goes to). The
 // compiler does not see that it writes LDS, so it places no waits of its own for it: the first loads of a tile are
 // issued this way, partly while the previous tile's epilogue is still running, and waited for with an exact count.
@@ -78,7 +94,7 @@ __device__ __forceinline__ void buffer_load_lds_quiet(u32x4 rsrc, uint32_t voff,
     asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
                  "s_mov_b32 m0, %0"
                  : "=&s"(saved_m0)
-                 : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr));
+                 : "v"(voff), "s"(uniform(rsrc)), "s"(uniform(soff)), "s"(uniform(lds_addr)));
 }
 // the 4-byte form of the same load (64 lanes x 4 bytes = 256 bytes of LDS per instruction)
 __device__ __forceinline__ void buffer_load_lds_quiet_b32(u32x4 rsrc, uint32_t voff, uint32_t soff, uint32_t lds_addr) {
@@ -86,7 +102,7 @@ __device__ __forceinline__ void buffer_load_lds_quiet_b32(u32x4 rsrc, uint32_t v
     asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %4\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds\n\t"
                  "s_mov_b32 m0, %0"
                  : "=&s"(saved_m0)
-                 : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_addr));
+                 : "v"(voff), "s"(uniform(rsrc)), "s"(uniform(soff)), "s"(uniform(lds_addr)));
 }
 // LDS words at addr, addr + 256, addr + 512 and addr + 768 bytes, read in assembly and waited for here: for a table that
 // only direct-to-LDS loads written in assembly fill, which the compiler therefore knows nothing about
@@ -119,7 +135,6 @@ __device__ __forceinline__ u32x4 make_rsrc_words(const uint16_t* p, uint32_t byt
     r.w = 0x00020000u;
     return r;
 }
-__device__ __forceinline__ uint32_t uniform(uint32_t x) { return __builtin_amdgcn_readfirstlane(x); }
 __device__ __forceinline__ uint64_t uniform(uint64_t x) {
     return ((uint64_t)uniform((uint32_t)(x >> 32)) << 32) | uniform((uint32_t)x);
 }
@@ -129,8 +144,8 @@ constexpr uint32_t kOutOfRange = 0x80000000u;  // lane offset no descriptor of t
 __device__ __forceinline__ s16x8 read_kc_frag(const uint8_t* p) { return *reinterpret_cast<const s16x8*>(p); }
 
 // ---- epilogue staging: a wavefront transposes its accumulator sub-tile, half at a time, through 8 KB of LDS ----
-// The MFMA leaves a lane with 4 consecutive columns of one row per 32x32 block, so storing straight from registers
-// writes 8-byte pieces of 32 different rows per instruction. Staged through LDS as rows of ROWB bytes, every store
+// The MFMA leaves a lane with 4 consecutive columns of one row per accumulator block, so storing straight from registers
+// writes 8-byte pieces of 16 or 32 different rows per instruction. Staged through LDS as rows of ROWB bytes, every store
 // instruction writes 16 bytes per lane and whole 64- or 128-byte row segments.
 // Row m, 16-byte chunk c of the image sits at m*ROWB + ((c ^ key(m)) << 4), key(m) = (m / rows-per-256-B) mod chunks:
 // the 8-byte writes of 32 consecutive rows conflict at most two ways, the 16-byte reads not at all.
@@ -227,17 +242,16 @@ __device__ __forceinline__ void stage_put_quiet(uint32_t image, uint32_t m, uint
     const uint32_t addr = image + stage_off<ROWB>(m, col >> 3) + ((col >> 2) & 1u) * 8u;
     asm volatile("ds_write_b64 %0, %1" ::"v"(addr), "v"(__builtin_bit_cast(uint64_t, v)) : "memory");
 }
-// eight 8-byte reads at LDS byte addresses a[0..7], complete on return (written in assembly for the same reason)
-__device__ __forceinline__ void lds_read8x8_quiet(const uint32_t (&a)[8], uint2 (&v)[8]) {
-    uint64_t r[8];
-    asm volatile("ds_read_b64 %0, %8\n\tds_read_b64 %1, %9\n\tds_read_b64 %2, %10\n\tds_read_b64 %3, %11\n\t"
-                 "ds_read_b64 %4, %12\n\tds_read_b64 %5, %13\n\tds_read_b64 %6, %14\n\tds_read_b64 %7, %15\n\t"
+// four 8-byte reads at LDS byte addresses a[0..3], complete on return (written in assembly for the same reason)
+__device__ __forceinline__ void lds_read4x8_quiet(const uint32_t (&a)[4], uint2 (&v)[4]) {
+    uint64_t r[4];
+    asm volatile("ds_read_b64 %0, %4\n\tds_read_b64 %1, %5\n\tds_read_b64 %2, %6\n\tds_read_b64 %3, %7\n\t"
                  "s_waitcnt lgkmcnt(0)"
-                 : "=&v"(r[0]), "=&v"(r[1]), "=&v"(r[2]), "=&v"(r[3]), "=&v"(r[4]), "=&v"(r[5]), "=&v"(r[6]), "=&v"(r[7])
-                 : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(a[4]), "v"(a[5]), "v"(a[6]), "v"(a[7])
+                 : "=&v"(r[0]), "=&v"(r[1]), "=&v"(r[2]), "=&v"(r[3])
+                 : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3])
                  : "memory");
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = __builtin_bit_cast(uint2, r[i]);
+    for (int i = 0; i < 4; ++i) v[i] = __builtin_bit_cast(uint2, r[i]);
 }
 // two 16-byte reads of the image (at byte offsets off0 and off1), complete on return
 __device__ __forceinline__ void stage_get2_quiet(uint32_t image, uint32_t off0, uint32_t off1, u32x4& v0, u32x4& v1) {
@@ -315,6 +329,17 @@ __device__ __forceinline__ uint32_t mc_frag_off(uint32_t r0, uint32_t lane) {
     const uint32_t q = j & 3u, kr = j >> 2;
     const uint32_t chunk = (r0 >> 3) + 2u * (g & 1u) + (q >> 1);
     return (8u * (g >> 1) + kr) * kTRowBytes + ((chunk ^ (4u * kr)) << 4) + (q & 1u) * 8u;
+}
+// The same for fragments of the 16x16x32 instruction (16 out rows, a lane holds 8 consecutive k of one row, lanes
+// 16g.. the g-th eight of the slice's 32 k): the fragment that starts at out row r0 (a multiple of 16), k slice 0 of two.
+// Slice 1 adds 32 rows, the second read of a fragment (k + 4) adds 4 rows. For a tile written by LoaderT<NW, true>: the
+// chunk position is also flipped by bit 3 of the k row, which keeps the reads of lanes 16..31 (k rows 8..15) off the
+// banks of lanes 0..15.
+__device__ __forceinline__ uint32_t mc_frag_off16(uint32_t r0, uint32_t lane) {
+    const uint32_t g = lane >> 4, j = lane & 15u;
+    const uint32_t q = j & 3u, kr = j >> 2;
+    const uint32_t chunk = (r0 >> 3) + (q >> 1);
+    return (8u * g + kr) * kTRowBytes + ((chunk ^ (4u * kr) ^ (2u * (g & 1u))) << 4) + (q & 1u) * 8u;
 }
 
 // Operand with the reduction dimension contiguous: tile [256 rows][64 k]. A wavefront instruction moves 8 physical rows
@@ -403,7 +428,8 @@ struct LoaderK {
 // Operand stored [reduction][out] (out contiguous): tile [64 k][256 out]. A wavefront instruction moves two k rows
 // (2 x 512 B). Rows past the end of the reduction are out of the descriptor's range (zeros); columns past the end of
 // the operand's rows read whatever follows, which only reaches outputs that are never stored.
-template <int NW>
+// SWZ16: the chunk positions that mc_frag_off16 reads (otherwise those of mc_frag_off).
+template <int NW, bool SWZ16 = false>
 struct LoaderT {
     static constexpr int NI = 32 / NW;
     const uint16_t* base;  // row 0 of the group's operand, first column of the tile
@@ -422,7 +448,10 @@ struct LoaderT {
         wave = wave_;
         const uint32_t khalf = lane >> 5;  // which of the two rows of an instruction this lane loads
         const uint32_t krow = wave_ * 2u + khalf;
-        voff = khalf * ldb + (((lane & 31u) ^ (4u * (krow & 3u))) << 4);
+        static_assert(!SWZ16 || NW == 8, "bit 3 of a lane's k row must be the same for every instruction");
+        // (an instruction's rows are 16 i + krow: bit 3 of the k row is bit 3 of krow for every instruction i)
+        const uint32_t flip = 4u * (krow & 3u) ^ (SWZ16 ? 2u * ((krow >> 3) & 1u) : 0u);
+        voff = khalf * ldb + (((lane & 31u) ^ flip) << 4);
     }
 
     __device__ __forceinline__ void issue(uint8_t* tile, uint32_t k0) const { issue_range<0, NI>(tile, k0); }

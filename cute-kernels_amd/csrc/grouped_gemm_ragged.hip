@@ -1,9 +1,14 @@
 // Grouped GEMM for launches whose groups differ in ONE dimension (every grouped GEMM of an MoE layer: rows per expert
 // in forward and input gradient, reduction length per expert in the weight gradient) for gfx950: bf16 or fp16 operands,
 // fp32 accumulation on the matrix cores, optional SwiGLU epilogue. The tile kernel of grouped_gemm.hip (256x256x64
-// tiles, eight wavefronts, two LDS stages filled by direct global -> LDS loads, the same LDS layouts and K loop) with a
-// different tile boundary:
+// tiles, eight wavefronts, two LDS stages filled by direct global -> LDS loads, the same LDS layouts) with another
+// matrix instruction and a different tile boundary:
 //
+//  * The products are 16x16x32 instructions (v_mfma_f32_16x16x32), not 32x32x16: the same arithmetic rate per
+//    instruction cycle, but the part holds a higher clock on them. Measured on N(0,1) operands: a loop of nothing but
+//    matrix instructions sustains 0.79 of the peak rate against 0.70, and this kernel ran 3.5 to 6 % faster on the
+//    Mixtral-shape layer's GEMMs than the same kernel on 32x32x16. A wavefront's 128 x 64 sub-tile is 8 x 4 blocks; a K
+//    step is two 32-wide slices, each worked through in four phases of two row blocks (see the K loop).
 //  * With two dimensions known on the host, a group's operand offsets follow from one 32-bit prefix of the varying
 //    dimension, so the group table takes 10 bytes per group instead of 30. The LDS that frees (16 KB) is a staging
 //    buffer of its own for the epilogue, which therefore no longer needs a piece of an operand stage.
@@ -40,7 +45,7 @@ constexpr uint32_t kPfDist = FMA_PF_DIST;
 
 constexpr int NWM = 2, NWN = 4, NW = NWM * NWN, NT = NW * 64;
 constexpr int WM = BM / NWM, WN = BN / NWN;  // 128 x 64 per wavefront
-constexpr int FM = WM / 32, FN = WN / 32;    // 4 x 2 accumulator blocks of 32 x 32
+constexpr int RB = WM / 16, CB = WN / 16;    // 8 x 4 accumulator blocks of 16 x 16 (the 16x16x32 matrix instruction)
 constexpr int kStageBytes = 2048;            // epilogue staging per wavefront: 16 rows of 128 bytes or 32 rows of 64
 
 struct Args {
@@ -74,6 +79,9 @@ struct Feed {
     uint32_t col_bytes;     // [k][out] tile: byte offset of the tile's first column inside a row
 };
 
+
+// Names an accumulator value as one 16-register value (no instruction, no ordering).
+__device__ __forceinline__ void anchor_value(f32x16& c) { asm("" : "+v"(c)); }
 
 template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K, bool BIAS, bool GATHER>
 __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
@@ -216,29 +224,31 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     __syncthreads();
     const uint32_t total_tiles = s_tile_start[E];
 
-    // first tile row of B fragment j of this wavefront
+    // first tile row of B fragment j (16 rows) of this wavefront
     auto b_frag_row = [&](int j) -> uint32_t {
         if constexpr (kGlu) {
-            return j < FN / 2 ? wn * (WN / 2) + j * 32 : BN / 2 + wn * (WN / 2) + (j - FN / 2) * 32;
+            return j < CB / 2 ? wn * (WN / 2) + j * 16 : BN / 2 + wn * (WN / 2) + (j - CB / 2) * 16;
         } else {
-            return wn * WN + j * 32;
+            return wn * WN + j * 16;
         }
     };
-    // per-lane LDS byte offsets of this wavefront's fragments for k slice 0 (slice ks adds a constant)
-    uint32_t a_off[FM], b_off[FN];
+    // per-lane LDS byte offsets of this wavefront's fragments for k slice 0 of the two 32-wide slices of a K step
+    // (slice 1 adds a constant). A fragment is 16 rows: lane l holds row l % 16, k 8 (l / 16) .. + 7 of the slice.
+    uint32_t a_off[RB], b_off[CB];
 #pragma unroll
-    for (int i = 0; i < FM; ++i) {
-        const uint32_t r0 = wm * WM + i * 32;
-        a_off[i] = A_KC ? r0 * kRowBytes : mc_frag_off(r0, lane);
+    for (int i = 0; i < RB; ++i) {
+        const uint32_t r0 = wm * WM + i * 16;
+        a_off[i] = A_KC ? r0 * kRowBytes : mc_frag_off16(r0, lane);
     }
 #pragma unroll
-    for (int j = 0; j < FN; ++j) {
+    for (int j = 0; j < CB; ++j) {
         const uint32_t r0 = b_frag_row(j);
-        b_off[j] = B_KC ? r0 * kRowBytes : mc_frag_off(r0, lane);
+        b_off[j] = B_KC ? r0 * kRowBytes : mc_frag_off16(r0, lane);
     }
-    uint32_t kc_slice[4];
+    uint32_t kc_slice[2];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) kc_slice[ks] = kc_off(lane & 31u, (uint32_t)ks * 2u + (lane >> 5));
+    for (int ks = 0; ks < 2; ++ks) kc_slice[ks] = kc_off(lane & 15u, (uint32_t)ks * 4u + (lane >> 4));
+    constexpr uint32_t kSliceT = 32 * kTRowBytes;  // from slice 0 to slice 1 in a [k][out] tile
 
     // workgroup id -> position in the round of gridDim.x tiles: workgroups of one XCD take 32 neighbours
     const uint32_t grid = gridDim.x;
@@ -319,7 +329,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     // ---- loaders: `cur` feeds the tile being computed, `nxt` the tile after it ----
     LoaderK<NW, false> lk_a;
     LoaderK<NW, kGlu> lk_b;
-    LoaderT<NW> lt_a, lt_b;
+    LoaderT<NW, true> lt_a, lt_b;
     Feed<A_KC> fa_cur{}, fa_nxt{};
     Feed<B_KC> fb_cur{}, fb_nxt{};
     uint32_t va_cur = 0, va_nxt = 0, vb_cur = 0, vb_nxt = 0;  // the loaders' per-lane offsets (they depend on the pitch)
@@ -569,41 +579,63 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         aim_a(fa_cur, va_cur);
         aim_b(fb_cur, vb_cur);
 
-        f32x16 acc[FM][FN];
+        // The CB column blocks of a row block are one 16-register value (block j in elements 4 j ..), and every K step ends
+        // by naming these values as such (anchor_acc): that keeps a matrix instruction's result in the register quadruple its
+        // addend came from. As 32 separate quadruples the results wander through the register file, which the allocator
+        // could not fit without spilling.
+        f32x16 acc[RB];
 #pragma unroll
-        for (int i = 0; i < FM; ++i)
+        for (int i = 0; i < RB; ++i)
 #pragma unroll
-            for (int j = 0; j < FN; ++j)
-#pragma unroll
-                for (int x = 0; x < 16; ++x) acc[i][j][x] = 0.0f;
+            for (int x = 0; x < 16; ++x) acc[i][x] = 0.0f;
+        auto mfma_block = [&](f32x16& c, int j, typename EL::frag b, typename EL::frag a) __attribute__((always_inline)) {
+            f32x4 q = {c[4 * j], c[4 * j + 1], c[4 * j + 2], c[4 * j + 3]};
+            q = EL::mfma16(b, a, q);
+            c[4 * j] = q[0];
+            c[4 * j + 1] = q[1];
+            c[4 * j + 2] = q[2];
+            c[4 * j + 3] = q[3];
+            anchor_value(c);
+        };
 
-        // MFMA operand fragments of one 16-wide k slice, double buffered in registers. The K loop exists in four
-        // versions, for wavefronts whose first FA = 4, 2, 1 or 0 row blocks (of 32 rows) hold rows of the group.
-        typename EL::frag fa[2][FM], fb[2][FN];
-        auto load_frags = [&](auto fa_c, int stage, int ks, int buf) {
+        // MFMA operand fragments of one 32-wide k slice: the A fragments of two row blocks (a "pair"), double buffered,
+        // and the B fragments of the four column blocks. A phase is one pair times the four column blocks, column block by
+        // column block; while it runs the next pair's A fragments are read. In the last phase of a slice every B fragment is
+        // replaced by the next slice's as soon as its two matrix instructions have been issued (one set of B registers).
+        // The K loop exists in five versions, for wavefronts whose first FA = 8, 4, 2, 1 or 0 row blocks (of 16 rows)
+        // hold rows of the group.
+        typename EL::frag fa[2][2], fb[CB];
+        // A fragments of pair `pair` of slice ks into buffer buf
+        auto load_a = [&](auto fa_c, int stage, int ks, int pair, int buf) __attribute__((always_inline)) {
             constexpr int FA = decltype(fa_c)::value;
-            if constexpr (FA > 0) {
-                const uint8_t* ta = stage ? s_a1 : s_a0;
-                const uint8_t* tb = stage ? s_b1 : s_b0;
+            constexpr int AB = FA < 2 ? FA : 2;
+            const uint8_t* ta = stage ? s_a1 : s_a0;
 #pragma unroll
-                for (int i = 0; i < FA; ++i) {
-                    if constexpr (A_KC) fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_kc_frag(ta + a_off[i] + kc_slice[ks]));
-                    else fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_tr_frag(ta + a_off[i] + ks * 16 * kTRowBytes));
-                }
-#pragma unroll
-                for (int j = 0; j < FN; ++j) {
-                    if constexpr (B_KC) fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_kc_frag(tb + b_off[j] + kc_slice[ks]));
-                    else fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_tr_frag(tb + b_off[j] + ks * 16 * kTRowBytes));
-                }
+            for (int i = 0; i < AB; ++i) {
+                const int b = pair * 2 + i;
+                if constexpr (A_KC) fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_kc_frag(ta + a_off[b] + kc_slice[ks]));
+                else fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_tr_frag(ta + a_off[b] + ks * kSliceT));
             }
         };
-        auto mma = [&](auto fa_c, int buf) {
+        auto load_b = [&](int stage, int ks, int j) __attribute__((always_inline)) {
+            const uint8_t* tb = stage ? s_b1 : s_b0;
+            if constexpr (B_KC) fb[j] = __builtin_bit_cast(typename EL::frag, read_kc_frag(tb + b_off[j] + kc_slice[ks]));
+            else fb[j] = __builtin_bit_cast(typename EL::frag, read_tr_frag(tb + b_off[j] + ks * kSliceT));
+        };
+        // pair `pair` from A buffer abuf times the B fragments; reload: each B fragment is then read anew from slice
+        // next_ks of stage next_stage
+        auto mma = [&](auto fa_c, int pair, int abuf, bool reload, int next_stage, int next_ks) __attribute__((always_inline)) {
             constexpr int FA = decltype(fa_c)::value;
+            constexpr int AB = FA < 2 ? FA : 2;
+            if constexpr (FA > 0) {
 #pragma unroll
-            for (int i = 0; i < FA; ++i)
+                for (int j = 0; j < CB; ++j) {
 #pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    acc[i][j] = EL::mfma(fb[buf][j], fa[buf][i], acc[i][j]);
+                    for (int i = 0; i < AB; ++i)
+                        mfma_block(acc[pair * 2 + i], j, fb[j], fa[abuf][i]);
+                    if (reload) load_b(next_stage, next_ks, j);
+                }
+            }
         };
 
         // ---- one K step (see grouped_gemm.hip for the placement of barrier, waits and loads) ----
@@ -611,24 +643,40 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         // kt + 2: of this tile, or, in the last two steps, steps 0 and 1 of the next tile (or nothing).
         // SRC: which tile the loads issued in the step belong to: 0 the current one, 1 the next one (the loaders are aimed
         // by the caller in both cases), 2 decided here (first steps of a tile, and the versions for tiles with few rows).
-        auto step = [&](auto fa_c, auto wait_c, auto src_c, int stage, uint32_t kt) {
+        auto step = [&](auto fa_c, auto wait_c, auto src_c, int stage, uint32_t kt) __attribute__((always_inline)) {
             constexpr int FA = decltype(fa_c)::value;
             constexpr int SRC = decltype(src_c)::value;
-            constexpr int kReads = (A_KC ? FA : 2 * FA) + (B_KC ? FN : 2 * FN);
-            load_frags(fa_c, stage, 1, 1);
-            mma(fa_c, 0);
-            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, 0>();
-            load_frags(fa_c, stage, 2, 0);
-            mma(fa_c, 1);
-            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, 0>();
-            load_frags(fa_c, stage, 3, 1);
-            mma(fa_c, 0);
-            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, 0>();
+            constexpr int AB = FA < 2 ? FA : 2;       // row blocks per phase
+            constexpr int PP = FA >= 2 ? FA / 2 : 1;  // phases per k slice
+            constexpr int NPH = 2 * PP;               // phases of the step
+            constexpr int kReadsA = (A_KC ? 1 : 2) * AB, kReadsB = (B_KC ? 1 : 2);  // LDS reads per pair, per B fragment
+            // On entry A buffer 0 and the B registers hold the fragments of the first phase.
+#pragma unroll
+            for (int ph = 0; ph < NPH - 1; ++ph) {
+                const bool last_of_slice = ph == PP - 1;
+                load_a(fa_c, stage, (ph + 1) / PP, (ph + 1) % PP, (ph + 1) & 1);
+                mma(fa_c, ph % PP, ph & 1, last_of_slice, stage, 1);
+                if constexpr (FA > 0) {
+                    if (last_of_slice) {
+                        // the A reads, then per column block its matrix instructions and the read of its next fragment
+                        __builtin_amdgcn_sched_group_barrier(0x100, kReadsA, 0);
+#pragma unroll
+                        for (int j = 0; j < CB; ++j) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, AB, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x100, kReadsB, 0);
+                        }
+                    } else {
+                        interleave3<0, AB * CB, kReadsA, 0>();
+                    }
+                    // nothing moves from one phase into another: reads issued earlier would hold their registers longer
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
             // every load of step kt+1 has landed and every LDS read of this stage has returned
             __builtin_amdgcn_s_waitcnt(decltype(wait_c)::value);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            load_frags(fa_c, stage ^ 1, 0, 0);
+            load_a(fa_c, stage ^ 1, 0, 0, 0);
             uint32_t k0;
             if constexpr (SRC == 0) {
                 k0 = (kt + 2u) * (uint32_t)BK;
@@ -657,10 +705,22 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             // counts on it being the newest load)
             if constexpr (kPrefetch) asm volatile("" : "+v"(pf_voff));
             issue_prefetch(kt + kPfDist);
-            mma(fa_c, 1);
+            mma(fa_c, PP - 1, 1, true, stage ^ 1, 0);
             if constexpr (FA > 0) {
-                __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
-                spread_mfma_vmem<0, FA * FN, (int)kStepLoads>();
+                // the A reads; per column block its matrix instructions, each followed by its share of the step's loads, and
+                // the read of the block's next fragment; the prefetch last
+                constexpr int kLoadsPer = (int)kStepLoads / (AB * CB);
+                static_assert(kLoadsPer * AB * CB == (int)kStepLoads, "the loads divide evenly over the matrix instructions");
+                __builtin_amdgcn_sched_group_barrier(0x100, kReadsA, 0);
+#pragma unroll
+                for (int j = 0; j < CB; ++j) {
+#pragma unroll
+                    for (int i = 0; i < AB; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x020, kLoadsPer, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x100, kReadsB, 0);
+                }
                 if constexpr (kPrefetch) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
             }
         };
@@ -688,7 +748,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         const uint32_t tile_rows = Me - m0 < (uint32_t)BM ? Me - m0 : (uint32_t)BM;
         const uint32_t wave_rows = tile_rows > wm * WM ? tile_rows - wm * WM : 0u;
         const bool has_columns = n0 + wn * (kGlu ? WN / 2 : WN) < n_lim;
-        const uint32_t row_blocks = has_columns ? uniform((wave_rows + 31u) / 32u) : 0u;
+        const uint32_t row_blocks = has_columns ? uniform((wave_rows + 15u) / 16u) : 0u;  // of 16 rows
         if (thin) {
             // three LDS stages in the space a tile of at most 64 rows leaves unused (grouped_gemm.hip); cold start
             constexpr uint32_t kThinLoads = 1 + kLoads;
@@ -717,25 +777,25 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 auto thin_step = [&](int st, uint32_t kt) {
                     if constexpr (FA > 0) {
 #pragma unroll
-                        for (int ks = 0; ks < 4; ++ks) {
-                            typename EL::frag ta[FA], tb[FN];
+                        for (int ks = 0; ks < 2; ++ks) {
+                            typename EL::frag ta[FA], tb[CB];
 #pragma unroll
                             for (int i = 0; i < FA; ++i)
                                 ta[i] = __builtin_bit_cast(typename EL::frag, read_kc_frag(a_at[st] + a_off[i] + kc_slice[ks]));
 #pragma unroll
-                            for (int j = 0; j < FN; ++j) {
+                            for (int j = 0; j < CB; ++j) {
                                 if constexpr (B_KC) {
                                     const uint8_t* half = b_frag_row(j) < 128u ? b_lo[st] + b_off[j] : b_hi[st] + (b_off[j] - 128u * kRowBytes);
                                     tb[j] = __builtin_bit_cast(typename EL::frag, read_kc_frag(half + kc_slice[ks]));
                                 } else {
-                                    const uint8_t* half = ks < 2 ? b_lo[st] + ks * 16 * kTRowBytes : b_hi[st] + (ks - 2) * 16 * kTRowBytes;
+                                    const uint8_t* half = ks == 0 ? b_lo[st] : b_hi[st];  // k rows 0..31 and 32..63 of the step
                                     tb[j] = __builtin_bit_cast(typename EL::frag, read_tr_frag(half + b_off[j]));
                                 }
                             }
 #pragma unroll
                             for (int i = 0; i < FA; ++i)
 #pragma unroll
-                                for (int j = 0; j < FN; ++j) acc[i][j] = EL::mfma(tb[j], ta[i], acc[i][j]);
+                                for (int j = 0; j < CB; ++j) mfma_block(acc[i], j, tb[j], ta[i]);
                         }
                     }
                     __builtin_amdgcn_s_waitcnt(waitcnt_imm((int)kThinLoads, false));
@@ -752,7 +812,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 if (kt < KT) thin_step(0, kt);
                 if (kt + 1 < KT) thin_step(1, kt + 1);
             };
-            if (row_blocks == 2) thin_loop(std::integral_constant<int, 2>{});
+            if (row_blocks > 2) thin_loop(std::integral_constant<int, 4>{});
+            else if (row_blocks == 2) thin_loop(std::integral_constant<int, 2>{});
             else if (row_blocks == 1) thin_loop(std::integral_constant<int, 1>{});
             else thin_loop(std::integral_constant<int, 0>{});
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, false));
@@ -779,10 +840,14 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             using SrcEither = std::integral_constant<int, 2>;
             auto k_loop = [&](auto fa_c) {
                 constexpr int FA = decltype(fa_c)::value;
-                load_frags(fa_c, 0, 0, 0);
+                load_a(fa_c, 0, 0, 0, 0);
+                if constexpr (FA > 0) {
+#pragma unroll
+                    for (int j = 0; j < CB; ++j) load_b(0, 0, j);
+                }
                 step(fa_c, WaitFirst{}, SrcEither{}, 0, 0);
                 step(fa_c, WaitStep{}, SrcEither{}, 1, 1);
-                if constexpr (FA == FM) {
+                if constexpr (FA == RB) {
                     // full tiles: the steps in the middle load from the current tile and the last two from the next, each
                     // with the loaders aimed once, so that the loop body carries no selects
                     if (KT2 > 2u) {
@@ -807,8 +872,9 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                     }
                 }
             };
-            static_assert(FM == 4, "the versions below are for four row blocks per wavefront");
-            if (row_blocks > 2) k_loop(std::integral_constant<int, 4>{});
+            static_assert(RB == 8, "the versions below are for eight row blocks per wavefront");
+            if (row_blocks > 4) k_loop(std::integral_constant<int, 8>{});
+            else if (row_blocks > 2) k_loop(std::integral_constant<int, 4>{});
             else if (row_blocks == 2) k_loop(std::integral_constant<int, 2>{});
             else if (row_blocks == 1) k_loop(std::integral_constant<int, 1>{});
             else k_loop(std::integral_constant<int, 0>{});
@@ -832,7 +898,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         g_issue_table(nn, round & 1u);
 
         // ---- epilogue: through this wavefront's 2 KB of the staging buffer, 16 rows of 128 bytes at a time ----
-        // A lane holds row (lane & 31), columns q*8 + (lane >> 5)*4 + 0..3 of each 32x32 accumulator block.
+        // A lane holds row (lane & 15), columns (lane >> 4)*4 + 0..3 of each 16x16 accumulator block.
         // (the lane id is made opaque so that the per-lane address arithmetic is redone per tile, not hoisted out of the
         // tile loop where it would occupy registers throughout the K loop)
         uint32_t el = lane;
@@ -841,51 +907,41 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         if (EPI == EPI_PLAIN && args.alpha != 1.0f) {
             const float alpha = args.alpha;
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
-#pragma unroll
-                for (int j = 0; j < FN; ++j) acc[i][j] *= alpha;
+            for (int i = 0; i < RB; ++i) acc[i] *= alpha;
         }
-        const bool upper = ((el >> 4) & 1u) != 0;  // this lane's row lies in the second 16 rows of its 32-row block
 #ifndef FMA_STREAM_OUT_STEPS
 #define FMA_STREAM_OUT_STEPS 16
 #endif
         // Tiles with a short reduction write much per flop (a weight gradient over ~500 rows: 8 K steps per 128 KB tile):
         // their stores carry the non-temporal hint (+4 to 5 % there); for long reductions plain stores are faster by 0 to 1 %
         const bool stream_out = FMA_STREAM_OUT_ALL_LAYOUTS ? KT <= FMA_STREAM_OUT_STEPS : (VARY_K && KT <= FMA_STREAM_OUT_STEPS);
-        // BIAS: the eight groups of four columns this lane holds of every row block: [j][q], as fp32
-        float bias_f[FN][4][4];
+        // BIAS: the four groups of four columns this lane holds of every row block, as fp32
+        float bias_f[CB][4];
         if constexpr (BIAS) {
-            uint32_t at[8];
-            uint2 raw[8];
+            uint32_t at[4];
+            uint2 raw[4];
             const uint32_t mine = lds_address(s_bias) + wave * (uint32_t)kBiasBytes;
+            // plain: 64 columns; swiglu: 32 "up" columns (j = 0, 1), then 32 "gate" columns
 #pragma unroll
-            for (int j = 0; j < FN; ++j)
+            for (int j = 0; j < CB; ++j) at[j] = mine + ((uint32_t)j * 16u + (el >> 4) * 4u) * 2u;
+            lds_read4x8_quiet(at, raw);
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    // plain: 64 columns; swiglu: 32 "up" columns (j = 0), then 32 "gate" columns
-                    const uint32_t c = j * 32 + q * 8 + (el >> 5) * 4;
-                    at[j * 4 + q] = mine + c * 2u;
-                }
-            lds_read8x8_quiet(at, raw);
-#pragma unroll
-            for (int j = 0; j < FN; ++j)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const uint2 r = raw[j * 4 + q];
-                    bias_f[j][q][0] = EL::from_bits((uint16_t)(r.x & 0xffffu));
-                    bias_f[j][q][1] = EL::from_bits((uint16_t)(r.x >> 16));
-                    bias_f[j][q][2] = EL::from_bits((uint16_t)(r.y & 0xffffu));
-                    bias_f[j][q][3] = EL::from_bits((uint16_t)(r.y >> 16));
-                }
+            for (int j = 0; j < CB; ++j) {
+                const uint2 r = raw[j];
+                bias_f[j][0] = EL::from_bits((uint16_t)(r.x & 0xffffu));
+                bias_f[j][1] = EL::from_bits((uint16_t)(r.x >> 16));
+                bias_f[j][2] = EL::from_bits((uint16_t)(r.y & 0xffffu));
+                bias_f[j][3] = EL::from_bits((uint16_t)(r.y >> 16));
+            }
         }
         // the value that is stored (plain) or activated (swiglu): the rounded product, plus the bias rounded again, which is
         // what the product followed by a separate bias pass gives
-        auto with_bias = [&](float product, int j, int q, int x) -> float {
-            if constexpr (BIAS) return EL::round(product) + bias_f[j][q][x];
+        auto with_bias = [&](float product, int j, int x) -> float {
+            if constexpr (BIAS) return EL::round(product) + bias_f[j][x];
             else return product;
         };
         // EPI_SWIGLU_BWD: the h values of the eight passes (16 rows each) of this wavefront's sub-tile: [pass][row 0/1][up, gate]
-        u32x4 bwd_h[EPI == EPI_SWIGLU_BWD ? 2 * FM : 1][2][2];
+        u32x4 bwd_h[EPI == EPI_SWIGLU_BWD ? RB : 1][2][2];
         // byte offset of this lane's piece of row `r` (0 or 1: rows lane / 8 and 8 + lane / 8 of the pass) from the pass's
         // first row and the wavefront's first column, or out of range
         auto bwd_offset = [&](int r, uint32_t cols_valid) -> uint32_t {
@@ -945,119 +1001,91 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 }
             }
         };
+        const uint32_t put_row = el & 15u, put_col = (el >> 4) * 4u;  // this lane's place in a 16 x 16 block
+        uint32_t ypack[2][2][2];  // swiglu: the activation of two row blocks, which share one image: [block][column block][2]
 #pragma unroll
-        for (int i = 0; i < FM; ++i) {
-            const uint32_t row0 = m0 + wm * WM + i * 32;  // first output row of this block
-            if constexpr (EPI == EPI_PLAIN) {
+        for (int i = 0; i < RB; ++i) {
+            const uint32_t r0 = m0 + wm * WM + i * 16;  // first output row of this block
+            const uint32_t rows_valid = r0 < Me ? (Me - r0 < 16u ? Me - r0 : 16u) : 0u;
+            if constexpr (EPI == EPI_PLAIN || EPI == EPI_SWIGLU_BWD) {
                 const uint32_t col0 = n0 + wn * WN;
                 const uint32_t cols_valid = col0 < n_lim ? n_lim - col0 : 0u;
-                uint2 w[FN][4];
+                uint2 w[CB];
 #pragma unroll
-                for (int j = 0; j < FN; ++j)
+                for (int j = 0; j < CB; ++j) {
+                    const f32x16& c = acc[i];
+                    w[j].x = EL::pack2(with_bias(c[4 * j + 0], j, 0), with_bias(c[4 * j + 1], j, 1));
+                    w[j].y = EL::pack2(with_bias(c[4 * j + 2], j, 2), with_bias(c[4 * j + 3], j, 3));
+                }
+                if constexpr (EPI == EPI_PLAIN) {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const f32x16& c = acc[i][j];
-                        w[j][q].x = EL::pack2(with_bias(c[q * 4 + 0], j, q, 0), with_bias(c[q * 4 + 1], j, q, 1));
-                        w[j][q].y = EL::pack2(with_bias(c[q * 4 + 2], j, q, 2), with_bias(c[q * 4 + 3], j, q, 3));
-                    }
-#pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                    if (upper == (half == 1)) {
-#pragma unroll
-                        for (int j = 0; j < FN; ++j)
-#pragma unroll
-                            for (int q = 0; q < 4; ++q) stage_put_quiet<WN * 2>(img, el & 15u, j * 32 + q * 8 + (el >> 5) * 4, w[j][q]);
-                    }
-                    const uint32_t r0 = row0 + half * 16;
-                    const uint32_t rows_valid = r0 < Me ? (Me - r0 < 16u ? Me - r0 : 16u) : 0u;
+                    for (int j = 0; j < CB; ++j) stage_put_quiet<WN * 2>(img, put_row, j * 16 + put_col, w[j]);
                     stage_flush_quiet<WN * 2, 16>(img, args.D + off_d + (uint64_t)r0 * Ne + col0, Ne, rows_valid, cols_valid, el,
                                                   stream_out);
-                }
-            } else if constexpr (EPI == EPI_SWIGLU_BWD) {
-                // The product (rounded) is the gradient of the activation; h and its gradient are [rows, 2 Ne] with "up" in
-                // columns 0.., "gate" in columns Ne... A pass is 16 rows x 64 columns: a lane takes 8 columns of two rows,
-                // fetches the 8 up and 8 gate values of each (requested two passes ahead), and stores both gradients.
-                const uint32_t col0 = n0 + wn * WN;
-                const uint32_t cols_valid = col0 < n_lim ? n_lim - col0 : 0u;
-                uint2 w[FN][4];
-#pragma unroll
-                for (int j = 0; j < FN; ++j)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const f32x16& c = acc[i][j];
-                        w[j][q].x = EL::pack2(c[q * 4 + 0], c[q * 4 + 1]);
-                        w[j][q].y = EL::pack2(c[q * 4 + 2], c[q * 4 + 3]);
-                    }
-#pragma unroll
-                for (int half = 0; half < 2; ++half) {
+                } else {
+                    // The product (rounded) is the gradient of the activation; h and its gradient are [rows, 2 Ne] with "up" in
+                    // columns 0.., "gate" in columns Ne... A pass is 16 rows x 64 columns: a lane takes 8 columns of two rows,
+                    // fetches the 8 up and 8 gate values of each (requested two passes ahead), and stores both gradients.
                     constexpr int kAhead = FMA_BWD_AHEAD;
-                    const int pass = i * 2 + half;
-                    if (pass == 0) {
+                    if (i == 0) {
 #pragma unroll
                         for (int a = 0; a < kAhead; ++a) bwd_request(a, col0, cols_valid);
                     }
-                    if (upper == (half == 1)) {
 #pragma unroll
-                        for (int j = 0; j < FN; ++j)
-#pragma unroll
-                            for (int q = 0; q < 4; ++q) stage_put_quiet<WN * 2>(img, el & 15u, j * 32 + q * 8 + (el >> 5) * 4, w[j][q]);
-                    }
-                    bwd_finish(pass, col0, cols_valid);
-                    if (pass + kAhead < 2 * FM) bwd_request(pass + kAhead, col0, cols_valid);
+                    for (int j = 0; j < CB; ++j) stage_put_quiet<WN * 2>(img, put_row, j * 16 + put_col, w[j]);
+                    bwd_finish(i, col0, cols_valid);
+                    if (i + kAhead < RB) bwd_request(i + kAhead, col0, cols_valid);
                 }
             } else {
-                // first the rounded pre-activation (32 "up" columns | 32 "gate" columns per row), then the activation
+                // first the rounded pre-activation (32 "up" columns | 32 "gate" columns per row) of this row block, then,
+                // after every second block, the activation of both
                 constexpr int HB = WN * 2;
                 constexpr int YB = WN;
-                static_assert(FN == 2, "one up block and one gate block per wavefront and row block");
+                static_assert(CB == 4, "two up blocks and two gate blocks per wavefront and row block");
                 const uint32_t col0 = n0 + wn * (WN / 2);
                 const uint32_t cols_valid = col0 < n_lim ? n_lim - col0 : 0u;
-                uint32_t ypack[4][2];
-                uint2 wu[4], wg[4];
+                uint2 wu[2], wg[2];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
+                for (int jj = 0; jj < 2; ++jj) {
                     float u[4], g[4], y[4];
 #pragma unroll
                     for (int x = 0; x < 4; ++x) {
-                        u[x] = EL::round(with_bias(acc[i][0][q * 4 + x], 0, q, x));
-                        g[x] = EL::round(with_bias(acc[i][1][q * 4 + x], 1, q, x));
+                        u[x] = EL::round(with_bias(acc[i][4 * jj + x], jj, x));
+                        g[x] = EL::round(with_bias(acc[i][4 * (2 + jj) + x], 2 + jj, x));
                         y[x] = u[x] * g[x] * sigmoid_for<typename EL::act_t>(g[x]);
                     }
-                    ypack[q][0] = EL::pack2(y[0], y[1]);
-                    ypack[q][1] = EL::pack2(y[2], y[3]);
+                    ypack[i & 1][jj][0] = EL::pack2(y[0], y[1]);
+                    ypack[i & 1][jj][1] = EL::pack2(y[2], y[3]);
                     if constexpr (EPI == EPI_SWIGLU) {
-                        wu[q].x = EL::pack2(u[0], u[1]);
-                        wu[q].y = EL::pack2(u[2], u[3]);
-                        wg[q].x = EL::pack2(g[0], g[1]);
-                        wg[q].y = EL::pack2(g[2], g[3]);
+                        wu[jj].x = EL::pack2(u[0], u[1]);
+                        wu[jj].y = EL::pack2(u[2], u[3]);
+                        wg[jj].x = EL::pack2(g[0], g[1]);
+                        wg[jj].y = EL::pack2(g[2], g[3]);
                     }
                 }
                 if constexpr (EPI == EPI_SWIGLU) {
 #pragma unroll
-                    for (int half = 0; half < 2; ++half) {
-                        if (upper == (half == 1)) {
-#pragma unroll
-                            for (int q = 0; q < 4; ++q) {
-                                const uint32_t c = q * 8 + (el >> 5) * 4;
-                                stage_put_quiet<HB>(img, el & 15u, c, wu[q]);
-                                stage_put_quiet<HB>(img, el & 15u, WN / 2 + c, wg[q]);
-                            }
-                        }
-                        const uint32_t r0 = row0 + half * 16;
-                        const uint32_t rows_valid = r0 < Me ? (Me - r0 < 16u ? Me - r0 : 16u) : 0u;
-                        stage_flush_split_quiet<HB, 16, WN / 2>(img, args.D + off_d + (uint64_t)r0 * Ne + col0, Ne, rows_valid, cols_valid,
-                                                          n_span, el);
+                    for (int jj = 0; jj < 2; ++jj) {
+                        stage_put_quiet<HB>(img, put_row, jj * 16 + put_col, wu[jj]);
+                        stage_put_quiet<HB>(img, put_row, WN / 2 + jj * 16 + put_col, wg[jj]);
                     }
+                    stage_flush_split_quiet<HB, 16, WN / 2>(img, args.D + off_d + (uint64_t)r0 * Ne + col0, Ne, rows_valid, cols_valid,
+                                                            n_span, el);
                 }
-                const uint32_t rows_valid = row0 < Me ? (Me - row0 < 32u ? Me - row0 : 32u) : 0u;
+                if (i & 1) {
+                    const uint32_t row0 = r0 - 16u;  // first row of the pair of blocks
+                    const uint32_t rows_pair = row0 < Me ? (Me - row0 < 32u ? Me - row0 : 32u) : 0u;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    uint2 wy;
-                    wy.x = ypack[q][0];
-                    wy.y = ypack[q][1];
-                    stage_put_quiet<YB>(img, el & 31u, q * 8 + (el >> 5) * 4, wy);
+                    for (int b = 0; b < 2; ++b)
+#pragma unroll
+                        for (int jj = 0; jj < 2; ++jj) {
+                            uint2 wy;
+                            wy.x = ypack[b][jj][0];
+                            wy.y = ypack[b][jj][1];
+                            stage_put_quiet<YB>(img, b * 16 + put_row, jj * 16 + put_col, wy);
+                        }
+                    stage_flush_quiet<YB, 32>(img, args.ACT + off_d / 2 + (uint64_t)row0 * n_span + col0, n_span, rows_pair, cols_valid, el);
                 }
-                stage_flush_quiet<YB, 32>(img, args.ACT + off_d / 2 + (uint64_t)row0 * n_span + col0, n_span, rows_valid, cols_valid, el);
             }
         }
 
