@@ -484,13 +484,17 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                                                              : (EPI == EPI_SWIGLU ? WM * WN * 2 / 1024 : 0) + WM * WN / 1024;
 
     // loads of one K step of the CURRENT loaders' aim into `stage` (compiler-visible: placed by the scheduling hints)
-    auto issue_a = [&](int stage, uint32_t k0) {
-        if constexpr (A_KC) lk_a.template issue_range<0, kLoads>(stage ? s_a1 : s_a0, k0);
-        else lt_a.template issue_range<0, kLoads>(stage ? s_a1 : s_a0, k0);
+    // (i0_c, i1_c: which of the kLoads instructions)
+    auto issue_a = [&](int stage, uint32_t k0, auto i0_c, auto i1_c) __attribute__((always_inline)) {
+        constexpr int I0 = decltype(i0_c)::value, I1 = decltype(i1_c)::value;
+        if constexpr (A_KC) lk_a.template issue_range<I0, I1>(stage ? s_a1 : s_a0, k0);
+        else lt_a.template issue_range<I0, I1>(stage ? s_a1 : s_a0, k0);
     };
     // GATHER: the same four loads through the row table in half `half`; `bytes`: how much of A they may read
     // kept: take the offsets from g_kept (the caller has set it for that tile) instead of reading the table
-    auto issue_a_gathered = [&](int stage, uint32_t k0, uint32_t half, uint32_t bytes, bool kept) {
+    auto issue_a_gathered = [&](int stage, uint32_t k0, uint32_t half, uint32_t bytes, bool kept, auto i0_c, auto i1_c)
+                                __attribute__((always_inline)) {
+        constexpr int I0 = decltype(i0_c)::value, I1 = decltype(i1_c)::value;
         uint32_t v[4];
         if (kept) {
 #pragma unroll
@@ -502,12 +506,13 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         const __amdgpu_buffer_rsrc_t r = make_rsrc(args.A, bytes);
         uint8_t* tile = stage ? s_a1 : s_a0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = I0; i < I1; ++i)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(tile + (i * NW + wave) * 1024), 16, v[i], k0 * 2u, 0, 0);
     };
-    auto issue_b = [&](int stage, uint32_t k0) {
-        if constexpr (B_KC) lk_b.template issue_range<0, kLoads>(stage ? s_b1 : s_b0, k0);
-        else lt_b.template issue_range<0, kLoads>(stage ? s_b1 : s_b0, k0);
+    auto issue_b = [&](int stage, uint32_t k0, auto i0_c, auto i1_c) __attribute__((always_inline)) {
+        constexpr int I0 = decltype(i0_c)::value, I1 = decltype(i1_c)::value;
+        if constexpr (B_KC) lk_b.template issue_range<I0, I1>(stage ? s_b1 : s_b0, k0);
+        else lt_b.template issue_range<I0, I1>(stage ? s_b1 : s_b0, k0);
     };
     // ... and written in assembly, for a cold start
     auto issue_quiet = [&](int stage, uint32_t k0) {
@@ -604,7 +609,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         // replaced by the next slice's as soon as its two matrix instructions have been issued (one set of B registers).
         // The K loop exists in five versions, for wavefronts whose first FA = 8, 4, 2, 1 or 0 row blocks (of 16 rows)
         // hold rows of the group.
-        typename EL::frag fa[2][2], fb[CB];
+        typename EL::frag fa[4][2], fb[CB];
         // A fragments of pair `pair` of slice ks into buffer buf
         auto load_a = [&](auto fa_c, int stage, int ks, int pair, int buf) __attribute__((always_inline)) {
             constexpr int FA = decltype(fa_c)::value;
@@ -651,14 +656,54 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             constexpr int NPH = 2 * PP;               // phases of the step
             constexpr int kReadsA = (A_KC ? 1 : 2) * AB, kReadsB = (B_KC ? 1 : 2);  // LDS reads per pair, per B fragment
             // On entry A buffer 0 and the B registers hold the fragments of the first phase.
+            typedef std::integral_constant<int, 0> I0_;
+            typedef std::integral_constant<int, 2> I2_;
+            typedef std::integral_constant<int, 3> I3_;
+            typedef std::integral_constant<int, kLoads> IN_;
+            static_assert(kLoads == 4, "the split of a step's loads over three phases is written for four per operand");
+            // the A loads [i0, i1) of the step's load slot
+            auto issue_a_part = [&](uint32_t k0, auto i0_c, auto i1_c) __attribute__((always_inline)) {
+                if constexpr (GATHER) {
+                    const bool of_next = SRC == 1 || (SRC == 2 && kt + 2u >= KT2);
+                    issue_a_gathered(stage, k0, (of_next ? round + 1u : round) & 1u, of_next ? g_bytes_nxt : g_full, SRC != 2, i0_c, i1_c);
+                } else {
+                    issue_a(stage, k0, i0_c, i1_c);
+                }
+            };
+            // what the loads issued in this step fetch: the K offset (returned) and, decided here (SRC == 2), whether the
+            // loaders aim at the current tile's operands or the next one's
+            auto aim_loads = [&]() __attribute__((always_inline)) -> uint32_t {
+                uint32_t k0;
+                if constexpr (SRC == 0) {
+                    k0 = (kt + 2u) * (uint32_t)BK;
+                } else if constexpr (SRC == 1) {
+                    k0 = (kt + 2u - KT2) * (uint32_t)BK;
+                } else {
+                    const bool of_next = kt + 2u >= KT2;
+                    k0 = (of_next ? kt + 2u - KT2 : kt + 2u) * (uint32_t)BK;
+                    if constexpr (!GATHER)
+                        aim_a(Feed<A_KC>{of_next ? fa_nxt.base0 : fa_cur.base0, nullptr, of_next ? fa_nxt.extent : fa_cur.extent,
+                                         of_next ? fa_nxt.ldb : fa_cur.ldb, of_next ? fa_nxt.col_bytes : fa_cur.col_bytes},
+                              of_next ? va_nxt : va_cur);
+                    aim_b(Feed<B_KC>{of_next ? fb_nxt.base0 : fb_cur.base0, of_next ? fb_nxt.base1 : fb_cur.base1,
+                                     of_next ? fb_nxt.extent : fb_cur.extent, of_next ? fb_nxt.ldb : fb_cur.ldb,
+                                     of_next ? fb_nxt.col_bytes : fb_cur.col_bytes},
+                          of_next ? vb_nxt : vb_cur);
+                }
+                return k0;
+            };
+            if constexpr (FA == RB) {
+                // Full tiles: the barrier comes after five of the eight phases, with the A fragments of the last three phases
+                // already in registers (four A buffers), so that the step's loads go out over three phases instead of one:
+                // eight wavefronts that leave the barrier together otherwise queue 72 loads on the one address path at once.
+                // A fragments are read two phases ahead (phase p's pair sits in buffer p % 4): phase 0 reads those of phases 1
+                // (the step before could not: they are behind its barrier) and 2, phase 4 those of 6 and 7 first thing
+                load_a(fa_c, stage, 0, 1, 1);
 #pragma unroll
-            for (int ph = 0; ph < NPH - 1; ++ph) {
-                const bool last_of_slice = ph == PP - 1;
-                load_a(fa_c, stage, (ph + 1) / PP, (ph + 1) % PP, (ph + 1) & 1);
-                mma(fa_c, ph % PP, ph & 1, last_of_slice, stage, 1);
-                if constexpr (FA > 0) {
-                    if (last_of_slice) {
-                        // the A reads, then per column block its matrix instructions and the read of its next fragment
+                for (int ph = 0; ph < 4; ++ph) {
+                    load_a(fa_c, stage, (ph + 2) / PP, (ph + 2) % PP, (ph + 2) & 3);
+                    mma(fa_c, ph, ph, ph == 3, stage, 1);
+                    if (ph == 3) {
                         __builtin_amdgcn_sched_group_barrier(0x100, kReadsA, 0);
 #pragma unroll
                         for (int j = 0; j < CB; ++j) {
@@ -666,62 +711,97 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                             __builtin_amdgcn_sched_group_barrier(0x100, kReadsB, 0);
                         }
                     } else {
-                        interleave3<0, AB * CB, kReadsA, 0>();
+                        if (ph == 0) interleave3<0, AB * CB, 2 * kReadsA, 0>();
+                        else interleave3<0, AB * CB, kReadsA, 0>();
                     }
-                    // nothing moves from one phase into another: reads issued earlier would hold their registers longer
                     __builtin_amdgcn_sched_barrier(0);
                 }
-            }
-            // every load of step kt+1 has landed and every LDS read of this stage has returned
-            __builtin_amdgcn_s_waitcnt(decltype(wait_c)::value);
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
-            load_a(fa_c, stage ^ 1, 0, 0, 0);
-            uint32_t k0;
-            if constexpr (SRC == 0) {
-                k0 = (kt + 2u) * (uint32_t)BK;
-            } else if constexpr (SRC == 1) {
-                k0 = (kt + 2u - KT2) * (uint32_t)BK;
-            } else {
-                const bool of_next = kt + 2u >= KT2;
-                k0 = (of_next ? kt + 2u - KT2 : kt + 2u) * (uint32_t)BK;
-                if constexpr (!GATHER)
-                    aim_a(Feed<A_KC>{of_next ? fa_nxt.base0 : fa_cur.base0, nullptr, of_next ? fa_nxt.extent : fa_cur.extent,
-                                     of_next ? fa_nxt.ldb : fa_cur.ldb, of_next ? fa_nxt.col_bytes : fa_cur.col_bytes},
-                          of_next ? va_nxt : va_cur);
-                aim_b(Feed<B_KC>{of_next ? fb_nxt.base0 : fb_cur.base0, of_next ? fb_nxt.base1 : fb_cur.base1,
-                                 of_next ? fb_nxt.extent : fb_cur.extent, of_next ? fb_nxt.ldb : fb_cur.ldb,
-                                 of_next ? fb_nxt.col_bytes : fb_cur.col_bytes},
-                      of_next ? vb_nxt : vb_cur);
-            }
-            if constexpr (GATHER) {
-                const bool of_next = SRC == 1 || (SRC == 2 && kt + 2u >= KT2);
-                issue_a_gathered(stage, k0, (of_next ? round + 1u : round) & 1u, of_next ? g_bytes_nxt : g_full, SRC != 2);
-            } else {
-                issue_a(stage, k0);
-            }
-            issue_b(stage, k0);
-            // the prefetch goes out behind this step's loads (the empty statement orders it: the wait of the next step
-            // counts on it being the newest load)
-            if constexpr (kPrefetch) asm volatile("" : "+v"(pf_voff));
-            issue_prefetch(kt + kPfDist);
-            mma(fa_c, PP - 1, 1, true, stage ^ 1, 0);
-            if constexpr (FA > 0) {
-                // the A reads; per column block its matrix instructions, each followed by its share of the step's loads, and
-                // the read of the block's next fragment; the prefetch last
-                constexpr int kLoadsPer = (int)kStepLoads / (AB * CB);
-                static_assert(kLoadsPer * AB * CB == (int)kStepLoads, "the loads divide evenly over the matrix instructions");
+                load_a(fa_c, stage, 1, 2, 2);
+                load_a(fa_c, stage, 1, 3, 3);
+                mma(fa_c, 0, 0, false, stage, 1);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2 * kReadsA, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, AB * CB, 0);
+                // every load of step kt+1 has landed and every LDS read of this stage has returned
+                __builtin_amdgcn_s_waitcnt(decltype(wait_c)::value);
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                const uint32_t k0 = aim_loads();
+                issue_a_part(k0, I0_{}, I3_{});
+                mma(fa_c, 1, 1, false, stage, 1);
+                spread_mfma_vmem<0, AB * CB, 3>();
+                __builtin_amdgcn_sched_barrier(0);
+                issue_a_part(k0, I3_{}, IN_{});
+                issue_b(stage, k0, I0_{}, I2_{});
+                mma(fa_c, 2, 2, false, stage, 1);
+                spread_mfma_vmem<0, AB * CB, 3>();
+                __builtin_amdgcn_sched_barrier(0);
+                load_a(fa_c, stage ^ 1, 0, 0, 0);
+                issue_b(stage, k0, I2_{}, IN_{});
+                if constexpr (kPrefetch) asm volatile("" : "+v"(pf_voff));
+                issue_prefetch(kt + kPfDist);
+                mma(fa_c, 3, 3, true, stage ^ 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x100, kReadsA, 0);
 #pragma unroll
                 for (int j = 0; j < CB; ++j) {
 #pragma unroll
                     for (int i = 0; i < AB; ++i) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x020, kLoadsPer, 0);
+                        if (j * AB + i < 2 + (kPrefetch ? 1 : 0)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
                     }
                     __builtin_amdgcn_sched_group_barrier(0x100, kReadsB, 0);
                 }
-                if constexpr (kPrefetch) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            } else {
+#pragma unroll
+                for (int ph = 0; ph < NPH - 1; ++ph) {
+                    const bool last_of_slice = ph == PP - 1;
+                    load_a(fa_c, stage, (ph + 1) / PP, (ph + 1) % PP, (ph + 1) & 1);
+                    mma(fa_c, ph % PP, ph & 1, last_of_slice, stage, 1);
+                    if constexpr (FA > 0) {
+                        if (last_of_slice) {
+                            // the A reads, then per column block its matrix instructions and the read of its next fragment
+                            __builtin_amdgcn_sched_group_barrier(0x100, kReadsA, 0);
+#pragma unroll
+                            for (int j = 0; j < CB; ++j) {
+                                __builtin_amdgcn_sched_group_barrier(0x008, AB, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x100, kReadsB, 0);
+                            }
+                        } else {
+                            interleave3<0, AB * CB, kReadsA, 0>();
+                        }
+                        // nothing moves from one phase into another: reads issued earlier would hold their registers longer
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+                // every load of step kt+1 has landed and every LDS read of this stage has returned
+                __builtin_amdgcn_s_waitcnt(decltype(wait_c)::value);
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                load_a(fa_c, stage ^ 1, 0, 0, 0);
+                const uint32_t k0 = aim_loads();
+                issue_a_part(k0, I0_{}, IN_{});
+                issue_b(stage, k0, I0_{}, IN_{});
+                // the prefetch goes out behind this step's loads (the empty statement orders it: the wait of the next step
+                // counts on it being the newest load)
+                if constexpr (kPrefetch) asm volatile("" : "+v"(pf_voff));
+                issue_prefetch(kt + kPfDist);
+                mma(fa_c, PP - 1, 1, true, stage ^ 1, 0);
+                if constexpr (FA > 0) {
+                    // the A reads; per column block its matrix instructions, each followed by its share of the step's loads,
+                    // and the read of the block's next fragment; the prefetch last
+                    constexpr int kLoadsPer = (int)kStepLoads / (AB * CB);
+                    static_assert(kLoadsPer * AB * CB == (int)kStepLoads, "the loads divide evenly over the matrix instructions");
+                    __builtin_amdgcn_sched_group_barrier(0x100, kReadsA, 0);
+#pragma unroll
+                    for (int j = 0; j < CB; ++j) {
+#pragma unroll
+                        for (int i = 0; i < AB; ++i) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x020, kLoadsPer, 0);
+                        }
+                        __builtin_amdgcn_sched_group_barrier(0x100, kReadsB, 0);
+                    }
+                    if constexpr (kPrefetch) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                }
             }
         };
         // waits of a step: all but the newest load when that is the previous step's prefetch; in a tile's first step the
