@@ -584,10 +584,10 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         aim_a(fa_cur, va_cur);
         aim_b(fb_cur, vb_cur);
 
-        // The CB column blocks of a row block are one 16-register value (block j in elements 4 j ..), and every K step ends
-        // by naming these values as such (anchor_acc): that keeps a matrix instruction's result in the register quadruple its
-        // addend came from. As 32 separate quadruples the results wander through the register file, which the allocator
-        // could not fit without spilling.
+        // The CB column blocks of a row block are one 16-register value (block j in elements 4 j ..), and every matrix
+        // instruction's result is named as part of that value again (anchor_value): the result then stays in the register
+        // quadruple its addend came from. The compiler has no tied-operand form of the 4-register instruction; as 32 separate
+        // quadruples the results wandered through the register file and the allocator spilled 3 to 40 registers.
         f32x16 acc[RB];
 #pragma unroll
         for (int i = 0; i < RB; ++i)
@@ -603,10 +603,11 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             anchor_value(c);
         };
 
-        // MFMA operand fragments of one 32-wide k slice: the A fragments of two row blocks (a "pair"), double buffered,
-        // and the B fragments of the four column blocks. A phase is one pair times the four column blocks, column block by
-        // column block; while it runs the next pair's A fragments are read. In the last phase of a slice every B fragment is
-        // replaced by the next slice's as soon as its two matrix instructions have been issued (one set of B registers).
+        // MFMA operand fragments of one 32-wide k slice: the A fragments of two row blocks (a "pair"), in four buffers (full
+        // tiles read them two phases ahead and hold three pairs across the step's barrier; the other versions use two), and
+        // the B fragments of the four column blocks. A phase is one pair times the four column blocks, column block by
+        // column block. In the last phase of a slice every B fragment is replaced by the next slice's as soon as its two
+        // matrix instructions have been issued (one set of B registers).
         // The K loop exists in five versions, for wavefronts whose first FA = 8, 4, 2, 1 or 0 row blocks (of 16 rows)
         // hold rows of the group.
         typename EL::frag fa[4][2], fb[CB];
