@@ -1037,14 +1037,17 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         auto bwd_origin = [&](int pass, uint32_t col0) -> uint64_t {  // element offset of the pass's first row and column
             return ((uint64_t)cur.row0 + m0 + wm * WM + (uint32_t)pass * 16u) * (2ull * Ne) + col0;
         };
+        // h is read once and its gradient written once, in whole 128-byte lines: both carry the non-temporal hint, which
+        // keeps them from displacing the operand panels in the L2 (+3 % on the Mixtral shape, +2 % large-E, +0.5 % fine-grained)
+        constexpr int kStreamAux = 2;
         auto bwd_request = [&](int pass, uint32_t col0, uint32_t cols_valid) {
             if constexpr (EPI == EPI_SWIGLU_BWD) {
                 const __amdgpu_buffer_rsrc_t rs = make_rsrc(args.h_in + bwd_origin(pass, col0), bwd_rows(pass) * (Ne * 4u));
 #pragma unroll
                 for (int r = 0; r < 2; ++r) {
                     const uint32_t off = bwd_offset(r, cols_valid);
-                    bwd_h[pass][r][0] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, 0);
-                    bwd_h[pass][r][1] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, (int)(Ne * 2u), 0);
+                    bwd_h[pass][r][0] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, kStreamAux);
+                    bwd_h[pass][r][1] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, (int)(Ne * 2u), kStreamAux);
                 }
             }
         };
@@ -1077,8 +1080,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                     // there (it does for stores with a constant scalar offset, as every other store of this library has).
                     const uint32_t off = bwd_offset(r, cols_valid);
                     const uint32_t off_gate = off == kOutOfRange ? kOutOfRange : off + Ne * 2u;
-                    __builtin_amdgcn_raw_buffer_store_b128(du, rs, (int)off, 0, 0);
-                    __builtin_amdgcn_raw_buffer_store_b128(dg, rs, (int)off_gate, 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(du, rs, (int)off, 0, kStreamAux);
+                    __builtin_amdgcn_raw_buffer_store_b128(dg, rs, (int)off_gate, 0, kStreamAux);
                 }
             }
         };
