@@ -153,9 +153,10 @@ __device__ __forceinline__ s16x8 read_kc_frag(const uint8_t* p) { return *reinte
 // 16-byte buffer store of a staged piece. A lane whose offset is not below the descriptor's size stores nothing, so
 // every lane always executes the instruction: the number of stores a wavefront issues per tile is a compile-time
 // constant, which the wait for the next tile's first loads relies on.
-// NT = the non-temporal hint. Measured both ways on the three benchmark layers: with the hint the six GEMMs ran 0.5 to
-// 1.5 points of peak slower than with plain stores (22 of 24 comparisons), and streamed 64-byte pieces are not merged
-// in the L2 and cost a read-modify-write each (SwiGLU epilogue: +35 % fetched and +28 % written bytes). No caller sets it.
+// NT = the non-temporal hint. Measured both ways on the three benchmark layers: hinted and plain stores of whole
+// 128-byte lines run within 0.5 % of each other, except for weight-gradient tiles with a short reduction, which write
+// much per flop and gain 1.5 to 4 % from the hint (the only caller that sets it); streamed 64-byte pieces are not merged
+// in the L2 and cost a read-modify-write each (SwiGLU epilogue: +35 % fetched and +28 % written bytes).
 template <bool NT>
 __device__ __forceinline__ void store_tile16(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint4 v) {
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc, (int)voff, 0, NT ? 2 : 0);
