@@ -23,18 +23,9 @@ static __device__ __align__(256) uint32_t scratch[FMA_STATIC_INDEX_WORDS];
 namespace fmahip {
 namespace {
 
-#ifndef FMA_COUNT_THREADS
-#define FMA_COUNT_THREADS 1024
-#endif
-#ifndef FMA_COUNT_UNROLL
-#define FMA_COUNT_UNROLL 4
-#endif
-#ifndef FMA_COUNT_BLOCKS_PER_CU
-#define FMA_COUNT_BLOCKS_PER_CU 2
-#endif
-constexpr int kCountThreads = FMA_COUNT_THREADS;
-constexpr int kCountUnroll = FMA_COUNT_UNROLL;
-constexpr int kCountBlocksPerCu = FMA_COUNT_BLOCKS_PER_CU;
+constexpr int kCountThreads = 1024;
+constexpr int kCountUnroll = 4;
+constexpr int kCountBlocksPerCu = 2;
 constexpr int kCountLdsWords = 16384;  // 64 KB of bins (all copies)
 
 __host__ __device__ inline uint32_t floor_pow2(uint32_t x) {

@@ -32,24 +32,12 @@ namespace fmahip {
 namespace gemm {
 
 // how the load instructions of a K step are spread over the slices after the barrier that frees their stage
-#ifndef FMA_PF_DIST
-#define FMA_PF_DIST 4
-#endif
-constexpr uint32_t kPfDist = FMA_PF_DIST;  // K steps between a line's prefetch and the step that loads it
-#ifndef FMA_LD_S3
-#define FMA_LD_S3 8
-#define FMA_LD_S0 0
-#define FMA_LD_S1 0
-#define FMA_LD_S2 0
-#endif
+constexpr uint32_t kPfDist = 4;  // K steps between a line's prefetch and the step that loads it
+// how many of a K step's eight loads per wavefront go out in the last k slice of the step (kLoadsS3) and in the first
+// three slices of the next one
+constexpr int kLoadsS3 = 8, kLoadsS0 = 0, kLoadsS1 = 0, kLoadsS2 = 0;
 
 
-#ifdef FMA_PROF
-// timing instrumentation of a diagnostic build: per (workgroup, wavefront): cycles waiting for loads, cycles in the
-// barrier, K steps, cycles in the kernel, cycles at the tile boundary (epilogue + next tile's set-up)
-__device__ unsigned long long fma_prof[2 * 1024 * 8 * 8];
-#define PROF_STAMP(t) asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t))
-#endif
 
 struct GemmArgs {
     const uint16_t* A;
@@ -377,14 +365,8 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     };
     // loads of the K step at k0 into `stage`: inside the K loop (compiler-visible, placed by the scheduling hints) ...
     auto issue = [&](int stage, uint32_t k0) {
-#if defined(FMA_DIAG) && FMA_DIAG == 4
-        return;
-#endif
         if constexpr (A_KC) lk_a.issue(stage ? s_a1 : s_a0, k0);
         else lt_a.issue(stage ? s_a1 : s_a0, k0);
-#if defined(FMA_DIAG) && FMA_DIAG == 3
-        return;
-#endif
         if constexpr (B_KC) lk_b.issue(stage ? s_b1 : s_b0, k0);
         else lt_b.issue(stage ? s_b1 : s_b0, k0);
     };
@@ -432,12 +414,6 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         else __builtin_amdgcn_s_waitcnt(0x0f70);               // vmcnt(0)
     };
 
-#ifdef FMA_PROF
-    uint64_t prof_wait = 0, prof_bar = 0, prof_steps = 0, prof_start, prof_edge = 0, prof_e0 = 0;
-    uint64_t prof_seg[6] = {0, 0, 0, 0, 0, 0}, prof_t = 0;
-#define PROF_SEG(i) do { uint64_t t_; PROF_STAMP(t_); if (prof_e0) prof_seg[i] += t_ - prof_t; prof_t = t_; } while (0)
-    PROF_STAMP(prof_start);
-#endif
     uint32_t round = 0;
     Tile cur = lookup(0);
     // prefetched: the loaders are set up for `cur` and the loads of its first K step went out (into stage 0) before the
@@ -484,17 +460,11 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                 const uint8_t* tb = stage ? s_b1 : s_b0;
 #pragma unroll
                 for (int i = 0; i < FA; ++i) {
-#if defined(FMA_DIAG) && (FMA_DIAG == 1 || FMA_DIAG == 2)
-                    if (ks & (FMA_DIAG == 1 ? 1 : 3)) { fa[buf][i] = fa[buf ^ 1][i]; continue; }
-#endif
                     if constexpr (A_KC) fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_kc_frag(ta + a_off[i] + kc_slice[ks]));
                     else fa[buf][i] = __builtin_bit_cast(typename EL::frag, read_tr_frag(ta + a_off[i] + ks * 16 * kTRowBytes));
                 }
 #pragma unroll
                 for (int j = 0; j < FN; ++j) {
-#if defined(FMA_DIAG) && FMA_DIAG == 2
-                    if (ks & 3) { fb[buf][j] = fb[buf ^ 1][j]; continue; }
-#endif
                     if constexpr (B_KC) fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_kc_frag(tb + b_off[j] + kc_slice[ks]));
                     else fb[buf][j] = __builtin_bit_cast(typename EL::frag, read_tr_frag(tb + b_off[j] + ks * 16 * kTRowBytes));
                 }
@@ -527,58 +497,34 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
         auto step = [&](auto fa_c, int stage, uint32_t kt) {
             constexpr int FA = decltype(fa_c)::value;
             constexpr int kReads = (A_KC ? FA : 2 * FA) + (B_KC ? FN : 2 * FN);
-            using L3 = std::integral_constant<int, FMA_LD_S3>;
-            using L0 = std::integral_constant<int, FMA_LD_S0>;
-            using L1 = std::integral_constant<int, FMA_LD_S1>;
-            using L2 = std::integral_constant<int, FMA_LD_S2>;
-            static_assert(FMA_LD_S3 + FMA_LD_S0 + FMA_LD_S1 + FMA_LD_S2 == 2 * (32 / NW), "every load of a step is issued once");
+            using L3 = std::integral_constant<int, kLoadsS3>;
+            using L0 = std::integral_constant<int, kLoadsS0>;
+            using L1 = std::integral_constant<int, kLoadsS1>;
+            using L2 = std::integral_constant<int, kLoadsS2>;
+            static_assert(kLoadsS3 + kLoadsS0 + kLoadsS1 + kLoadsS2 == 2 * (32 / NW), "every load of a step is issued once");
             load_frags(fa_c, stage, 1, 1);
             issue_some(L3{}, L0{}, stage ^ 1, (kt + 1) * BK);
             mma(fa_c, 0);
-            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, FMA_LD_S0>();
+            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, kLoadsS0>();
             load_frags(fa_c, stage, 2, 0);
-            issue_some(std::integral_constant<int, FMA_LD_S3 + FMA_LD_S0>{}, L1{}, stage ^ 1, (kt + 1) * BK);
+            issue_some(std::integral_constant<int, kLoadsS3 + kLoadsS0>{}, L1{}, stage ^ 1, (kt + 1) * BK);
             mma(fa_c, 1);
-            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, FMA_LD_S1>();
+            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, kLoadsS1>();
             load_frags(fa_c, stage, 3, 1);
-            issue_some(std::integral_constant<int, FMA_LD_S3 + FMA_LD_S0 + FMA_LD_S1>{}, L2{}, stage ^ 1, (kt + 1) * BK);
+            issue_some(std::integral_constant<int, kLoadsS3 + kLoadsS0 + kLoadsS1>{}, L2{}, stage ^ 1, (kt + 1) * BK);
             mma(fa_c, 0);
-            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, FMA_LD_S2>();
+            if constexpr (FA > 0) interleave3<0, FA * FN, kReads, kLoadsS2>();
             // every load of step kt+1 has landed and every LDS read of this stage has returned
-#ifdef FMA_PROF
-            uint64_t pt0, pt1, pt2;
-            asm volatile("s_memtime %0" : "=s"(pt0));
-#endif
-#if defined(FMA_DIAG) && FMA_DIAG >= 5
-            __builtin_amdgcn_s_waitcnt(0x0070 + (FMA_DIAG - 3));  // all but the newest 2 / 3 / 4 loads
-#else
             // all but the newest load when that is the previous step's prefetch, else all
             if constexpr (kPrefetch) __builtin_amdgcn_s_waitcnt(0x0071);
             else __builtin_amdgcn_s_waitcnt(0x0070);
-#endif
-#ifdef FMA_PROF
-            PROF_STAMP(pt1);
-#endif
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-#ifdef FMA_PROF
-            PROF_STAMP(pt2);
-            prof_wait += pt1 - pt0;
-            prof_bar += pt2 - pt1;
-            prof_steps += 1;
-#endif
             // unconditional (after the last step the fragments are simply not used): straight-line code lets the
             // compiler count outstanding LDS reads exactly, so the MFMAs below do not wait for these reads
             load_frags(fa_c, stage ^ 1, 0, 0);
             // past the end of K the loads are all out of range (zero-fill), which keeps the loop body free of branches
-#if defined(FMA_DIAG) && FMA_DIAG >= 5
-            // timing only (wrong results): the last loads of the burst belong to step kt+3, so that they are not waited
-            // for at the next barrier; what a partial third stage would allow
-            issue_some(std::integral_constant<int, 0>{}, std::integral_constant<int, 8 - (FMA_DIAG - 3)>{}, stage, (kt + 2) * BK);
-            issue_some(std::integral_constant<int, 8 - (FMA_DIAG - 3)>{}, std::integral_constant<int, FMA_DIAG - 3>{}, stage, (kt + 3) * BK);
-#else
             issue_some(std::integral_constant<int, 0>{}, L3{}, stage, (kt + 2) * BK);
-#endif
             // the prefetch goes out behind this step's loads (the empty statement orders it: the wait of the next step
             // counts on it being the newest load) and has until the wait of the step after next to complete
             if constexpr (kPrefetch) asm volatile("" : "+v"(pf_voff));
@@ -586,7 +532,7 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             mma(fa_c, 1);
             if constexpr (FA > 0) {
                 __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);
-                spread_mfma_vmem<0, FA * FN, FMA_LD_S3>();
+                spread_mfma_vmem<0, FA * FN, kLoadsS3>();
                 if constexpr (kPrefetch) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
             }
         };
@@ -684,26 +630,11 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                 issue_quiet_a(1, BK);
                 if (!prefetched_b1) issue_quiet_b(1, BK);
             }
-#ifdef FMA_PROF
-            PROF_SEG(2);  // rest of the first loads issued
-#endif
             nxt = lookup(++round);  // in the shadow of the loads
-#ifdef FMA_PROF
-            PROF_SEG(3);  // look-up of the tile after
-#endif
             // the first K step's loads have landed; the second step's, and the previous tile's stores, may still be out
             wait_outstanding((prefetched ? tile_stores : 0u) + (KT > 1 ? kStepLoads : 0u));
-#ifdef FMA_PROF
-            PROF_SEG(4);  // wait for the first K step's operands
-#endif
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-#ifdef FMA_PROF
-            PROF_SEG(5);  // barrier
-#endif
-#ifdef FMA_PROF
-            if (prof_e0) { uint64_t t; PROF_STAMP(t); prof_edge += t - prof_e0; }
-#endif
             issue_prefetch(kPfDist - 1);
             auto k_loop = [&](auto fa_c) {
                 load_frags(fa_c, 0, 0, 0);
@@ -725,10 +656,6 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
             __builtin_amdgcn_s_waitcnt(0x0f70);
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-#ifdef FMA_PROF
-            PROF_STAMP(prof_e0);
-            prof_t = prof_e0;
-#endif
         }
 
         // ---- next tile: its first loads go out now, into stage 0, and fly while this tile's results are stored ----
@@ -745,9 +672,6 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                 prefetched_b1 = true;
             }
         }
-#ifdef FMA_PROF
-        PROF_SEG(0);  // next tile's loaders set up and first loads issued
-#endif
 
         // ---- epilogue ----
         // Past the last barrier of the K loop nobody reads the LDS stages any more. The A half of stage 1 is the staging
@@ -829,23 +753,8 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
                 stage_flush<YB, 32>(img, args.ACT + off_d / 2 + (uint64_t)row0 * n_span + col0, n_span, rows_valid, cols_valid, el);
             }
         }
-#ifdef FMA_PROF
-        PROF_SEG(1);  // epilogue
-#endif
         cur = nxt;
     }
-#ifdef FMA_PROF
-    {
-        uint64_t t;
-        PROF_STAMP(t);
-        if (lane == 0) {
-            unsigned long long* o = fma_prof + ((size_t)blockIdx.x * 8 + wave) * 8;
-            o[0] = prof_wait; o[1] = prof_bar; o[2] = prof_steps; o[3] = t - prof_start; o[4] = prof_edge;
-            unsigned long long* o2 = fma_prof + 1024 * 8 * 8 + ((size_t)blockIdx.x * 8 + wave) * 8;
-            for (int i = 0; i < 6; ++i) o2[i] = prof_seg[i];
-        }
-    }
-#endif
 }
 
 // wavefronts per workgroup: kWavesM x kWavesN = eight 128x64 wave tiles (the hand-counted waits are written for eight)
@@ -884,11 +793,6 @@ int launch_plain(const GemmArgs& args, bool a_kc, bool b_kc, hipStream_t st) {
 
 extern "C" {
 
-#ifdef FMA_PROF
-int fma_debug_prof(void* host, int64_t bytes) {
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(fmahip::gemm::fma_prof), (size_t)bytes, 0, hipMemcpyDeviceToHost);
-}
-#endif
 
 int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_arr, const uint32_t* N_arr,
                      const uint32_t* K_arr, int64_t E, int trans_a, int trans_b, float alpha, int dtype,

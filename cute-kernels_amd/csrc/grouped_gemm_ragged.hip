@@ -32,16 +32,9 @@ namespace fmahip {
 namespace gemm {
 namespace ragged {
 
-#ifndef FMA_PF_DIST
-#define FMA_PF_DIST 4
-#endif
-constexpr uint32_t kPfDist = FMA_PF_DIST;
-#ifndef FMA_STREAM_OUT_ALL_LAYOUTS
-#define FMA_STREAM_OUT_ALL_LAYOUTS 0
-#endif
-#ifndef FMA_BWD_AHEAD
-#define FMA_BWD_AHEAD 2  // passes of the SwiGLU-gradient epilogue whose h values are requested ahead
-#endif  // K steps between a line's prefetch and the step that loads it
+constexpr uint32_t kPfDist = 4;     // K steps between a line's prefetch and the step that loads it
+constexpr int kBwdAhead = 2;        // passes of the SwiGLU-gradient epilogue whose h values are requested ahead
+constexpr uint32_t kStreamOutSteps = 16;  // weight-gradient tiles of at most this many K steps store with the non-temporal hint
 
 constexpr int NWM = 2, NWN = 4, NW = NWM * NWN, NT = NW * 64;
 constexpr int WM = BM / NWM, WN = BN / NWN;  // 128 x 64 per wavefront
@@ -990,12 +983,9 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
 #pragma unroll
             for (int i = 0; i < RB; ++i) acc[i] *= alpha;
         }
-#ifndef FMA_STREAM_OUT_STEPS
-#define FMA_STREAM_OUT_STEPS 16
-#endif
         // Tiles with a short reduction write much per flop (a weight gradient over ~500 rows: 8 K steps per 128 KB tile):
         // their stores carry the non-temporal hint (+4 to 5 % there); for long reductions plain stores are faster by 0 to 1 %
-        const bool stream_out = FMA_STREAM_OUT_ALL_LAYOUTS ? KT <= FMA_STREAM_OUT_STEPS : (VARY_K && KT <= FMA_STREAM_OUT_STEPS);
+        const bool stream_out = VARY_K && KT <= kStreamOutSteps;
         // BIAS: the four groups of four columns this lane holds of every row block, as fp32
         float bias_f[CB][4];
         if constexpr (BIAS) {
@@ -1110,7 +1100,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                     // The product (rounded) is the gradient of the activation; h and its gradient are [rows, 2 Ne] with "up" in
                     // columns 0.., "gate" in columns Ne... A pass is 16 rows x 64 columns: a lane takes 8 columns of two rows,
                     // fetches the 8 up and 8 gate values of each (requested two passes ahead), and stores both gradients.
-                    constexpr int kAhead = FMA_BWD_AHEAD;
+                    constexpr int kAhead = kBwdAhead;
                     if (i == 0) {
 #pragma unroll
                         for (int a = 0; a < kAhead; ++a) bwd_request(a, col0, cols_valid);

@@ -18,12 +18,9 @@ namespace {
 
 constexpr int kNormThreads = 256;
 constexpr int kNormWaves = kNormThreads / kWave;
-#ifndef FMA_NORM_BWD_WORKGROUPS_PER_CU
-#define FMA_NORM_BWD_WORKGROUPS_PER_CU 2
-#endif
 // chunks of rows (= rows of the weight-gradient workspace) per compute unit; measured on [16384, 4096] bf16: 1 -> 214 us,
 // 2 -> 143 us, 3 -> 151 us, 4 -> 173 us, 8 -> 162 us for both launches
-constexpr int kBwdWorkgroupsPerCU = FMA_NORM_BWD_WORKGROUPS_PER_CU;
+constexpr int kBwdWorkgroupsPerCU = 2;
 
 struct Sum2 {
     float a, b;

@@ -526,10 +526,6 @@ int launch_router_wide(const RouterArgs& a, hipStream_t st) {
     return launch_status("router_topk");
 }
 
-#ifndef FMA_ROUTER_FORCE_RB
-#define FMA_ROUTER_FORCE_RB 0  // tuning builds: 1, 2 or 4 row blocks per workgroup regardless of T
-#endif
-
 template <typename EL, int NBLK, int RB, int EMAX>
 int launch_router_as(const RouterArgs& a, hipStream_t st) {
     const int64_t toks = (int64_t)RB * kTok;
@@ -546,7 +542,6 @@ int launch_router_rows(const RouterArgs& a, hipStream_t st) {
     int rb = 1;
     if (RBMAX >= 4 && a.T >= want * 4 * kTok) rb = 4;
     else if (RBMAX >= 2 && a.T >= want * 2 * kTok) rb = 2;
-    if (FMA_ROUTER_FORCE_RB) rb = FMA_ROUTER_FORCE_RB <= RBMAX ? FMA_ROUTER_FORCE_RB : RBMAX;
     if constexpr (RBMAX >= 4)
         if (rb == 4) return launch_router_as<EL, NBLK, 4, EMAX>(a, st);
     if constexpr (RBMAX >= 2)
