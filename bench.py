@@ -304,6 +304,31 @@ def measure_workload(name, args, full):
     mfma("up_projection_wgrad(TN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, xg, dw1, counts, VARY_K, 2 * I, H, 0, 1, 0),
          nbytes=R * 2 * I * s + R * H * s + w1_b)
 
+    # The public op, fma_grouped_gemm (per-group M, N and K arrays in device memory: three launches of which one works), on
+    # the shape of the reference's own test (tests/ops/grouped_gemm_test.py:38-52: E=16, N=512, K=4096, sum M = 65536), in
+    # the three layouts the layer uses, and the same NT problem through the one-size-array entry point the layer calls
+    if full and want("grouped_gemm_op"):
+        Mo = [512, 3176, 2048] * 5 + [36856]
+        Eo, No, Ko, Ro = len(Mo), 512, 4096, sum(Mo)
+        m_o = torch.tensor(Mo, dtype=torch.int32, device=dev).view(torch.uint32)
+        n_o, k_o = torch.full_like(m_o, No), torch.full_like(m_o, Ko)
+        a_o = torch.randn(Ro * Ko, device=dev).bfloat16()
+        b_o = (torch.randn(Eo * No * Ko, device=dev) * 0.02).bfloat16()
+        d_o2 = torch.empty(Ro * No, **bf)
+        if args.zero_operands:
+            a_o.zero_(), b_o.zero_()
+        fl_o = 2.0 * Ro * No * Ko
+        by_o = (Ro * Ko + Eo * No * Ko + Ro * No) * s
+        for lname, ta, tb in (("NT", 0, 1), ("NN", 0, 0), ("TN", 1, 0)):
+            mfma(f"grouped_gemm_op({lname}, E=16 N=512 K=4096 sum M=65536, 3 launches)", fl_o,
+                 lambda i: ok(lib.fma_grouped_gemm(a_o.data_ptr(), b_o.data_ptr(), d_o2.data_ptr(), m_o.data_ptr(),
+                                                   n_o.data_ptr(), k_o.data_ptr(), Eo, ta, tb, 1.0, BF16, stream)),
+                 nbytes=by_o)
+        mfma("grouped_gemm_op_shape_through_ragged_entry(NT, 1 launch)", fl_o,
+             lambda i: ok(lib.fma_grouped_gemm_ragged(a_o.data_ptr(), b_o.data_ptr(), d_o2.data_ptr(), m_o.data_ptr(), None, Eo,
+                                                      VARY_M, 0, No, Ko, 0, 1, 1.0, BF16, stream)), nbytes=by_o)
+        del a_o, b_o, d_o2
+
     # the fp32 grouped GEMM (fp32 matrix instruction, 157.3 TFLOP/s peak) on the down-projection's forward shape;
     # only on request (--only fp32): it is not part of the bf16 layer and takes 40 ms per launch
     if only and want("down_projection_fwd_fp32(NT)"):
@@ -498,6 +523,19 @@ def measure_workload(name, args, full):
         expect = np.bincount(make_ids(n_ids, bins, kind, seed=100 + 49 % 5), minlength=bins)
         assert np.array_equal(out_cnt.cpu().view(torch.int32).numpy().astype(np.int64), expect), "count mismatch"
         del ids
+    # The same histogram over 256 Mi ids (1 GiB per launch, two buffers rotated): the launch's fixed cost (second launch,
+    # ramp-up) is then a few percent of the time and the figure is the rate the count kernel streams at.
+    if want("continuous_count_256Mi_uniform"):
+        n_big = 256 << 20
+        ws_big = torch.empty(lib.fma_continuous_count_workspace_bytes(n_big, bins), dtype=torch.uint8, device=dev)
+        out_big = torch.empty(bins, dtype=torch.uint32, device=dev)
+        big = [torch.randint(0, bins, (n_big,), dtype=torch.int32, device=dev) for _ in range(2)]
+        hbm("continuous_count_256Mi_uniform", n_big * 4 + bins * 4,
+            lambda i: ok(lib.fma_continuous_count(big[i % 2].data_ptr(), 4, n_big, out_big.data_ptr(), bins,
+                                                  ws_big.data_ptr(), ws_big.numel(), stream)), n=20, warmup=3)
+        expect_big = torch.bincount(big[19 % 2], minlength=bins)
+        assert torch.equal(out_big.view(torch.int32).long(), expect_big), "count mismatch (256 Mi ids)"
+        del big, ws_big
     return layer, kernels, context
 
 
@@ -517,61 +555,37 @@ def cpu_baseline(context, name):
     def progress(msg):  # keeps a watchdog that looks for output quiet during the CPU leg
         print(f"bench.py: cpu baseline: {msg}", file=sys.stderr, flush=True)
 
-    def timed_leg(dtype, T_cpu, budget_s):
-        """seconds per forward + backward step of the first T_cpu tokens in dtype, number of steps; None if the first
-        step alone exceeds twice the budget"""
-        sel_c, w_c = selected[:T_cpu], weights[:T_cpu].to(dtype).requires_grad_()
-        x_c = x[:T_cpu].cpu().to(dtype).requires_grad_()
-        w1_c = moe.c_fc.weight.detach().cpu().to(dtype).requires_grad_()
-        w2_c = moe.c_proj.weight.detach().cpu().to(dtype).requires_grad_()
-        dy_c = dy[:T_cpu].cpu().to(dtype)
+    # One fixed configuration whatever the host's speed, so that the figure compares between runs: bf16, the first T/16
+    # tokens, one warm-up step and three timed ones (about 2 s per step on the hosts measured).
+    dtype, T_cpu, n = torch.bfloat16, max(64, T // 16), 3
+    sel_c, w_c = selected[:T_cpu], weights[:T_cpu].to(dtype).requires_grad_()
+    x_c = x[:T_cpu].cpu().to(dtype).requires_grad_()
+    w1_c = moe.c_fc.weight.detach().cpu().to(dtype).requires_grad_()
+    w2_c = moe.c_proj.weight.detach().cpu().to(dtype).requires_grad_()
+    dy_c = dy[:T_cpu].cpu().to(dtype)
 
-        def cpu_step():
-            for t in (x_c, w_c, w1_c, w2_c):
-                t.grad = None
-            O.moe_experts(x_c, w_c, sel_c, w1_c, w2_c).backward(dy_c)
+    def cpu_step():
+        for t in (x_c, w_c, w1_c, w2_c):
+            t.grad = None
+        O.moe_experts(x_c, w_c, sel_c, w1_c, w2_c).backward(dy_c)
 
-        progress(f"{dtype}, {T_cpu} tokens on {cores} threads, warm-up step")
-        t0 = time.perf_counter()
+    progress(f"{dtype}, {T_cpu} tokens on {cores} threads, warm-up step")
+    cpu_step()
+    t0 = time.perf_counter()
+    for i in range(n):
         cpu_step()
-        first = time.perf_counter() - t0
-        progress(f"warm-up step took {first:.1f} s")
-        if first > 2 * budget_s:
-            return None, first
-        n, t0 = 0, time.perf_counter()
-        while n < 1 or (time.perf_counter() - t0 < budget_s and n < 50):
-            cpu_step()
-            n += 1
-            progress(f"step {n}, {time.perf_counter() - t0:.1f} s")
-        return (time.perf_counter() - t0) / n, n
-
-    # bf16 on the first T/16 tokens, as long as that fits the time box (about 30 s of CPU
-    # work). A first bf16 step on T/64 tokens sizes it: if four times its duration is beyond the box the sample stays at
-    # T/64 tokens, and if the host's bf16 kernels are so slow that even that step takes more than 10 s the leg runs in fp32.
-    note = ""
-    dtype, T_cpu = torch.bfloat16, max(64, T // 64)
-    cpu_s, n = timed_leg(dtype, T_cpu, 5.0)
-    if cpu_s is None:
-        note = f" (one bf16 step of {T_cpu} tokens took {n:.0f} s on this host, beyond the time box: fp32 instead)"
-        dtype = torch.float32
-        cpu_s, n = timed_leg(dtype, T_cpu, 10.0)
-        if cpu_s is None:
-            cpu_s, n = n, 1
-    elif 4 * cpu_s <= 30.0:
-        T_cpu = max(64, T // 16)
-        cpu_s, n = timed_leg(dtype, T_cpu, 15.0)
-        if cpu_s is None:
-            cpu_s, n = n, 1
-    else:
-        note = f" (T/16 tokens would take about {4 * cpu_s:.0f} s per step on this host, beyond the time box)"
+        progress(f"step {i + 1} of {n}, {time.perf_counter() - t0:.1f} s")
+    wall = time.perf_counter() - t0
+    cpu_s = wall / n
     out = {
         "value": T_cpu / cpu_s,
         "unit": "tokens/s",
         "cores": cores,
         "kind": "port",
         "sample": f"first {T_cpu} of {T} tokens of the {name} workload (same H, I, E, k, same routing), {dtype} eager torch on "
-        f"the host CPU, forward + backward, mean of {n} steps{note}. Not linear in the token count: the weight-gradient "
-        "pass writes (and the step then zeroes) the full-size expert weights whatever the number of tokens.",
+        f"the host CPU, forward + backward, mean of {n} steps after one warm-up step ({wall:.1f} s of wall time). Not linear "
+        "in the token count: the weight-gradient pass writes (and the step then zeroes) the full-size expert weights whatever "
+        "the number of tokens.",
     }
     # continuous_count beside it: torch.bincount, the routine the reference's torch backend calls
     # (fma/ops/continuous_count/__init__.py:36), on the same 16 Mi int32 ids on the host

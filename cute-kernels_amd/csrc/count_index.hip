@@ -543,7 +543,14 @@ int fma_moe_build_index_from_hist(const int32_t* ids, int64_t R, int64_t E, int6
                                         (hipStream_t)stream);
 }
 
-int64_t fma_moe_build_index_static_max_words(void) { return FMA_STATIC_INDEX_WORDS; }
+int64_t fma_moe_build_index_static_max_words(void) {
+    // The first call on a device looks the array's address up (hipGetSymbolAddress, under a mutex). Doing it here, where a
+    // caller asks for the limit before its first build, keeps that lookup out of a stream capture; the result is ignored
+    // (a failure is reported by the build itself).
+    uint32_t* unused = nullptr;
+    (void)fmahip::static_scratch(&unused);
+    return FMA_STATIC_INDEX_WORDS;
+}
 
 int fma_moe_build_index_static(const void* ids, int id_bytes, int64_t R, int64_t E, uint32_t* counts, uint32_t* offsets,
                                int32_t* perm, int32_t* eid, int32_t* inv, void* stream) {

@@ -88,10 +88,12 @@ __device__ __forceinline__ u32x4 uniform(u32x4 x) {
 // The same load written in assembly, with its M0 set-up (M0 holds the LDS address the wavefront's 1 KB goes to). The
 // compiler does not see that it writes LDS, so it places no waits of its own for it: the first loads of a tile are
 // issued this way, partly while the previous tile's epilogue is still running, and waited for with an exact count.
+// (s_nop 2: the scalar operands may come from a v_readfirstlane right in front of the assembly, and a vector-memory
+// instruction must not read such a register within five wait states; the compiler does not check assembly for that.)
 __device__ __forceinline__ void buffer_load_lds_quiet(u32x4 rsrc, uint32_t voff, uint32_t soff, uint32_t lds_addr) {
     // M0 is put back afterwards: the compiler keeps its own values in it and does not honour a clobber of it
     uint32_t saved_m0;
-    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %4\n\ts_nop 2\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
                  "s_mov_b32 m0, %0"
                  : "=&s"(saved_m0)
                  : "v"(voff), "s"(uniform(rsrc)), "s"(uniform(soff)), "s"(uniform(lds_addr)));
@@ -99,7 +101,7 @@ __device__ __forceinline__ void buffer_load_lds_quiet(u32x4 rsrc, uint32_t voff,
 // the 4-byte form of the same load (64 lanes x 4 bytes = 256 bytes of LDS per instruction)
 __device__ __forceinline__ void buffer_load_lds_quiet_b32(u32x4 rsrc, uint32_t voff, uint32_t soff, uint32_t lds_addr) {
     uint32_t saved_m0;
-    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %4\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds\n\t"
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %4\n\ts_nop 2\n\tbuffer_load_dword %1, %2, %3 offen lds\n\t"
                  "s_mov_b32 m0, %0"
                  : "=&s"(saved_m0)
                  : "v"(voff), "s"(uniform(rsrc)), "s"(uniform(soff)), "s"(uniform(lds_addr)));
@@ -160,6 +162,13 @@ __device__ __forceinline__ s16x8 read_kc_frag(const uint8_t* p) { return *reinte
 template <bool NT>
 __device__ __forceinline__ void store_tile16(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint4 v) {
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc, (int)voff, 0, NT ? 2 : 0);
+}
+// The same store with the non-temporal hint, written in assembly: for an epilogue whose store COUNT the next tile's waits
+// rely on, where nothing may merge, split or drop one. rsrc: the descriptor as four words (make_rsrc_words). A vector
+// instruction that overwrites the data registers must not follow a 16-byte store directly; the compiler places that wait
+// state behind its own stores only, so it is part of the assembly here.
+__device__ __forceinline__ void store_tile16_quiet_nt(u32x4 rsrc, uint32_t voff, u32x4 v) {
+    asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen nt\n\ts_nop 1" ::"v"(v), "v"(voff), "s"(uniform(rsrc)) : "memory");
 }
 template <int ROWB>
 __device__ __forceinline__ uint32_t stage_off(uint32_t m, uint32_t chunk16) {

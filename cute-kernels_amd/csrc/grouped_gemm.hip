@@ -52,6 +52,9 @@ struct GemmArgs {
     uint32_t const_n;
     uint32_t const_k;
     float alpha;
+    // fma_grouped_gemm also offers its launch to the kernels of grouped_gemm_ragged.hip, which take it when the groups differ
+    // in one dimension only; with this flag set the kernel here applies the same test and ends at once in that case
+    uint32_t only_if_irregular;
 };
 
 template <typename EL, int NWM, int NWN, bool A_KC, bool B_KC, int EPI>
@@ -91,6 +94,18 @@ __global__ __launch_bounds__(NWM* NWN * 64) void grouped_gemm_kernel(const GemmA
     auto group_m = [&](uint32_t e) { return m_arr ? m_arr[e] : args.const_m; };
     auto group_n = [&](uint32_t e) { return n_arr ? n_arr[e] : args.const_n; };
     auto group_k = [&](uint32_t e) { return k_arr ? k_arr[e] : args.const_k; };
+    if (args.only_if_irregular) {
+        // (the test of ragged_gemm_kernel: rows vary with N and K shared, or the reduction varies with M and N shared)
+        const uint32_t m0 = group_m(0), n0 = group_n(0), k0 = group_k(0);
+        bool m_differs = false, n_differs = false, k_differs = false;
+        for (uint32_t e = tid; e < E; e += NT) {
+            m_differs = m_differs || args.M_arr[e] != m0;
+            n_differs = n_differs || args.N_arr[e] != n0;
+            k_differs = k_differs || args.K_arr[e] != k0;
+        }
+        const bool m_same = !__syncthreads_or(m_differs), n_same = !__syncthreads_or(n_differs), k_same = !__syncthreads_or(k_differs);
+        if ((n_same && k_same) || (m_same && n_same)) return;
+    }
     // Column tiles of half the width for groups of at most 64 rows (a few rows per group: the kernel is then a stream of
     // the B operand), when that fills the workgroups better: a launch with tiles for at most half of them, or one made of
     // such groups only whose last round of tiles would be at most half full. Decided once per launch, below, from the
@@ -791,8 +806,15 @@ int launch_plain(const GemmArgs& args, bool a_kc, bool b_kc, hipStream_t st) {
 }  // namespace gemm
 }  // namespace fmahip
 
-extern "C" {
+namespace fmahip {
+namespace gemm {
+// grouped_gemm_ragged.hip
+int launch_ragged_from_arrays(const void* A, const void* B, void* D, const uint32_t* M_arr, const uint32_t* N_arr,
+                              const uint32_t* K_arr, int64_t E, bool a_kc, bool b_kc, float alpha, int dtype, hipStream_t st);
+}  // namespace gemm
+}  // namespace fmahip
 
+extern "C" {
 
 int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_arr, const uint32_t* N_arr,
                      const uint32_t* K_arr, int64_t E, int trans_a, int trans_b, float alpha, int dtype,
@@ -811,6 +833,12 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
     const bool a_kc = trans_a == 0;  // A stored [M, K]: reduction dim contiguous
     const bool b_kc = trans_b != 0;  // B stored [N, K]: reduction dim contiguous
     if (dtype == FMA_F32) return gemm_f32::launch(A, B, D, M_arr, N_arr, K_arr, E, a_kc, b_kc, alpha, st);
+    // Three launches, of which one does the work: the group sizes live in device memory, so each kernel decides for itself
+    // (reading the arrays costs a kernel that then ends about 2 us). Launches whose groups differ in one dimension only
+    // (every grouped GEMM of an MoE layer, the reference's own test shapes) go to the streaming kernels of
+    // grouped_gemm_ragged.hip, anything else to the kernel of this file.
+    const int rc = launch_ragged_from_arrays(A, B, D, M_arr, N_arr, K_arr, E, a_kc, b_kc, alpha, dtype, st);
+    if (rc != FMA_OK) return rc;
     GemmArgs args{};
     args.A = (const uint16_t*)A;
     args.B = (const uint16_t*)B;
@@ -821,6 +849,7 @@ int fma_grouped_gemm(const void* A, const void* B, void* D, const uint32_t* M_ar
     args.K_arr = K_arr;
     args.E = (uint32_t)E;
     args.alpha = alpha;
+    args.only_if_irregular = 1u;
     return dtype == FMA_BF16 ? launch_plain<ElemBf16>(args, a_kc, b_kc, st) : launch_plain<ElemF16>(args, a_kc, b_kc, st);
 }
 

@@ -55,6 +55,11 @@ struct Args {
     uint32_t E;
     uint32_t m, n, k;  // the dimensions all groups share (the varying one is ignored)
     float alpha;
+    // fma_grouped_gemm (per-group M, N and K arrays in device memory): when n_dev is set, the shared dimensions are the
+    // first entries of the arrays, and the kernel runs only if the launch has its form (see the top of the kernel)
+    const uint32_t* m_dev;
+    const uint32_t* n_dev;
+    const uint32_t* k_dev;
 };
 
 // s_waitcnt immediate: vmcnt(vm), and lgkmcnt(0) too if lgkm0 (expcnt untouched)
@@ -114,6 +119,28 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     const uint32_t wn = wave % NWN;
     const uint32_t E = args.E;
 
+    // The dimensions all groups share. Called with per-group arrays of all three dimensions (fma_grouped_gemm), the kernel
+    // first looks whether the launch has its form: rows vary -> N and K the same for every group; reduction varies -> M and
+    // N the same and K not (when all three are the same the rows-vary kernel runs). If not, it leaves the launch to the
+    // kernel launched beside it: the three kernels of fma_grouped_gemm agree on one of them without a word to the host.
+    uint32_t dim_m = args.m, dim_n = args.n, dim_k = args.k;
+    if (args.n_dev) {
+        typedef const __attribute__((address_space(4))) uint32_t* const_dim_ptr;
+        const const_dim_ptr ma = (const_dim_ptr)args.m_dev, na = (const_dim_ptr)args.n_dev, ka = (const_dim_ptr)args.k_dev;
+        dim_m = ma[0];
+        dim_n = na[0];
+        dim_k = ka[0];
+        bool m_differs = false, n_differs = false, k_differs = false;
+        for (uint32_t e = tid; e < E; e += NT) {
+            m_differs = m_differs || args.m_dev[e] != dim_m;
+            n_differs = n_differs || args.n_dev[e] != dim_n;
+            k_differs = k_differs || args.k_dev[e] != dim_k;
+        }
+        const bool m_same = !__syncthreads_or(m_differs), n_same = !__syncthreads_or(n_differs), k_same = !__syncthreads_or(k_differs);
+        const bool mine = VARY_K ? (m_same && n_same && !k_same) : (n_same && k_same);
+        if (!mine) return;
+    }
+
     // The compiler orders LDS accesses behind direct-to-LDS loads in flight per LDS object: an access to an object that
     // some load has written waits for the loads into THAT object only, an access to an object no load has ever written
     // waits for all of them. The group table is read while the next tile's operand loads are in flight, so it gets
@@ -129,9 +156,9 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     // (nothing writes the array while the kernel runs), not a vector load that every tile would wait for.
     typedef const __attribute__((address_space(4))) uint32_t* const_u32_ptr;
     const const_u32_ptr sizes = (const_u32_ptr)args.sizes;
-    auto group_m = [&](uint32_t e) { return VARY_K ? args.m : sizes[e]; };
-    auto group_k = [&](uint32_t e) { return VARY_K ? sizes[e] : args.k; };
-    const uint32_t Ne = args.n;
+    auto group_m = [&](uint32_t e) { return VARY_K ? dim_m : sizes[e]; };
+    auto group_k = [&](uint32_t e) { return VARY_K ? sizes[e] : dim_k; };
+    const uint32_t Ne = dim_n;
     constexpr bool kCanNarrow = A_KC && B_KC;
     constexpr uint32_t kTileN = kGlu ? BN / 2 : BN;  // columns of the tile grid one tile covers
     const uint32_t n_span = kGlu ? Ne / 2 : Ne;      // columns the tile grid runs over
@@ -293,13 +320,13 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         // packed element offsets of the group: the varying dimension's prefix times the other dimension of the operand
         const uint64_t before = uniform(s_prefix[e]);
         if constexpr (VARY_K) {
-            t.off_a = before * args.m;
+            t.off_a = before * dim_m;
             t.off_b = before * Ne;
-            t.off_d = (uint64_t)e * args.m * Ne;
+            t.off_d = (uint64_t)e * dim_m * Ne;
         } else {
             t.row0 = (uint32_t)before;
-            t.off_a = before * args.k;
-            t.off_b = (uint64_t)e * Ne * args.k;
+            t.off_a = before * dim_k;
+            t.off_b = (uint64_t)e * Ne * dim_k;
             t.off_d = before * Ne;
         }
         // 16-byte accesses need every contiguous dimension a multiple of 8 elements and packed group bases that stayed
@@ -372,8 +399,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     // The tile of round r keeps the row_index entries of its 256 rows in half r % 2 of s_rows. A wavefront's four load
     // instructions of a K step fetch tile rows g_row, g_row + 64, + 128, + 192 of this lane: four table entries, divided by
     // the divisor, times the row pitch. Entries past the group's rows read as zero (row 0 of A: rows never stored).
-    const uint32_t g_full = GATHER ? args.a_rows * args.k * 2u : 0u;  // bytes of A (below 2^31)
-    const uint32_t g_ldb = args.k * 2u;
+    const uint32_t g_full = GATHER ? args.a_rows * dim_k * 2u : 0u;  // bytes of A (below 2^31)
+    const uint32_t g_ldb = dim_k * 2u;
     const uint32_t g_row = logical_row(wave * 8u + (lane >> 3));
     const uint32_t g_chunk = (lane & 7u) ^ (g_row & 7u);
     // n / divisor for n < 2^31: the high word of n * ceil(2^32 / divisor) is the quotient or one more
@@ -391,11 +418,15 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         uint32_t n[4];
         lds_read4_stride64_quiet(lds_address(reinterpret_cast<const uint8_t*>(s_rows)) + half * 1024u + g_row * 4u, n);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = g_source_row(n[i]) * g_ldb + g_chunk * 16u;
+        for (int i = 0; i < 4; ++i) {
+            // an entry that names no row of A (negative, or past the last row) reads as a row of zeros
+            const uint32_t src = g_source_row(n[i]);
+            v[i] = (n[i] < 0x80000000u && src < args.a_rows) ? src * g_ldb + g_chunk * 16u : kOutOfRange;
+        }
     };
     // last, partial K step: chunks past the end of K are pushed out of range, which zero-fills them
     auto g_clip = [&](uint32_t k0, uint32_t (&v)[4]) {
-        const bool past = k0 + (uint32_t)BK > args.k && k0 + g_chunk * 8u >= args.k;
+        const bool past = k0 + (uint32_t)BK > dim_k && k0 + g_chunk * 8u >= dim_k;
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = past ? kOutOfRange : v[i];
     };
@@ -434,7 +465,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 const uint32_t n = lds_read1_quiet(lds_address(reinterpret_cast<const uint8_t*>(s_rows)) + (round & 1u) * 1024u +
                                                    (lane < 16u ? 4u * i + t.pf_c : 0u) * 4u);
                 pf_base = args.A; pf_bytes = g_full;
-                pf_voff = lane < 16u ? g_source_row(n) * g_ldb : kOutOfRange;
+                pf_voff = (lane < 16u && n < 0x80000000u && g_source_row(n) < args.a_rows) ? g_source_row(n) * g_ldb : kOutOfRange;
             } else if constexpr (A_KC) {
                 pf_base = fa_cur.base0; pf_bytes = fa_cur.extent;
                 pf_voff = lane < 16u ? (4u * i + t.pf_c) * (t.Ke * 2u) : kOutOfRange;
@@ -1046,7 +1077,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 const uint32_t c16 = el & 7u;
                 u32x4 dy[2];
                 stage_get2_quiet(img, stage_off<WN * 2>(el >> 3, c16), stage_off<WN * 2>(8u + (el >> 3), c16), dy[0], dy[1]);
-                const __amdgpu_buffer_rsrc_t rs = make_rsrc(args.D + bwd_origin(pass, col0), bwd_rows(pass) * (Ne * 4u));
+                const u32x4 rs = make_rsrc_words(args.D + bwd_origin(pass, col0), bwd_rows(pass) * (Ne * 4u));
 #pragma unroll
                 for (int r = 0; r < 2; ++r) {
                     u32x4 du, dg;
@@ -1070,8 +1101,9 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                     // there (it does for stores with a constant scalar offset, as every other store of this library has).
                     const uint32_t off = bwd_offset(r, cols_valid);
                     const uint32_t off_gate = off == kOutOfRange ? kOutOfRange : off + Ne * 2u;
-                    __builtin_amdgcn_raw_buffer_store_b128(du, rs, (int)off, 0, kStreamAux);
-                    __builtin_amdgcn_raw_buffer_store_b128(dg, rs, (int)off_gate, 0, kStreamAux);
+                    // (in assembly: the next tile's first wait counts these stores, so their number must be exactly this)
+                    store_tile16_quiet_nt(rs, off, du);
+                    store_tile16_quiet_nt(rs, off_gate, dg);
                 }
             }
         };
@@ -1281,6 +1313,29 @@ int up_projection(const char* who, const void* x, int64_t x_rows, const int32_t*
 }
 
 }  // namespace ragged
+
+// fma_grouped_gemm's launch (per-group M, N and K arrays in device memory) offered to the two kernels of this file: each
+// reads the arrays and runs only if the launch has its form (one varying dimension), otherwise it ends at once.
+int launch_ragged_from_arrays(const void* A, const void* B, void* D, const uint32_t* M_arr, const uint32_t* N_arr,
+                              const uint32_t* K_arr, int64_t E, bool a_kc, bool b_kc, float alpha, int dtype, hipStream_t st) {
+    ragged::Args args{};
+    args.A = (const uint16_t*)A;
+    args.B = (const uint16_t*)B;
+    args.D = (uint16_t*)D;
+    args.E = (uint32_t)E;
+    args.alpha = alpha;
+    args.m_dev = M_arr;
+    args.n_dev = N_arr;
+    args.k_dev = K_arr;
+    args.sizes = M_arr;
+    int rc = dtype == FMA_BF16 ? ragged::launch_plain<ElemBf16, false>(args, a_kc, b_kc, st)
+                               : ragged::launch_plain<ElemF16, false>(args, a_kc, b_kc, st);
+    if (rc != FMA_OK) return rc;
+    args.sizes = K_arr;
+    return dtype == FMA_BF16 ? ragged::launch_plain<ElemBf16, true>(args, a_kc, b_kc, st)
+                             : ragged::launch_plain<ElemF16, true>(args, a_kc, b_kc, st);
+}
+
 }  // namespace gemm
 }  // namespace fmahip
 

@@ -238,7 +238,8 @@ int fma_grouped_gemm_swiglu_bwd(const void* dy, const void* W, const void* h, vo
  * i.e. fma_grouped_gemm_ragged (swiglu == 0: out [R, N], act ignored) or fma_grouped_gemm_swiglu (swiglu != 0:
  * N = 2 I, out = the pre-activation h [R, 2 I] or NULL, act [R, I]) applied to the output of
  * fma_gather_rows(x, row_index, R, K, divisor), bit for bit, without that [R, K] buffer ever being written.
- * x: [x_rows, K] with x_rows * K * 2 < 2^31 bytes; every row_index[i] / divisor < x_rows; divisor in [1, 65536]
+ * x: [x_rows, K] with x_rows * K * 2 < 2^31 bytes; an entry row_index[i] that is negative or whose row_index[i] / divisor is
+ * not below x_rows names no row and is taken as a row of zeros (its output row is bias_e, or zero); divisor in [1, 65536]
  * (top_k with row_index = the stable routing order perm of fma_moe_build_index; 1 for a plain row index).
  * N % 8 == 0 (16 for swiglu), K % 8 == 0, N < 2^23, K < 2^21; dtype FMA_BF16 or FMA_F16.
  * Replaces the gather inside the reference's fused Triton expert kernel (fma/modules/moe/triton_implementation/

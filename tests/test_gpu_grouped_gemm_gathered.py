@@ -79,6 +79,25 @@ def test_swiglu_epilogue(counts, T, K, N, divisor, with_bias, dtype):
     assert torch.equal(act_only, act_ref)
 
 
+@pytest.mark.parametrize("counts,T,K,N,divisor", [CASES[0], CASES[3], CASES[5]])
+def test_index_entries_that_name_no_row_read_as_zero_rows(counts, T, K, N, divisor):
+    # negative entries and entries past the last row of x: their rows of the operand are zeros, so the output row is the
+    # bias (plain epilogue); every other row as before
+    x, w, bias, row_index, xg, M = _inputs(counts, T, K, N, divisor, torch.bfloat16, seed=5)
+    R = sum(counts)
+    bad = torch.arange(R, device=DEV) % 7 == 3
+    broken = row_index.clone()
+    broken[bad & (torch.arange(R, device=DEV) % 2 == 0)] = -5
+    broken[bad & (torch.arange(R, device=DEV) % 2 == 1)] = T * divisor + 11
+    xg_zeroed = xg.clone()
+    xg_zeroed[bad] = 0
+    expect = torch.full((R, N), 7.0, dtype=torch.bfloat16, device=DEV)
+    grouped_gemm_ragged_cuda(xg_zeroed, w, expect, M, False, 0, N, K, False, True, bias)
+    got = torch.full((R, N), 7.0, dtype=torch.bfloat16, device=DEV)
+    grouped_gemm_gathered_cuda(x, broken, divisor, w, bias, M, got, None)
+    assert torch.equal(got, expect)
+
+
 def test_repeated_launches_and_the_routing_order():
     # the layer's use: row_index = the stable routing order of T * k slots, divisor = k; three launches into fresh buffers
     T, k, E, K, N = 3000, 2, 8, 256, 512

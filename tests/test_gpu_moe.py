@@ -88,6 +88,11 @@ def test_moe_reference_cases(E, k, H, I, act_name):
     for name, a, b, bar in zip(["output", "input gradient", "c_fc weight gradient", "c_proj weight gradient"], got, ref16, bars):
         err = (a.detach().cpu().float() - b).abs()
         over = err > bar
+        # every tensor of every case is held to the reference's bar as written, with one exception that is named here: the
+        # c_fc weight gradient of the nn.GLU cases (see below)
+        if bool(over.any()) and not (name == "c_fc weight gradient" and act_name == "glu"):
+            raise AssertionError(f"{name} ({act_name}, E={E}, k={k}): {int(over.sum())} elements beyond the reference's bar "
+                                 f"{bar}, largest error {float(err.max()):.4g}")
         if bool(over.any()):
             # The reference's bars are absolute, set on its own seed and GPU. A weight-gradient element is a sum over the 7
             # tokens of (activation gradient) x (input); where the two sides round one activation gradient of magnitude
@@ -96,7 +101,8 @@ def test_moe_reference_cases(E, k, H, I, act_name):
             # in 2.7e8, all in c_fc's gradient of the nn.GLU cases, the HIP result closer to the fp32 oracle than the bf16
             # oracle is on average. Accepted: at most one element per million beyond the bar, none beyond twice the bar.
             print(f"{name}: {int(over.sum())} of {over.numel()} elements beyond {bar} (largest |expected| among them "
-                  f"{float(b.abs()[over].max()):.4g}, largest error {float(err[over].max()):.4g})")
+                  f"{float(b.abs()[over].max()):.4g}, largest error {float(err[over].max()):.4g}); their (expert, row, "
+                  f"column, error): {[tuple(i) + (round(float(err[tuple(i)]), 4),) for i in over.nonzero().tolist()[:20]]}")
             assert float(err.max()) <= 2 * bar, f"{name}: {float(err.max())} is beyond twice the bar {bar}"
             assert int(over.sum()) <= max(1, over.numel() // 1000000), f"{name}: {int(over.sum())} elements beyond {bar}"
 
