@@ -178,6 +178,10 @@ int fma_swiglu_backward(const void* gate, const void* up, const void* dy, void* 
  * (fp32 runs on the fp32 matrix instruction, one sixteenth of the 16-bit rate, with no restriction on sizes).
  * For the 16-bit types each group's contiguous dimension should be a multiple of 8 elements (16 bytes); other
  * groups are computed by a slow scalar path. E <= FMA_MAX_GROUPS.
+ * The 16-bit call enqueues three kernels of which one does the work: the sizes live in device memory, so each kernel
+ * reads them and runs only if the launch has its form. Launches whose groups differ in one dimension only (every
+ * grouped GEMM of an MoE layer, the reference's own test shapes) are computed by the kernel of
+ * fma_grouped_gemm_ragged, anything else by a general kernel; a kernel that declines ends after reading the arrays.
  * Replaces grouped_gemm_cuda(A, B, C, output, M_array, N_array, K_array, is_A_transposed,
  * is_B_transposed, alpha, beta, benchmark) (fma/ops/grouped_gemm/cuda_implementation/ops.cpp,
  * kernel.cu:354-388); beta must be 0 and C absent there, so neither exists here. */
