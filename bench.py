@@ -129,6 +129,13 @@ def measure_workload(name, args, full):
         return y
 
     steps, warmup = (0, 0) if args.no_layer else (args.steps, args.warmup)
+    if steps:
+        # a fresh process on a fresh box runs its first second of steps 5 to 10 % slower (clocks, allocator, page tables):
+        # that second is spent here, ahead of the warm-up steps the caller asked for
+        t_pre = time.perf_counter()
+        while time.perf_counter() - t_pre < 1.0:
+            step()
+            torch.cuda.synchronize()
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -160,8 +167,23 @@ def measure_workload(name, args, full):
         torch.cuda.synchronize()
         ms_with_router = (time.perf_counter() - t1) * 1e3 / steps
 
-    # the forward alone with autograd off (evaluation / serving): with the first projection gathering its rows through the
-    # routing order, and with the grouped copy of the tokens written first (what the training step above does)
+    # the training step with the choice forced either way: the first projection and its weight gradient gathering their rows
+    # through the routing order, or a grouped copy of the tokens written first (ms_per_step above is the layer's own choice)
+    ms_step = {}
+    if steps:
+        for label, gather in (("gather_in_gemm", True), ("grouped_copy", False)):
+            moe.gather_in_gemm = gather
+            for _ in range(max(1, warmup)):
+                step()
+            torch.cuda.synchronize()
+            t3 = time.perf_counter()
+            for _ in range(steps):
+                step()
+            torch.cuda.synchronize()
+            ms_step[label] = (time.perf_counter() - t3) * 1e3 / steps
+        moe.gather_in_gemm = None
+
+    # the forward alone with autograd off (evaluation / serving), either way
     ms_forward = {}
     if steps:
         for label, gather in (("gather_in_gemm", True), ("grouped_copy", False)):
@@ -187,6 +209,7 @@ def measure_workload(name, args, full):
         "tokens_per_s": tokens_per_s,
         "ms_per_step_with_router": ms_with_router,
         "tokens_per_s_with_router": None if ms_with_router is None else T / (ms_with_router * 1e-3),
+        "ms_per_step_by_row_movement": ms_step or None,
         "ms_forward_no_grad": ms_forward or None,
         "layer_gemm_tflops": gemm_flops_step / (ms_per_step * 1e-3) / 1e12,
         "layer_gemm_frac_of_peak": gemm_flops_step / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
@@ -303,6 +326,12 @@ def measure_workload(name, args, full):
          nbytes=R * 2 * I * s + w1_b + R * H * s)
     mfma("up_projection_wgrad(TN)", 2.0 * R * 2 * I * H, lambda i: gemm(dh, xg, dw1, counts, VARY_K, 2 * I, H, 0, 1, 0),
          nbytes=R * 2 * I * s + R * H * s + w1_b)
+    # the same product with the gather of the routed rows inside the operand load (x read through perm; no xg): with the
+    # gathered forward above, a training step then never writes the grouped copy of the tokens (dispatch_rows below)
+    mfma("up_projection_wgrad_gathered(TN, reduction rows gathered in the operand load)", 2.0 * R * 2 * I * H,
+         lambda i: ok(lib.fma_grouped_gemm_gathered_wgrad(dh.data_ptr(), x.data_ptr(), T, perm.data_ptr(), k, dw1.data_ptr(),
+                                                          counts.data_ptr(), E, 2 * I, H, 1.0, BF16, stream)),
+         nbytes=R * 2 * I * s + T * H * s + R * 4 + w1_b)
 
     # The public op, fma_grouped_gemm (per-group M, N and K arrays in device memory: three launches of which one works), on
     # the shape of the reference's own test (tests/ops/grouped_gemm_test.py:38-52: E=16, N=512, K=4096, sum M = 65536), in
@@ -638,6 +667,7 @@ def main():
             "router": "excluded (routing computed once, outside the timed region); ms_per_step_with_router includes it",
         },
         "ms_per_step_with_router": layer["ms_per_step_with_router"],
+        "ms_per_step_by_row_movement": layer["ms_per_step_by_row_movement"],
         "ms_forward_no_grad": layer["ms_forward_no_grad"],
         "tokens_per_s_with_router": layer["tokens_per_s_with_router"],
         "layer_gemm_tflops": layer["layer_gemm_tflops"],
@@ -671,7 +701,7 @@ def main():
         layer, kernels, context = measure_workload(name, args, full=False)
         del context
         entry = {key: layer[key] for key in ("workload", "ms_per_step", "tokens_per_s", "ms_per_step_with_router",
-                                             "ms_forward_no_grad", "layer_gemm_tflops", "layer_gemm_frac_of_peak")}
+                                             "ms_per_step_by_row_movement", "ms_forward_no_grad", "layer_gemm_tflops", "layer_gemm_frac_of_peak")}
         entry["kernels"] = kernels
         result["workloads"][name] = entry
         torch.cuda.empty_cache()

@@ -49,7 +49,9 @@ struct Args {
     const uint32_t* sizes;  // E values of the varying dimension
     const uint16_t* bias;   // BIAS kernels: [E, n] added to the rounded product before anything else
     const uint16_t* h_in;   // EPI_SWIGLU_BWD: the packed pre-activation [rows, 2 n] whose gradient goes to D
-    // GATHER kernels: row i of the packed A operand is row row_index[i] / divisor of A, which has a_rows rows
+    // GATHER kernels, rows vary: row i of the packed A operand is row row_index[i] / divisor of A, which has a_rows rows.
+    // GATHER kernels, reduction varies (weight gradient): reduction row i of the packed B operand is row
+    // row_index[i] / divisor of B, which has a_rows rows of n elements.
     const int32_t* row_index;
     uint32_t divisor, a_rows;
     uint32_t E;
@@ -81,15 +83,19 @@ struct Feed {
 // Names an accumulator value as one 16-register value (no instruction, no ordering).
 __device__ __forceinline__ void anchor_value(f32x16& c) { asm("" : "+v"(c)); }
 
-template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K, bool BIAS, bool GATHER>
+template <typename EL, bool A_KC, bool B_KC, int EPI, bool VARY_K, bool BIAS, bool GATHER_ANY>
 __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
+    // GATHER: the rows of A are picked through row_index (forward); kGatherK: the reduction rows of B are (weight gradient)
+    constexpr bool GATHER = GATHER_ANY && !VARY_K;
+    constexpr bool kGatherK = GATHER_ANY && VARY_K;
     // kGlu: a forward SwiGLU epilogue (the tile holds 128 "up" and 128 "gate" columns of the product)
     constexpr bool kGlu = EPI == EPI_SWIGLU || EPI == EPI_SWIGLU_ACT;
     static_assert(!kGlu || (A_KC && B_KC && !VARY_K), "the SwiGLU epilogue exists for the NT layout only");
-    static_assert(EPI != EPI_SWIGLU_BWD || (A_KC && !B_KC && !VARY_K && !BIAS && !GATHER),
+    static_assert(EPI != EPI_SWIGLU_BWD || (A_KC && !B_KC && !VARY_K && !BIAS && !GATHER_ANY),
                   "the SwiGLU-gradient epilogue exists for the input-gradient (NN) layout only");
     static_assert(!BIAS || (A_KC && B_KC && !VARY_K), "the bias term exists for the forward (NT) layout only");
-    static_assert(!GATHER || (A_KC && B_KC && !VARY_K), "rows are gathered in the forward (NT) layout only");
+    static_assert(!GATHER || (A_KC && B_KC), "rows are gathered in the forward (NT) layout only");
+    static_assert(!kGatherK || (!A_KC && !B_KC && EPI == EPI_PLAIN), "reduction rows are gathered in the weight-gradient (TN) layout only");
 
     // one array per stage and operand: distinct LDS objects let the compiler see that a direct-to-LDS load
     // into one stage cannot alias the fragment reads of the other, so it does not wait for the load first
@@ -280,7 +286,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         bool valid, fast;
         uint32_t Me, Ke, m0, n0, n_lim;  // n_lim: first column past the tile (kTileN columns wide, or half of that)
         uint32_t e;                      // the group
-        uint32_t row0;                   // rows vary: first packed row of the group
+        uint32_t row0;                   // first packed row (reduction row, if the reduction varies) of the group
         uint64_t off_a, off_b, off_d;
         uint32_t pf_r, pf_c;  // position of the tile in its XCD's 8 x 4 block of tiles (row, column)
     };
@@ -319,12 +325,12 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         t.n_lim = n_span - t.n0 < tile_n ? n_span : t.n0 + tile_n;
         // packed element offsets of the group: the varying dimension's prefix times the other dimension of the operand
         const uint64_t before = uniform(s_prefix[e]);
+        t.row0 = (uint32_t)before;
         if constexpr (VARY_K) {
             t.off_a = before * dim_m;
-            t.off_b = before * Ne;
+            t.off_b = kGatherK ? 0u : before * Ne;  // gathered: the loads address all of B
             t.off_d = (uint64_t)e * dim_m * Ne;
         } else {
-            t.row0 = (uint32_t)before;
             t.off_a = before * dim_k;
             t.off_b = (uint64_t)e * Ne * dim_k;
             t.off_d = before * Ne;
@@ -342,7 +348,9 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     // groups of at most 64 rows run a K loop of their own with a third LDS stage (grouped_gemm.hip); they start cold
     auto is_thin = [&](const Tile& t) { return A_KC && t.Me <= 64u && k_steps(t) >= 3u; };
     // a tile whose first two K steps can be fetched by the tile before it, and which can fetch the next tile's
-    auto streams = [&](const Tile& t) { return t.valid && t.fast && t.Ke > 0 && !is_thin(t); };
+    // (gathered reduction rows: their indices are fetched two K steps ahead of the loads, four ahead of the step itself,
+    // which looks at most one tile ahead if every tile in the stream has four steps)
+    auto streams = [&](const Tile& t) { return t.valid && t.fast && t.Ke > 0 && !is_thin(t) && (!kGatherK || k_steps(t) >= 3u); };
 
     uint32_t round = 0;  // tiles this workgroup has finished
 
@@ -381,7 +389,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         } else {
             lt_b.setup(Be, Ne, t.Ke, t.n0, wave, lane);
             f = Feed<B_KC>{lt_b.base, nullptr, t.Ke, lt_b.ldb, lt_b.col_bytes};
-            v = lt_b.voff;
+            v = kGatherK ? t.row0 : lt_b.voff;  // gathered: where the group's entries of row_index begin (same in every lane)
         }
     };
     // points a loader object at a feed (what depends on lane and wavefront only stays as the last setup left it)
@@ -404,7 +412,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     const uint32_t g_row = logical_row(wave * 8u + (lane >> 3));
     const uint32_t g_chunk = (lane & 7u) ^ (g_row & 7u);
     // n / divisor for n < 2^31: the high word of n * ceil(2^32 / divisor) is the quotient or one more
-    const uint32_t g_magic = (GATHER && args.divisor > 1u) ? (uint32_t)((0x100000000ull + args.divisor - 1u) / args.divisor) : 0u;
+    const uint32_t g_magic = (GATHER_ANY && args.divisor > 1u) ? (uint32_t)((0x100000000ull + args.divisor - 1u) / args.divisor) : 0u;
     auto g_source_row = [&](uint32_t n) -> uint32_t {
         if (args.divisor == 1u) return n;
         uint32_t q = __umulhi(n, g_magic);
@@ -446,7 +454,49 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             if (lane < 32u) buffer_load_lds_quiet_b32(rs, (wave * 32u + lane) * 4u, 0u, to);
         }
     };
-    static_assert(!GATHER || 32 / NW == 4, "four load instructions per wavefront and K step");
+    static_assert(!GATHER_ANY || 32 / NW == 4, "four load instructions per wavefront and K step");
+
+    // ---- kGatherK: the reduction rows of the B operand are rows of args.B picked through args.row_index ----
+    // A wavefront's four load instructions of a K step fetch the step's reduction rows 8 wave + 2 i + (lane >> 5), i = 0..3
+    // (the packed loader's are 16 i + 2 wave + (lane >> 5)): eight consecutive entries of row_index per wavefront and step.
+    // They land where the packed loader puts the same rows: rows 2 s and 2 s + 1 of the step lie in kilobyte s of the stage
+    // either way, so the LDS image, the fragment reads and the order of the sums are those of the packed kernel.
+    // The eight entries are one vector load per wavefront and step (lane l: entry l % 8; a position past the end of
+    // row_index reads as 0), issued two steps ahead of the loads that use them, behind the step's own loads: a step's loads
+    // for K step kt + 2 go out with the entries requested in step kt - 2, which the wait of step kt - 1 has seen arrive
+    // (loads complete in issue order). gk_ring[s]: the entries requested in the latest step that ran in LDS stage s.
+    const __amdgpu_buffer_rsrc_t gk_index = make_rsrc(reinterpret_cast<const uint16_t*>(args.row_index),
+                                                      kGatherK ? uniform(s_prefix[E]) * 4u : 0u);
+    const uint32_t gk_bytes = kGatherK ? args.a_rows * Ne * 2u : 0u;  // bytes of B (below 2^31)
+    const uint32_t gk_half = lane >> 5;
+    // the 16-byte chunk of a row this lane loads, swizzled as the packed loader does it for the row's place in the step;
+    // instruction i: ^ 128 (i & 1)
+    const uint32_t gk_chunk = ((lane & 31u) ^ (4u * gk_half) ^ (2u * (wave & 1u))) << 4;
+    uint32_t gk_ring[2] = {0u, 0u}, gk_v[4] = {0u, 0u, 0u, 0u};
+    // this lane's entry of the eight that begin at position `first` of row_index
+    auto gk_request = [&](uint32_t first) -> uint32_t {
+        return __builtin_amdgcn_raw_buffer_load_b32(gk_index, (lane & 7u) * 4u, first * 4u, 0);
+    };
+    // per-lane offsets of the four loads of the K step at k0 of a group with `limit` reduction rows, from the entries n
+    // (lane l holds entry l % 8): every lane forms the byte offset of its entry's row, then picks, per instruction, the
+    // offset of one of the instruction's two rows from the lane that holds it, and adds its chunk.
+    // n / divisor for n < 2^31: the high word of n * floor((2^32 - 1) / divisor) is the quotient or one less
+    const uint32_t gk_magic = kGatherK ? 0xffffffffu / args.divisor : 0u;
+    auto gk_offsets = [&](uint32_t k0, uint32_t limit, uint32_t n, uint32_t (&v)[4]) {
+        uint32_t q = __umulhi(n, gk_magic);
+        q += (n - q * args.divisor >= args.divisor) ? 1u : 0u;
+        // an entry that names no row of B (negative, or past the last row) reads as a row of zeros, and so does a
+        // reduction row past the group's end
+        q |= n & 0x80000000u;
+        q = k0 + wave * 8u + (lane & 7u) < limit ? q : 0xffffffffu;
+        const uint32_t off = q < args.a_rows ? q * (Ne * 2u) : kOutOfRange;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t even = (uint32_t)__builtin_amdgcn_readlane((int)off, 2 * i);
+            const uint32_t odd = (uint32_t)__builtin_amdgcn_readlane((int)off, 2 * i + 1);
+            v[i] = (gk_half ? odd : even) + (gk_chunk ^ (128u * ((uint32_t)i & 1u)));
+        }
+    };
 
     // ---- L2 prefetch by designated workgroups (grouped_gemm.hip): one 4-byte load per shared line, kPfDist steps ahead ----
     constexpr bool kPrefetch = A_KC == B_KC;
@@ -485,7 +535,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 }
             } else {
                 pf_base = fb_cur.base0; pf_ldb = fb_cur.ldb; pf_col_bytes = fb_cur.col_bytes; pf_kdim = t.Ke;
-                pf_voff = lane < 8u ? (2u * (p * 8u + lane) + (t.pf_r >> 2)) * fb_cur.ldb + (t.pf_r & 3u) * 128u : kOutOfRange;
+                // (gathered reduction rows: no prefetch of B, the instruction fetches nothing)
+                pf_voff = (!kGatherK && lane < 8u) ? (2u * (p * 8u + lane) + (t.pf_r >> 2)) * fb_cur.ldb + (t.pf_r & 3u) * 128u : kOutOfRange;
             }
         }
     };
@@ -535,7 +586,15 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     };
     auto issue_b = [&](int stage, uint32_t k0, auto i0_c, auto i1_c) __attribute__((always_inline)) {
         constexpr int I0 = decltype(i0_c)::value, I1 = decltype(i1_c)::value;
-        if constexpr (B_KC) lk_b.template issue_range<I0, I1>(stage ? s_b1 : s_b0, k0);
+        if constexpr (kGatherK) {
+            // the offsets of all four loads are formed with the first of them, from the entries requested two steps ago
+            if constexpr (I0 == 0) gk_offsets(k0, lt_b.kdim, gk_ring[stage], gk_v);
+            const __amdgpu_buffer_rsrc_t r = make_rsrc(lt_b.base, gk_bytes - lt_b.col_bytes);
+            uint8_t* tile = stage ? s_b1 : s_b0;
+#pragma unroll
+            for (int i = I0; i < I1; ++i)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(tile + (wave * 4 + i) * 1024), 16, gk_v[i], 0u, 0, 0);
+        } else if constexpr (B_KC) lk_b.template issue_range<I0, I1>(stage ? s_b1 : s_b0, k0);
         else lt_b.template issue_range<I0, I1>(stage ? s_b1 : s_b0, k0);
     };
     // ... and written in assembly, for a cold start
@@ -549,7 +608,14 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
             for (int i = 0; i < 4; ++i) buffer_load_lds_quiet(r, v[i], k0 * 2u, lds0 + (uint32_t)(i * NW) * 1024u);
         } else if constexpr (A_KC) lk_a.issue_quiet(stage ? s_a1 : s_a0, k0);
         else lt_a.issue_quiet(stage ? s_a1 : s_a0, k0);
-        if constexpr (B_KC) lk_b.issue_quiet(stage ? s_b1 : s_b0, k0);
+        if constexpr (kGatherK) {
+            uint32_t v[4];
+            gk_offsets(k0, lt_b.kdim, gk_request(vb_cur + k0 + wave * 8u), v);
+            const u32x4 r = make_rsrc_words(lt_b.base, gk_bytes - lt_b.col_bytes);
+            const uint32_t lds0 = lds_address(stage ? s_b1 : s_b0) + wave * 4096u;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) buffer_load_lds_quiet(r, v[i], 0u, lds0 + (uint32_t)i * 1024u);
+        } else if constexpr (B_KC) lk_b.issue_quiet(stage ? s_b1 : s_b0, k0);
         else lt_b.issue_quiet(stage ? s_b1 : s_b0, k0);
     };
 
@@ -564,7 +630,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
 
         if (!streamed) {
             if (!cur.fast) {
-                if constexpr (EPI == EPI_PLAIN) {
+                if constexpr (EPI == EPI_PLAIN && !kGatherK) {  // (the gathered entry point admits only sizes without such tiles)
                     scalar_tile<EL, A_KC, B_KC, BM, BN>(args.A + cur.off_a, args.B + cur.off_b, args.D + off_d, Me, Ne, Ke, m0, n0,
                                                         args.alpha, NT);
                 }
@@ -587,6 +653,12 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         const uint32_t KT = (Ke + BK - 1) / BK;
         const uint32_t KT2 = (KT + 1u) & ~1u;  // steps of the K loop: an odd count gets a step of zeros
         const bool thin = is_thin(cur);
+        // kGatherK: requests the row_index entries of this wavefront for K step `abs_step` of the load stream: a step of
+        // this tile, or, past its end, of the next (vb_cur, vb_nxt: where the two groups' entries begin)
+        auto gk_request_step = [&](uint32_t abs_step) __attribute__((always_inline)) -> uint32_t {
+            const bool of_next = abs_step >= KT2;
+            return gk_request((of_next ? vb_nxt + (abs_step - KT2) * (uint32_t)BK : vb_cur + abs_step * (uint32_t)BK) + wave * 8u);
+        };
         // the next tile's first two K steps ride on this tile's last two load slots
         const bool stream_next = streams(cur) && streams(nxt);
         if (stream_next) {
@@ -764,6 +836,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 issue_b(stage, k0, I2_{}, IN_{});
                 if constexpr (kPrefetch) asm volatile("" : "+v"(pf_voff));
                 issue_prefetch(kt + kPfDist);
+                // the entries for the loads of step kt + 2 (K step kt + 4 of the stream): the step's last load
+                if constexpr (kGatherK) gk_ring[stage] = gk_request_step(kt + 4u);
                 mma(fa_c, 3, 3, true, stage ^ 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x100, kReadsA, 0);
 #pragma unroll
@@ -771,7 +845,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
 #pragma unroll
                     for (int i = 0; i < AB; ++i) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        if (j * AB + i < 2 + (kPrefetch ? 1 : 0)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                        if (j * AB + i < 2 + (kPrefetch ? 1 : 0) + (kGatherK ? 1 : 0)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
                     }
                     __builtin_amdgcn_sched_group_barrier(0x100, kReadsB, 0);
                 }
@@ -809,6 +883,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 // counts on it being the newest load)
                 if constexpr (kPrefetch) asm volatile("" : "+v"(pf_voff));
                 issue_prefetch(kt + kPfDist);
+                if constexpr (kGatherK) gk_ring[stage] = gk_request_step(kt + 4u);
                 mma(fa_c, PP - 1, 1, true, stage ^ 1, 0);
                 if constexpr (FA > 0) {
                     // the A reads; per column block its matrix instructions, each followed by its share of the step's loads,
@@ -826,14 +901,16 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                         __builtin_amdgcn_sched_group_barrier(0x100, kReadsB, 0);
                     }
                     if constexpr (kPrefetch) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    if constexpr (kGatherK) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
                 }
             }
         };
         // waits of a step: all but the newest load when that is the previous step's prefetch; in a tile's first step the
         // stores of the previous epilogue (or the cold start's stand-ins) and the one load of the bias values are newer
         // than the loads waited for as well
-        using WaitStep = std::integral_constant<int, waitcnt_imm(kPrefetch ? 1 : 0, true)>;
-        using WaitFirst = std::integral_constant<int, waitcnt_imm((int)kTileStores + (kPrefetch ? 1 : 0) + (BIAS ? 1 : 0), true)>;
+        // (kGatherK: and the request for row_index entries that follows every step's loads)
+        using WaitStep = std::integral_constant<int, waitcnt_imm((kPrefetch ? 1 : 0) + (kGatherK ? 1 : 0), true)>;
+        using WaitFirst = std::integral_constant<int, waitcnt_imm((int)kTileStores + (kPrefetch ? 1 : 0) + (BIAS ? 1 : 0) + (kGatherK ? 1 : 0), true)>;
 
         // BIAS: the bias values of this wavefront's columns of the tile into its 128 bytes of LDS: one load by 32 lanes
         // (every wavefront issues it, so that all count the same loads), complete (loads and stores complete in issue
@@ -927,6 +1004,12 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         } else if (KT > 0) {
             if (!streamed) {
                 // cold start: the first two K steps, then as many stores outside every buffer as an epilogue issues
+                // (kGatherK: the entries for the loads of steps 0 and 1 first, so that everything the waits below leave
+                // outstanding is what they count; a streamed tile has them from the last two steps of the tile before it)
+                if constexpr (kGatherK) {
+                    gk_ring[0] = gk_request_step(2u);
+                    gk_ring[1] = gk_request_step(3u);
+                }
                 issue_quiet(0, 0);
                 issue_quiet(1, BK);
                 const __amdgpu_buffer_rsrc_t nowhere = make_rsrc(args.D, 0u);
@@ -1232,7 +1315,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false, false, true>(const Args); \
     template __global__ void ragged_gemm_kernel<EL, true, true, EPI_PLAIN, false, true, true>(const Args);      \
     template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU, false, true, true>(const Args);     \
-    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false, true, true>(const Args);
+    template __global__ void ragged_gemm_kernel<EL, true, true, EPI_SWIGLU_ACT, false, true, true>(const Args); \
+    template __global__ void ragged_gemm_kernel<EL, false, false, EPI_PLAIN, true, false, true>(const Args);
 FMA_RAGGED_INSTANTIATE(ElemBf16)
 FMA_RAGGED_INSTANTIATE(ElemF16)
 #undef FMA_RAGGED_INSTANTIATE
@@ -1434,6 +1518,47 @@ int fma_grouped_gemm_swiglu_bwd(const void* dy, const void* W, const void* h, vo
     hipStream_t st = (hipStream_t)stream;
     return dtype == FMA_BF16 ? ragged::launch<ElemBf16, true, false, EPI_SWIGLU_BWD, false>(args, st)
                              : ragged::launch<ElemF16, true, false, EPI_SWIGLU_BWD, false>(args, st);
+}
+
+int fma_grouped_gemm_gathered_wgrad(const void* dy, const void* x, int64_t x_rows, const int32_t* row_index, int32_t divisor,
+                                    void* dW, const uint32_t* K_arr, int64_t E, int64_t M, int64_t N, float alpha, int dtype,
+                                    void* stream) {
+    using namespace fmahip;
+    using namespace fmahip::gemm;
+    const char* who = "grouped_gemm_gathered_wgrad";
+    FMA_REQUIRE(dtype == FMA_BF16 || dtype == FMA_F16, dtype_bytes(dtype) ? FMA_ERR_UNSUPPORTED : FMA_ERR_BAD_DTYPE,
+                "%s: bf16 and fp16 operands are implemented (dtype code %d)", who, dtype);
+    FMA_REQUIRE(E >= 0, FMA_ERR_BAD_SIZE, "%s: negative group count %lld", who, (long long)E);
+    FMA_REQUIRE(E <= FMA_MAX_GROUPS, FMA_ERR_TOO_MANY_EXPERTS, "%s: E=%lld exceeds the limit %d", who, (long long)E,
+                FMA_MAX_GROUPS);
+    // (with these sizes every tile takes the matrix-instruction path, the only one that gathers)
+    FMA_REQUIRE(M >= 8 && M % 8 == 0 && M < (1ll << 23) && N >= 8 && N % 8 == 0 && N < (1ll << 23), FMA_ERR_BAD_SIZE,
+                "%s: M=%lld and N=%lld must be positive multiples of 8 below 2^23", who, (long long)M, (long long)N);
+    FMA_REQUIRE(divisor >= 1 && divisor <= 65536, FMA_ERR_BAD_SIZE, "%s: divisor must lie in [1, 65536] (got %d)", who, divisor);
+    if (E == 0) return FMA_OK;
+    FMA_REQUIRE(dy && x && row_index && dW && K_arr, FMA_ERR_NULL_POINTER, "%s: NULL pointer", who);
+    FMA_REQUIRE(x_rows >= 1, FMA_ERR_BAD_SIZE, "%s: x has no rows (%lld)", who, (long long)x_rows);
+    // the loads address x with 32-bit byte offsets below 2^31
+    FMA_REQUIRE(x_rows <= ((1ll << 31) - 1) / (2 * N), FMA_ERR_UNSUPPORTED,
+                "%s: x must be smaller than 2 GiB (%lld rows of %lld elements)", who, (long long)x_rows, (long long)N);
+    FMA_REQUIRE(aligned16(dy) && aligned16(x) && aligned16(dW), FMA_ERR_MISALIGNED, "%s: dy, x and dW must be 16-byte aligned", who);
+    FMA_REQUIRE((reinterpret_cast<uintptr_t>(row_index) & 3u) == 0, FMA_ERR_MISALIGNED, "%s: row_index must be 4-byte aligned", who);
+    ragged::Args args{};
+    args.A = (const uint16_t*)dy;
+    args.B = (const uint16_t*)x;
+    args.D = (uint16_t*)dW;
+    args.sizes = K_arr;
+    args.row_index = row_index;
+    args.divisor = (uint32_t)divisor;
+    args.a_rows = (uint32_t)x_rows;
+    args.E = (uint32_t)E;
+    args.m = (uint32_t)M;
+    args.n = (uint32_t)N;
+    args.k = 0;
+    args.alpha = alpha;
+    hipStream_t st = (hipStream_t)stream;
+    return dtype == FMA_BF16 ? ragged::launch<ElemBf16, false, false, EPI_PLAIN, true, false, true>(args, st)
+                             : ragged::launch<ElemF16, false, false, EPI_PLAIN, true, false, true>(args, st);
 }
 
 int fma_grouped_gemm_gathered(const void* x, int64_t x_rows, const int32_t* row_index, int32_t divisor, const void* W,

@@ -48,6 +48,7 @@ SIGNATURES = {
     "fma_grouped_gemm_ragged": (_i32, [_p, _p, _p, _p, _p, _i64, _i32, _i64, _i64, _i64, _i32, _i32, _f32, _i32, _p]),
     "fma_grouped_gemm_swiglu_bwd": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "fma_grouped_gemm_gathered": (_i32, [_p, _i64, _p, _i32, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i32, _i32, _p]),
+    "fma_grouped_gemm_gathered_wgrad": (_i32, [_p, _p, _i64, _p, _i32, _p, _p, _i64, _i64, _i64, _f32, _i32, _p]),
     "fma_grouped_gemm_swiglu": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "fma_expert_bias_add": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "fma_expert_bias_grad_workspace_bytes": (_i64, [_i64, _i64, _i64]),

@@ -291,6 +291,39 @@ def grouped_gemm_gathered_cuda(
     _lib.check(rc, "grouped_gemm_gathered_cuda")
 
 
+@custom_op(f"{LIBRARY_NAME}::grouped_gemm_gathered_wgrad_cuda", mutates_args={"weight_grad"})
+def grouped_gemm_gathered_wgrad_cuda(
+    output_grad: torch.Tensor,
+    x: torch.Tensor,
+    row_index: torch.Tensor,
+    divisor: int,
+    K_array: torch.Tensor,
+    weight_grad: torch.Tensor,
+) -> None:
+    """The weight gradient of an expert projection on the rows x[row_index[i] // divisor] (i over the packed rows of all
+    experts, K_array[e] of them for expert e), gathered inside the operand load: weight_grad[e] [N, K] = output_grad_e^T @
+    those rows (fma_grouped_gemm_gathered_wgrad)."""
+    _lib.require_gpu(output_grad, x, row_index, K_array, weight_grad)
+    E, N, K = weight_grad.shape
+    R = row_index.numel()
+    assert x.dim() == 2 and x.size(1) == K and output_grad.shape == (R, N)
+    assert x.dtype == output_grad.dtype == weight_grad.dtype and x.dtype in (torch.bfloat16, torch.float16)
+    assert row_index.dtype == torch.int32 and K_array.dtype == torch.uint32 and K_array.numel() == E
+    for t in (output_grad, x, row_index, K_array, weight_grad):
+        assert t.is_contiguous()
+    if weight_grad.numel() == 0:
+        return
+    if R == 0:
+        weight_grad.zero_()
+        return
+    with torch.cuda.device(x.device):
+        rc = _lib.load().fma_grouped_gemm_gathered_wgrad(
+            output_grad.data_ptr(), x.data_ptr(), x.size(0), row_index.data_ptr(), divisor, weight_grad.data_ptr(),
+            K_array.data_ptr(), E, N, K, 1.0, _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
+        )
+    _lib.check(rc, "grouped_gemm_gathered_wgrad_cuda")
+
+
 @custom_op(f"{LIBRARY_NAME}::expert_bias_add_cuda", mutates_args={"y"})
 def expert_bias_add_cuda(y: torch.Tensor, bias: torch.Tensor, M_array: torch.Tensor) -> None:
     _lib.require_gpu(y, bias, M_array)
@@ -723,9 +756,9 @@ def swiglu_experts(
 
 class _GatheredUpProjection(torch.autograd.Function):
     """The first expert projection on tokens instead of grouped rows: y_i = x[perm[i] // top_k] @ W_e^T (+ bias_e), with
-    swiglu_packed applied in the epilogue if `swiglu`. The rows are gathered inside the GEMM's operand load, so the
-    [T * top_k, H] buffer of grouped rows is neither written in the forward nor kept for the backward, which rebuilds it
-    (one row-movement pass) for the weight gradient and returns the gradient per token."""
+    swiglu_packed applied in the epilogue if `swiglu`. The rows are gathered inside the operand loads of the forward GEMM
+    and of the weight-gradient GEMM, so the [T * top_k, H] buffer of grouped rows never exists; the backward returns the
+    gradient per token."""
 
     @staticmethod
     @ensure_contiguous
@@ -746,7 +779,7 @@ class _GatheredUpProjection(torch.autograd.Function):
             output = torch.empty(R, N, device=x.device, dtype=x.dtype)
             grouped_gemm_gathered_cuda(x, perm, top_k, weight, bias, M_array, output, None)
         if needs_backward:
-            ctx.save_for_backward(x, weight, h, inv, M_array, K_array, N_array)
+            ctx.save_for_backward(x, weight, h, perm, inv, M_array, K_array, N_array)
         ctx.top_k = top_k
         ctx.has_bias = bias is not None
         return output
@@ -756,7 +789,7 @@ class _GatheredUpProjection(torch.autograd.Function):
     def backward(ctx, output_grad: torch.Tensor) -> tuple[torch.Tensor | None]:
         from ...ops.swiglu.cuda_implementation import swiglu_backward_cuda
 
-        x, weight, h, inv, M_array, K_array, N_array = ctx.saved_tensors
+        x, weight, h, perm, inv, M_array, K_array, N_array = ctx.saved_tensors
         _, N, K = weight.size()
         if h is not None:
             h_grad = torch.empty_like(h)
@@ -776,16 +809,88 @@ class _GatheredUpProjection(torch.autograd.Function):
             x_grad = torch.empty_like(x)
             combine_cuda(grouped_grad, inv, None, ctx.top_k, x_grad)
         if ctx.needs_input_grad[1]:
-            grouped = torch.empty(h_grad.size(0), K, device=x.device, dtype=x.dtype)
-            dispatch_rows_cuda(x, inv, ctx.top_k, grouped)
-            weight_grad = _expert_gemm(
-                h_grad, grouped, N_array, K_array, M_array, weight.size(), "K", N, K, 0,
-                is_A_transposed=True, is_B_transposed=False,
-            )
+            weight_grad = torch.empty_like(weight)
+            grouped_gemm_gathered_wgrad_cuda(h_grad, x, perm, ctx.top_k, M_array, weight_grad)
         if ctx.has_bias and ctx.needs_input_grad[2]:
             bias_grad = torch.empty(weight.size(0), N, device=h_grad.device, dtype=h_grad.dtype)
             expert_bias_grad_cuda(h_grad, M_array, bias_grad)
         return x_grad, weight_grad, bias_grad, None, None, None, None, None, None, None, None
+
+
+class _GatheredSwigluExperts(torch.autograd.Function):
+    """_SwigluExperts on tokens instead of grouped rows: o_e = swiglu_packed(x[perm[i] // top_k] @ W1_e^T + b1_e) @ W2_e^T +
+    b2_e. The first projection and its weight gradient gather the rows inside their operand loads, so a training step
+    neither writes nor keeps the [T * top_k, H] buffer of grouped rows; the input gradient is summed per token here.
+    Same values, bit for bit, as gather_rows followed by _SwigluExperts."""
+
+    @staticmethod
+    @ensure_contiguous
+    def forward(
+        ctx, x: torch.Tensor, weight1: torch.Tensor, bias1: torch.Tensor | None, weight2: torch.Tensor,
+        bias2: torch.Tensor | None, perm: torch.Tensor, inv: torch.Tensor, M_array: torch.Tensor, N1_array: torch.Tensor,
+        K1_array: torch.Tensor, N2_array: torch.Tensor, K2_array: torch.Tensor, top_k: int, grad_enabled: bool,
+    ) -> torch.Tensor:  # fmt: skip
+        _, N1, K1 = weight1.size()
+        _, N2, K2 = weight2.size()
+        assert N1 % 16 == 0 and K1 % 8 == 0 and N2 % 8 == 0 and K2 == N1 // 2
+        R = perm.numel()
+        needs_backward = grad_enabled and any(ctx.needs_input_grad[:5])
+        h = torch.empty(R, N1, device=x.device, dtype=x.dtype) if needs_backward else None
+        act = torch.empty(R, K2, device=x.device, dtype=x.dtype)
+        grouped_gemm_gathered_cuda(x, perm, top_k, weight1, bias1, M_array, h, act)
+        output = _expert_gemm(
+            act, weight2, M_array, N2_array, K2_array, (R, N2), "M", 0, N2, K2, is_A_transposed=False, is_B_transposed=True,
+            bias=bias2,
+        )
+        if needs_backward:
+            ctx.save_for_backward(x, weight1, weight2, h, act, perm, inv, M_array, N1_array, K1_array, N2_array, K2_array)
+        ctx.has_bias = (bias1 is not None, bias2 is not None)
+        ctx.top_k = top_k
+        return output
+
+    @staticmethod
+    @ensure_contiguous
+    def backward(ctx, output_grad: torch.Tensor) -> tuple[torch.Tensor | None]:
+        x, weight1, weight2, h, act, perm, inv, M_array, N1_array, K1_array, N2_array, K2_array = ctx.saved_tensors
+        _, N1, K1 = weight1.size()
+        _, N2, K2 = weight2.size()
+        x_grad = weight1_grad = bias1_grad = weight2_grad = bias2_grad = None
+        if ctx.needs_input_grad[3]:
+            weight2_grad = _expert_gemm(
+                output_grad, act, N2_array, K2_array, M_array, weight2.size(), "K", N2, K2, 0,
+                is_A_transposed=True, is_B_transposed=False,
+            )
+        if ctx.has_bias[1] and ctx.needs_input_grad[4]:
+            bias2_grad = torch.empty(weight2.size(0), N2, device=output_grad.device, dtype=output_grad.dtype)
+            expert_bias_grad_cuda(output_grad, M_array, bias2_grad)
+        if any(ctx.needs_input_grad[:3]):
+            h_grad = torch.empty_like(h)
+            grouped_gemm_swiglu_bwd_cuda(output_grad, weight2, h, M_array, h_grad)
+            if ctx.needs_input_grad[0]:
+                grouped_grad = _expert_gemm(
+                    h_grad, weight1, M_array, K1_array, N1_array, (h_grad.size(0), K1), "M", 0, K1, N1,
+                    is_A_transposed=False, is_B_transposed=False,
+                )
+                x_grad = torch.empty_like(x)
+                combine_cuda(grouped_grad, inv, None, ctx.top_k, x_grad)
+            if ctx.needs_input_grad[1]:
+                weight1_grad = torch.empty_like(weight1)
+                grouped_gemm_gathered_wgrad_cuda(h_grad, x, perm, ctx.top_k, M_array, weight1_grad)
+            if ctx.has_bias[0] and ctx.needs_input_grad[2]:
+                bias1_grad = torch.empty(weight1.size(0), N1, device=h_grad.device, dtype=h_grad.dtype)
+                expert_bias_grad_cuda(h_grad, M_array, bias1_grad)
+        return (x_grad, weight1_grad, bias1_grad, weight2_grad, bias2_grad) + (None,) * 9
+
+
+def gathered_swiglu_experts(
+    x: torch.Tensor, weight1: torch.Tensor, bias1: torch.Tensor | None, weight2: torch.Tensor, bias2: torch.Tensor | None,
+    perm: torch.Tensor, inv: torch.Tensor, M_array: torch.Tensor, N1_array: torch.Tensor, K1_array: torch.Tensor,
+    N2_array: torch.Tensor, K2_array: torch.Tensor, top_k: int,
+) -> torch.Tensor:  # fmt: skip
+    return _GatheredSwigluExperts.apply(
+        x, weight1, bias1, weight2, bias2, perm, inv, M_array, N1_array, K1_array, N2_array, K2_array, top_k,
+        torch.is_grad_enabled(),
+    )
 
 
 def gathered_up_projection_experts(

@@ -253,6 +253,23 @@ int fma_grouped_gemm_gathered(const void* x, int64_t x_rows, const int32_t* row_
                               const void* bias, void* out, void* act, const uint32_t* M_arr, int64_t E, int64_t N,
                               int64_t K, int swiglu, int dtype, void* stream);
 
+/* The weight gradient of an expert projection with the gather of the routed rows inside the operand load: for each
+ * expert e with K_e rows (packed rows i of all experts back to back, R = sum K_e)
+ *   dW_e[M, N] = alpha * dy_e[K_e, M]^T * xg_e[K_e, N],   xg[i, :] = x[row_index[i] / divisor, :]
+ * i.e. fma_grouped_gemm_ragged (reduction varies, trans_a = 1, trans_b = 0) applied to dy and the output of
+ * fma_gather_rows(x, row_index, R, N, divisor), bit for bit, without that [R, N] buffer ever being written or read.
+ * dy: [R, M] packed; x: [x_rows, N] with x_rows * N * 2 < 2^31 bytes; dW: [E, M, N]; an expert without rows gets zeros.
+ * An entry row_index[i] that is negative or whose row_index[i] / divisor is not below x_rows names no row and contributes
+ * nothing; divisor in [1, 65536] (top_k with row_index = the stable routing order perm of fma_moe_build_index).
+ * M % 8 == 0, N % 8 == 0, both below 2^23 (K_e is arbitrary); dtype FMA_BF16 or FMA_F16.
+ * The weight-gradient product of _GroupedGemmExperts.backward (fma/modules/moe/cuda_implementation/__init__.py:46-80) on
+ * the rows the reference first materialises: with group_with_padding on the grouped-GEMM path (the same file, :107-183)
+ * and with group() in front of group_bwd_W on the Triton path (triton_implementation/__init__.py:105-123,
+ * group_backward_kernel.py:23-101). */
+int fma_grouped_gemm_gathered_wgrad(const void* dy, const void* x, int64_t x_rows, const int32_t* row_index, int32_t divisor,
+                                    void* dW, const uint32_t* K_arr, int64_t E, int64_t M, int64_t N, float alpha, int dtype,
+                                    void* stream);
+
 /* ---- per-expert bias ------------------------------------------------------------------------ */
 
 /* y[i, :] += bias[e, :] for every row i of expert e, rows packed expert by expert with M_arr[e] rows each (device

@@ -1,6 +1,7 @@
-"""GPU parity of fma_grouped_gemm_gathered (the forward expert product with the gather of the routed rows inside the
-operand load) against fma_gather_rows followed by the entry points that take packed rows: the same bits, for the plain
-and the fused-SwiGLU epilogue, with and without a bias."""
+"""GPU parity of fma_grouped_gemm_gathered and fma_grouped_gemm_gathered_wgrad (the forward expert product and the weight
+gradient with the gather of the routed rows inside the operand load) against fma_gather_rows followed by the entry points
+that take packed rows: the same bits, for the plain and the fused-SwiGLU epilogue, with and without a bias; the weight
+gradient also against a float64 product of the same rows."""
 
 import pytest
 import torch
@@ -9,6 +10,7 @@ from fma import _lib, swiglu_packed
 from fma.modules.moe.cuda_implementation import (
     gather_rows_cuda,
     grouped_gemm_gathered_cuda,
+    grouped_gemm_gathered_wgrad_cuda,
     grouped_gemm_ragged_cuda,
     grouped_gemm_swiglu_cuda,
 )
@@ -131,6 +133,80 @@ def test_argument_validation():
     assert call(p, 8, p, 1, p, None, p, None, m, 0, 16, 16, 0, _lib.FMA_BF16, None) == 0  # no groups
 
 
+WGRAD_CASES = [
+    # rows per expert, T, N (rows of the gradient's output, = out features), K (= in features, width of x), divisor
+    ([2048 + 8 * (e % 7) for e in range(8)], 4096, 512, 1024, 2),  # long reductions: every tile streams into the next
+    ([1500, 0, 263, 7, 3001, 40, 777], 700, 768, 192, 3),  # reductions of any length, empty groups, K one partial tile
+    ([520] * 40, 2000, 256, 512, 1),  # 9 K steps per tile (the last one partial), many tiles per workgroup
+    ([64, 63, 65, 128, 129, 191, 192, 193, 1, 2], 50, 256, 512, 4),  # 1 to 4 K steps: tiles that start cold
+    ([300, 5000, 16, 16, 16, 2000], 997, 264, 1088, 6),  # N and K with partial tiles
+    ([0, 0, 5], 9, 256, 256, 1),
+    ([0, 0, 0], 9, 256, 256, 1),
+]
+
+
+def _wgrad_inputs(counts, T, N, K, divisor, dtype, seed, spoil=False):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    R, E = sum(counts), len(counts)
+    x = torch.randn(T, K, device=DEV, generator=g).to(dtype)
+    dy = torch.randn(R, N, device=DEV, generator=g).to(dtype)
+    row_index = torch.randint(0, T * divisor, (R,), device=DEV, generator=g, dtype=torch.int32)
+    if spoil and R > 10:
+        row_index[3] = -5
+        row_index[R // 2] = T * divisor + 7
+        row_index[R - 1] = -(2**31)
+    xg = torch.zeros(R, K, device=DEV, dtype=dtype)
+    if R:
+        src = torch.div(row_index.long(), divisor, rounding_mode="floor")
+        ok = (row_index >= 0) & (src < T)
+        xg[ok] = x[src[ok]]
+    return x, dy, row_index, xg, _u32(counts)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("spoil", [False, True])
+@pytest.mark.parametrize("counts,T,N,K,divisor", WGRAD_CASES)
+def test_weight_gradient_gathers_its_reduction_rows(counts, T, N, K, divisor, spoil, dtype):
+    x, dy, row_index, xg, sizes = _wgrad_inputs(counts, T, N, K, divisor, dtype, seed=N + K + divisor, spoil=spoil)
+    E = len(counts)
+    # the packed kernel on an explicit copy of the rows (entries that name no row: rows of zeros): the same bits
+    expect = torch.full((E, N, K), 7.0, dtype=dtype, device=DEV)
+    grouped_gemm_ragged_cuda(dy, xg, expect, sizes, True, N, K, 0, True, False)
+    got = torch.full((E, N, K), 7.0, dtype=dtype, device=DEV)
+    grouped_gemm_gathered_wgrad_cuda(dy, x, row_index, divisor, sizes, got)
+    assert torch.equal(got, expect)
+    # and the product itself, in float64 (one rounding of an fp32-accumulated sum: 2^-8 relative for bf16, 2^-11 for fp16,
+    # of the largest element of the group's gradient, plus the accumulation's own error)
+    start = 0
+    for e, m in enumerate(counts):
+        ref = dy[start : start + m].double().T @ xg[start : start + m].double()
+        tol = (2.0**-8 if dtype == torch.bfloat16 else 2.0**-11) * float(ref.abs().max()) + 1e-6 * m
+        assert float((got[e].double() - ref).abs().max()) <= tol, f"expert {e}"
+        start += m
+
+
+def test_weight_gradient_argument_validation():
+    lib = _lib.load()
+    call = lib.fma_grouped_gemm_gathered_wgrad
+    buf = torch.zeros(1 << 16, dtype=torch.bfloat16, device=DEV)
+    idx = torch.zeros(64, dtype=torch.int32, device=DEV)
+    k = _u32([8])
+    p, i, s = buf.data_ptr(), idx.data_ptr(), k.data_ptr()
+    bf = _lib.FMA_BF16
+    assert call(p, p, 8, i, 1, p, s, 1, 16, 16, 1.0, bf, None) == 0
+    torch.cuda.synchronize()
+    assert call(p, p, 8, i, 1, p, s, 1, 12, 16, 1.0, bf, None) != 0  # M not a multiple of 8
+    assert call(p, p, 8, i, 1, p, s, 1, 16, 20, 1.0, bf, None) != 0  # N not a multiple of 8
+    assert call(p, p, 8, i, 0, p, s, 1, 16, 16, 1.0, bf, None) != 0  # divisor
+    assert call(p, p, 0, i, 1, p, s, 1, 16, 16, 1.0, bf, None) != 0  # x without rows
+    assert call(p, p, 1 << 28, i, 1, p, s, 1, 16, 16, 1.0, bf, None) != 0  # x of 2 GiB or more
+    assert call(p, p, 8, None, 1, p, s, 1, 16, 16, 1.0, bf, None) != 0  # no row_index
+    assert call(p, p, 8, i, 1, p, s, 1, 16, 16, 1.0, _lib.FMA_F32, None) != 0  # 16-bit types only
+    assert call(p + 2, p, 8, i, 1, p, s, 1, 16, 16, 1.0, bf, None) != 0  # misaligned
+    assert call(p, p, 8, i, 1, p, s, 0, 16, 16, 1.0, bf, None) == 0  # no groups
+    assert "grouped_gemm_gathered_wgrad" in lib.fma_last_error_string().decode()
+
+
 @pytest.mark.parametrize("act_name,add_bias", [("swiglu", False), ("swiglu", True), ("gelu", True), ("glu", False)])
 def test_layer_with_the_gather_inside_the_first_projection(act_name, add_bias):
     # the layer with and without the grouped copy of the tokens: the same bits in the output and in every gradient
@@ -161,19 +237,25 @@ def test_layer_with_the_gather_inside_the_first_projection(act_name, add_bias):
         assert torch.equal(a, b)
 
 
-def test_evaluation_skips_the_grouped_copy(monkeypatch):
-    # without a backward to follow, a narrow first projection gathers by itself: no row-movement pass before it
+def test_a_narrow_first_projection_never_needs_the_grouped_copy(monkeypatch):
+    # a narrow first projection gathers by itself, in its forward and in its weight gradient: no row-movement pass in
+    # front of it, with or without a backward; a wide one reads a grouped copy of the tokens
     from fma import KernelBackend, MoE
     from fma.modules.moe import cuda_implementation as ci
 
     torch.manual_seed(4)
-    moe = MoE(8, 2, 256, 512, swiglu_packed, True, False, 0.02).to(torch.bfloat16).to(DEV)
-    x = torch.randn(100, 256, device=DEV).bfloat16()
     calls = []
     real = ci.dispatch_rows_cuda
     monkeypatch.setattr(ci, "dispatch_rows_cuda", lambda *a: (calls.append(1), real(*a))[1])
-    y_train, _ = moe(x.clone().requires_grad_(), kernel_backend=KernelBackend.cuda)
-    assert calls == [1]
+    x = torch.randn(100, 256, device=DEV).bfloat16()
+    moe = MoE(8, 2, 256, 512, swiglu_packed, True, False, 0.02).to(torch.bfloat16).to(DEV)
+    xi = x.clone().requires_grad_()
+    y_train, _ = moe(xi, kernel_backend=KernelBackend.cuda)
+    y_train.sum().backward()
     with torch.no_grad():
         y_eval, _ = moe(x, kernel_backend=KernelBackend.cuda)
-    assert calls == [1] and torch.equal(y_eval, y_train.detach())
+    assert calls == [] and torch.equal(y_eval, y_train.detach())
+    assert xi.grad is not None and moe.c_fc.weight.grad is not None
+    wide = MoE(2, 2, 256, 3200, swiglu_packed, True, False, 0.02).to(torch.bfloat16).to(DEV)
+    wide(x.clone().requires_grad_(), kernel_backend=KernelBackend.cuda)
+    assert calls == [1]
