@@ -80,6 +80,39 @@ def test_grouped_gemm_with_groups_past_2_32_bytes():
         row += m
 
 
+def test_gathered_products_on_a_token_matrix_of_almost_2_31_bytes():
+    # the gathered kernels address x with 32-bit byte offsets below 2^31: x as large as they admit, with most of the
+    # routed rows taken from its last rows, and the dy operand of the weight gradient past 2^32 bytes
+    T, H, N, k = 262143, 4096, 512, 2  # x: 2^31 - 8192 bytes
+    counts = [40000, 8, 60000, 31064]
+    R = sum(counts)
+    g = torch.Generator(device=DEV).manual_seed(2)
+    x = torch.randint(-8, 9, (T, H), device=DEV, generator=g).to(BF16)
+    perm = torch.randint(T * k - 4096, T * k, (R,), device=DEV, generator=g, dtype=torch.int32)
+    perm[::7] = torch.randint(0, T * k, (len(perm[::7]),), device=DEV, generator=g, dtype=torch.int32)
+    perm[-1] = T * k - 1
+    xg = x[perm.long() // k]
+    sizes = _u32(counts)
+    w = torch.randint(-8, 9, (len(counts), N, H), device=DEV, generator=g).to(BF16)
+    expect = torch.empty(R, N, device=DEV, dtype=BF16)
+    C.grouped_gemm_ragged_cuda(xg, w, expect, sizes, False, 0, N, H, False, True)
+    got = torch.empty(R, N, device=DEV, dtype=BF16)
+    C.grouped_gemm_gathered_cuda(x, perm, k, w, None, sizes, got, None)
+    assert torch.equal(got, expect)
+    del w, expect, got
+    M = 32768  # dy: 131072 rows of 32768 elements, 8.6e9 bytes
+    dy = torch.randint(-2, 3, (R, M), device=DEV, generator=g).to(BF16)
+    dw_expect = torch.empty(len(counts), M, H, device=DEV, dtype=BF16)
+    C.grouped_gemm_ragged_cuda(dy, xg, dw_expect, sizes, True, M, H, 0, True, False)
+    dw = torch.empty(len(counts), M, H, device=DEV, dtype=BF16)
+    C.grouped_gemm_gathered_wgrad_cuda(dy, x, perm, k, sizes, dw)
+    assert torch.equal(dw, dw_expect)
+    # integer operands, sums below 2^24: the small group's gradient is exact
+    e0 = counts[0]
+    ref = dy[e0 : e0 + 8].float().T @ xg[e0 : e0 + 8].float()
+    assert torch.equal(dw[1].float(), ref)
+
+
 def test_row_kernels_on_10_gb_of_grouped_rows():
     T, k, H, E = 300000, 4, 4096, 16  # 1.2M grouped rows of 8 KB
     R = T * k
