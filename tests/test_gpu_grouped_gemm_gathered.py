@@ -185,6 +185,22 @@ def test_weight_gradient_gathers_its_reduction_rows(counts, T, N, K, divisor, sp
         start += m
 
 
+def test_weight_gradient_scaled_by_alpha():
+    counts, T, N, K, divisor = [700, 0, 129], 300, 264, 512, 2
+    x, dy, row_index, xg, sizes = _wgrad_inputs(counts, T, N, K, divisor, torch.bfloat16, seed=9)
+    lib, E = _lib.load(), len(counts)
+    stream = torch.cuda.current_stream().cuda_stream
+    expect = torch.empty(E, N, K, dtype=torch.bfloat16, device=DEV)
+    got = torch.empty(E, N, K, dtype=torch.bfloat16, device=DEV)
+    rc = lib.fma_grouped_gemm_ragged(dy.data_ptr(), xg.data_ptr(), expect.data_ptr(), sizes.data_ptr(), None, E, _lib.FMA_VARY_K,
+                                     N, K, 0, 1, 0, -0.375, _lib.FMA_BF16, stream)
+    _lib.check(rc, "fma_grouped_gemm_ragged")
+    rc = lib.fma_grouped_gemm_gathered_wgrad(dy.data_ptr(), x.data_ptr(), T, row_index.data_ptr(), divisor, got.data_ptr(),
+                                             sizes.data_ptr(), E, N, K, -0.375, _lib.FMA_BF16, stream)
+    _lib.check(rc, "fma_grouped_gemm_gathered_wgrad")
+    assert torch.equal(got, expect) and bool((got[1] == 0).all()) and float(got[0].abs().max()) > 0
+
+
 def test_weight_gradient_argument_validation():
     lib = _lib.load()
     call = lib.fma_grouped_gemm_gathered_wgrad
