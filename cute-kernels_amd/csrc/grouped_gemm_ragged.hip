@@ -473,9 +473,13 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     // instruction i: ^ 128 (i & 1)
     const uint32_t gk_chunk = ((lane & 31u) ^ (4u * gk_half) ^ (2u * (wave & 1u))) << 4;
     uint32_t gk_ring[2] = {0u, 0u}, gk_v[4] = {0u, 0u, 0u, 0u};
-    // this lane's entry of the eight that begin at position `first` of row_index
-    auto gk_request = [&](uint32_t first) -> uint32_t {
-        return __builtin_amdgcn_raw_buffer_load_b32(gk_index, (lane & 7u) * 4u, first * 4u, 0);
+    // this lane's entry of the eight that begin at position `first` of row_index. pinned: the request may not be issued
+    // ahead of anything that precedes it in the program (the empty statement the lane's offset passes through is ordered
+    // behind every load before it): the step waits count on the request being the newest load of its step
+    auto gk_request = [&](uint32_t first, bool pinned) __attribute__((always_inline)) -> uint32_t {
+        uint32_t mine = (lane & 7u) * 4u;
+        if (pinned) asm volatile("" : "+v"(mine));
+        return __builtin_amdgcn_raw_buffer_load_b32(gk_index, mine, first * 4u, 0);
     };
     // per-lane offsets of the four loads of the K step at k0 of a group with `limit` reduction rows, from the entries n
     // (lane l holds entry l % 8): every lane forms the byte offset of its entry's row, then picks, per instruction, the
@@ -610,7 +614,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         else lt_a.issue_quiet(stage ? s_a1 : s_a0, k0);
         if constexpr (kGatherK) {
             uint32_t v[4];
-            gk_offsets(k0, lt_b.kdim, gk_request(vb_cur + k0 + wave * 8u), v);
+            gk_offsets(k0, lt_b.kdim, gk_request(vb_cur + k0 + wave * 8u, false), v);
             const u32x4 r = make_rsrc_words(lt_b.base, gk_bytes - lt_b.col_bytes);
             const uint32_t lds0 = lds_address(stage ? s_b1 : s_b0) + wave * 4096u;
 #pragma unroll
@@ -655,9 +659,10 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         const bool thin = is_thin(cur);
         // kGatherK: requests the row_index entries of this wavefront for K step `abs_step` of the load stream: a step of
         // this tile, or, past its end, of the next (vb_cur, vb_nxt: where the two groups' entries begin)
-        auto gk_request_step = [&](uint32_t abs_step) __attribute__((always_inline)) -> uint32_t {
+        auto gk_request_step = [&](uint32_t abs_step, bool pinned) __attribute__((always_inline)) -> uint32_t {
             const bool of_next = abs_step >= KT2;
-            return gk_request((of_next ? vb_nxt + (abs_step - KT2) * (uint32_t)BK : vb_cur + abs_step * (uint32_t)BK) + wave * 8u);
+            return gk_request((of_next ? vb_nxt + (abs_step - KT2) * (uint32_t)BK : vb_cur + abs_step * (uint32_t)BK) + wave * 8u,
+                              pinned);
         };
         // the next tile's first two K steps ride on this tile's last two load slots
         const bool stream_next = streams(cur) && streams(nxt);
@@ -837,7 +842,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 if constexpr (kPrefetch) asm volatile("" : "+v"(pf_voff));
                 issue_prefetch(kt + kPfDist);
                 // the entries for the loads of step kt + 2 (K step kt + 4 of the stream): the step's last load
-                if constexpr (kGatherK) gk_ring[stage] = gk_request_step(kt + 4u);
+                if constexpr (kGatherK) gk_ring[stage] = gk_request_step(kt + 4u, true);
                 mma(fa_c, 3, 3, true, stage ^ 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x100, kReadsA, 0);
 #pragma unroll
@@ -883,7 +888,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 // counts on it being the newest load)
                 if constexpr (kPrefetch) asm volatile("" : "+v"(pf_voff));
                 issue_prefetch(kt + kPfDist);
-                if constexpr (kGatherK) gk_ring[stage] = gk_request_step(kt + 4u);
+                if constexpr (kGatherK) gk_ring[stage] = gk_request_step(kt + 4u, true);
                 mma(fa_c, PP - 1, 1, true, stage ^ 1, 0);
                 if constexpr (FA > 0) {
                     // the A reads; per column block its matrix instructions, each followed by its share of the step's loads,
@@ -908,9 +913,11 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         // waits of a step: all but the newest load when that is the previous step's prefetch; in a tile's first step the
         // stores of the previous epilogue (or the cold start's stand-ins) and the one load of the bias values are newer
         // than the loads waited for as well
-        // (kGatherK: and the request for row_index entries that follows every step's loads)
+        // (kGatherK: and the request for row_index entries that follows every step's loads. In a tile's first step that
+        // request, like the prefetch of the same step, is older than the stores, and a cold start issues none behind the
+        // loads waited for: the count stays the one of the cold start, which only waits for more in a streamed tile)
         using WaitStep = std::integral_constant<int, waitcnt_imm((kPrefetch ? 1 : 0) + (kGatherK ? 1 : 0), true)>;
-        using WaitFirst = std::integral_constant<int, waitcnt_imm((int)kTileStores + (kPrefetch ? 1 : 0) + (BIAS ? 1 : 0) + (kGatherK ? 1 : 0), true)>;
+        using WaitFirst = std::integral_constant<int, waitcnt_imm((int)kTileStores + (kPrefetch ? 1 : 0) + (BIAS ? 1 : 0), true)>;
 
         // BIAS: the bias values of this wavefront's columns of the tile into its 128 bytes of LDS: one load by 32 lanes
         // (every wavefront issues it, so that all count the same loads), complete (loads and stores complete in issue
@@ -1007,8 +1014,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 // (kGatherK: the entries for the loads of steps 0 and 1 first, so that everything the waits below leave
                 // outstanding is what they count; a streamed tile has them from the last two steps of the tile before it)
                 if constexpr (kGatherK) {
-                    gk_ring[0] = gk_request_step(2u);
-                    gk_ring[1] = gk_request_step(3u);
+                    gk_ring[0] = gk_request_step(2u, false);
+                    gk_ring[1] = gk_request_step(3u, false);
                 }
                 issue_quiet(0, 0);
                 issue_quiet(1, BK);
