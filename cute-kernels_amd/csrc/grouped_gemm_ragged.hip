@@ -111,6 +111,9 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     // GATHER: the row_index entries of the 256 rows of a tile, for the tile of round r in half r % 2. Filled by
     // direct-to-LDS loads and read in assembly: the compiler never sees an access to it.
     __shared__ __attribute__((aligned(256))) uint32_t s_rows[GATHER ? 512 : 4];
+    // kGatherK: row_index entries on their way from one tile's last two steps (or a cold start) to the next tile's first two:
+    // per LDS stage and wavefront the 64 dwords of one direct-to-LDS load. Read in assembly only.
+    __shared__ __attribute__((aligned(256))) uint32_t s_gk[kGatherK ? 2 * NW * 64 : 4];
     // The group table, one LDS object: first tile of the group at position p of the tile sequence, exclusive prefix of the
     // varying dimension over the groups, and which group is at position p.
     __shared__ uint32_t s_table[2 * (FMA_MAX_GROUPS + 1) + FMA_MAX_GROUPS / 2];
@@ -464,7 +467,10 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     // The eight entries are one vector load per wavefront and step (lane l: entry l % 8; a position past the end of
     // row_index reads as 0), issued two steps ahead of the loads that use them, behind the step's own loads: a step's loads
     // for K step kt + 2 go out with the entries requested in step kt - 2, which the wait of step kt - 1 has seen arrive
-    // (loads complete in issue order). gk_ring[s]: the entries requested in the latest step that ran in LDS stage s.
+    // (loads complete in issue order). Inside a tile the entries travel in a register (gk_ring[s]: requested in the latest
+    // step that ran in LDS stage s). Across a tile boundary they travel through LDS (s_gk, a direct-to-LDS load read back
+    // in assembly): a register loaded in one tile and used in the next makes the compiler, which cannot count the
+    // epilogue's stores, wait for everything in flight at the top of the tile.
     const __amdgpu_buffer_rsrc_t gk_index = make_rsrc(reinterpret_cast<const uint16_t*>(args.row_index),
                                                       kGatherK ? uniform(s_prefix[E]) * 4u : 0u);
     const uint32_t gk_bytes = kGatherK ? args.a_rows * Ne * 2u : 0u;  // bytes of B (below 2^31)
@@ -472,7 +478,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     // the 16-byte chunk of a row this lane loads, swizzled as the packed loader does it for the row's place in the step;
     // instruction i: ^ 128 (i & 1)
     const uint32_t gk_chunk = ((lane & 31u) ^ (4u * gk_half) ^ (2u * (wave & 1u))) << 4;
-    uint32_t gk_ring[2] = {0u, 0u}, gk_v[4] = {0u, 0u, 0u, 0u};
+    uint32_t gk_v[4] = {0u, 0u, 0u, 0u};
     // this lane's entry of the eight that begin at position `first` of row_index. pinned: the request may not be issued
     // ahead of anything that precedes it in the program (the empty statement the lane's offset passes through is ordered
     // behind every load before it): the step waits count on the request being the newest load of its step
@@ -480,6 +486,15 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         uint32_t mine = (lane & 7u) * 4u;
         if (pinned) asm volatile("" : "+v"(mine));
         return __builtin_amdgcn_raw_buffer_load_b32(gk_index, mine, first * 4u, 0);
+    };
+    // the same request into this wavefront's dwords of LDS stage `slot` of s_gk, and the entry read back from there
+    auto gk_request_lds = [&](uint32_t first, int slot, bool pinned) __attribute__((always_inline)) {
+        uint32_t mine = (lane & 7u) * 4u;
+        if (pinned) asm volatile("" : "+v"(mine));
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(gk_index, (lds_void*)(s_gk + (slot * NW + wave) * 64), 4, mine, first * 4u, 0, 0);
+    };
+    auto gk_from_lds = [&](int slot) __attribute__((always_inline)) -> uint32_t {
+        return lds_read1_quiet(lds_address(reinterpret_cast<const uint8_t*>(s_gk)) + (((uint32_t)slot * NW + wave) * 64u + lane) * 4u);
     };
     // per-lane offsets of the four loads of the K step at k0 of a group with `limit` reduction rows, from the entries n
     // (lane l holds entry l % 8): every lane forms the byte offset of its entry's row, then picks, per instruction, the
@@ -591,8 +606,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     auto issue_b = [&](int stage, uint32_t k0, auto i0_c, auto i1_c) __attribute__((always_inline)) {
         constexpr int I0 = decltype(i0_c)::value, I1 = decltype(i1_c)::value;
         if constexpr (kGatherK) {
-            // the offsets of all four loads are formed with the first of them, from the entries requested two steps ago
-            if constexpr (I0 == 0) gk_offsets(k0, lt_b.kdim, gk_ring[stage], gk_v);
+            // (gk_v: the offsets of the step's four loads, formed by the caller from the entries requested two steps ago)
             const __amdgpu_buffer_rsrc_t r = make_rsrc(lt_b.base, gk_bytes - lt_b.col_bytes);
             uint8_t* tile = stage ? s_b1 : s_b0;
 #pragma unroll
@@ -657,13 +671,13 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         const uint32_t KT = (Ke + BK - 1) / BK;
         const uint32_t KT2 = (KT + 1u) & ~1u;  // steps of the K loop: an odd count gets a step of zeros
         const bool thin = is_thin(cur);
-        // kGatherK: requests the row_index entries of this wavefront for K step `abs_step` of the load stream: a step of
-        // this tile, or, past its end, of the next (vb_cur, vb_nxt: where the two groups' entries begin)
-        auto gk_request_step = [&](uint32_t abs_step, bool pinned) __attribute__((always_inline)) -> uint32_t {
+        // kGatherK: where in row_index the entries of this wavefront for K step `abs_step` of the load stream begin: a step
+        // of this tile, or, past its end, of the next (vb_cur, vb_nxt: where the two groups' entries begin)
+        auto gk_first = [&](uint32_t abs_step) __attribute__((always_inline)) -> uint32_t {
             const bool of_next = abs_step >= KT2;
-            return gk_request((of_next ? vb_nxt + (abs_step - KT2) * (uint32_t)BK : vb_cur + abs_step * (uint32_t)BK) + wave * 8u,
-                              pinned);
+            return (of_next ? vb_nxt + (abs_step - KT2) * (uint32_t)BK : vb_cur + abs_step * (uint32_t)BK) + wave * 8u;
         };
+        uint32_t gk_ring[2] = {0u, 0u};
         // the next tile's first two K steps ride on this tile's last two load slots
         const bool stream_next = streams(cur) && streams(nxt);
         if (stream_next) {
@@ -772,6 +786,25 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                     issue_a(stage, k0, i0_c, i1_c);
                 }
             };
+            // kGatherK: the entries for this step's loads were requested two steps ago: by a step of this tile into a register,
+            // or, for a tile's first two steps (SRC == 2 in a full tile), by the tile before or the cold start into LDS; the
+            // versions for tiles with few rows do not know at compile time which of their steps are the last two and use LDS
+            // throughout
+            auto gk_step_offsets = [&](uint32_t k0) __attribute__((always_inline)) {
+                if constexpr (kGatherK) {
+                    constexpr bool kFromLds = FA != RB || SRC == 2;
+                    gk_offsets(k0, lt_b.kdim, kFromLds ? gk_from_lds(stage) : gk_ring[stage], gk_v);
+                }
+            };
+            // ... and the entries for the loads of step kt + 2 (K step kt + 4 of the stream) are requested as the step's last
+            // load: into LDS by a full tile's last two steps (SRC == 1)
+            auto gk_step_request = [&]() __attribute__((always_inline)) {
+                if constexpr (kGatherK) {
+                    constexpr bool kToLds = FA != RB || SRC == 1;
+                    if constexpr (kToLds) gk_request_lds(gk_first(kt + 4u), stage, true);
+                    else gk_ring[stage] = gk_request(gk_first(kt + 4u), true);
+                }
+            };
             // what the loads issued in this step fetch: the K offset (returned) and, decided here (SRC == 2), whether the
             // loaders aim at the current tile's operands or the next one's
             auto aim_loads = [&]() __attribute__((always_inline)) -> uint32_t {
@@ -833,6 +866,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 spread_mfma_vmem<0, AB * CB, 3>();
                 __builtin_amdgcn_sched_barrier(0);
                 issue_a_part(k0, I3_{}, IN_{});
+                gk_step_offsets(k0);
                 issue_b(stage, k0, I0_{}, I2_{});
                 mma(fa_c, 2, 2, false, stage, 1);
                 spread_mfma_vmem<0, AB * CB, 3>();
@@ -841,8 +875,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 issue_b(stage, k0, I2_{}, IN_{});
                 if constexpr (kPrefetch) asm volatile("" : "+v"(pf_voff));
                 issue_prefetch(kt + kPfDist);
-                // the entries for the loads of step kt + 2 (K step kt + 4 of the stream): the step's last load
-                if constexpr (kGatherK) gk_ring[stage] = gk_request_step(kt + 4u, true);
+                gk_step_request();
                 mma(fa_c, 3, 3, true, stage ^ 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x100, kReadsA, 0);
 #pragma unroll
@@ -883,12 +916,13 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 load_a(fa_c, stage ^ 1, 0, 0, 0);
                 const uint32_t k0 = aim_loads();
                 issue_a_part(k0, I0_{}, IN_{});
+                gk_step_offsets(k0);
                 issue_b(stage, k0, I0_{}, IN_{});
                 // the prefetch goes out behind this step's loads (the empty statement orders it: the wait of the next step
                 // counts on it being the newest load)
                 if constexpr (kPrefetch) asm volatile("" : "+v"(pf_voff));
                 issue_prefetch(kt + kPfDist);
-                if constexpr (kGatherK) gk_ring[stage] = gk_request_step(kt + 4u, true);
+                gk_step_request();
                 mma(fa_c, PP - 1, 1, true, stage ^ 1, 0);
                 if constexpr (FA > 0) {
                     // the A reads; per column block its matrix instructions, each followed by its share of the step's loads,
@@ -1014,8 +1048,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 // (kGatherK: the entries for the loads of steps 0 and 1 first, so that everything the waits below leave
                 // outstanding is what they count; a streamed tile has them from the last two steps of the tile before it)
                 if constexpr (kGatherK) {
-                    gk_ring[0] = gk_request_step(2u, false);
-                    gk_ring[1] = gk_request_step(3u, false);
+                    gk_request_lds(gk_first(2u), 0, false);
+                    gk_request_lds(gk_first(3u), 1, false);
                 }
                 issue_quiet(0, 0);
                 issue_quiet(1, BK);

@@ -273,17 +273,13 @@ class MoE(nn.Module):
     def _gathers_inside_gemm(self, hidden_states: torch.Tensor) -> bool:
         """Whether the first projection (forward and weight gradient) gathers its rows itself instead of reading a grouped
         copy of the tokens. gather_in_gemm None: when the projection is narrow enough for the saved row-movement pass to
-        outweigh the slower operand fetch of scattered rows (measured: 1 to 5 % of the forward product and 0.4 to 4 % of the
-        weight-gradient product, against one pass that reads T and writes T * top_k rows) and, if a backward follows, the
-        experts get 1024 rows or more on average (with some 500 rows per expert the gathered weight gradient, whose tiles
-        then reduce over 8 steps only, loses more than the pass costs); True / False force it."""
+        outweigh the slower operand fetch of scattered rows (measured: 1 to 5 % of the forward product and -2 to +4 % of the
+        weight-gradient product, against one pass that reads T and writes T * top_k rows); True / False force it."""
         if self.gather_in_gemm is False or not can_gather_inside_gemm(hidden_states, self.c_fc.weight, self.c_fc.bias):
             return False
         if self.gather_in_gemm:
             return True
-        if self.c_fc.out_features > 6144:
-            return False
-        return not torch.is_grad_enabled() or hidden_states.size(0) * self.top_k >= 1024 * self.num_experts
+        return self.c_fc.out_features <= 6144
 
     def _get_topk(self, x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
         if self.top_k == 1:
