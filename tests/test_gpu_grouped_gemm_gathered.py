@@ -142,6 +142,8 @@ WGRAD_CASES = [
     ([300, 5000, 16, 16, 16, 2000], 997, 264, 1088, 6),  # N and K with partial tiles
     ([0, 0, 5], 9, 256, 256, 1),
     ([0, 0, 0], 9, 256, 256, 1),
+    ([(37 * e) % 211 for e in range(300)], 1234, 264, 520, 5),  # many short groups: every tile starts cold; partial tiles both ways
+    ([193 + (e % 3) * 64 for e in range(40)], 4000, 512, 256, 2),  # 4 or 5 K steps: streamed tiles of the shortest kind
 ]
 
 
