@@ -566,7 +566,13 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         const bool inside = kstep < pf_steps;
         const uint32_t rows = k0 >= pf_kdim ? 0u : (pf_kdim - k0 < (uint32_t)BK ? pf_kdim - k0 : (uint32_t)BK);
         const uint16_t* base = pf_t ? pf_base + (uint64_t)k0 * (pf_ldb / 2u) : pf_base;
-        const uint32_t bytes = !inside ? 0u : (pf_t ? (rows ? rows * pf_ldb - pf_col_bytes : 0u) : pf_bytes);
+        uint32_t bytes = !inside ? 0u : (pf_t ? (rows ? rows * pf_ldb - pf_col_bytes : 0u) : pf_bytes);
+        if constexpr (GATHER) {
+            // (the same in every lane, which the compiler does not see in these kernels: without this it wraps the load
+            // in a loop over the distinct descriptors it fears)
+            base = reinterpret_cast<const uint16_t*>(uniform((uint64_t)(uintptr_t)base));
+            bytes = uniform(bytes);
+        }
         __builtin_amdgcn_raw_ptr_buffer_load_lds(make_rsrc(base, bytes), (lds_void*)s_pf, 4, pf_voff, pf_t ? 0u : k0 * 2u, 0, 0);
     };
 
@@ -597,7 +603,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         } else {
             g_offsets(half, k0, v);
         }
-        const __amdgpu_buffer_rsrc_t r = make_rsrc(args.A, bytes);
+        const __amdgpu_buffer_rsrc_t r = make_rsrc(args.A, uniform(bytes));
         uint8_t* tile = stage ? s_a1 : s_a0;
 #pragma unroll
         for (int i = I0; i < I1; ++i)
