@@ -15,7 +15,13 @@ for every instantiation of ragged_gemm_kernel, that the instruction stream has t
  * the cold start issues sixteen operand loads, as many stand-in stores as an epilogue issues stores, and waits for all but
    the eight loads of the second step and the stores;
  * the three-stage loop of groups of at most 64 rows issues five loads per step and waits for all but five;
- * no instantiation touches scratch memory.
+ * no instantiation touches scratch memory, and none contains a loop over the distinct values of an operand that the
+   hardware wants in scalar registers (what the compiler generates around a vector-memory instruction whose descriptor or
+   scalar offset it cannot prove to be the same in every lane: each costs a dozen instructions and a branch per use).
+
+The kernels that gather the rows of their first operand (forward form) read a row table between a step's barrier and its
+loads, which spreads a step over several basic blocks in ways that differ from version to version of the loop: for them
+only the loop bodies of two steps, the scratch memory and the loops over scalar operands are checked.
 """
 
 import os
@@ -39,13 +45,15 @@ def compile_to_assembly(path: str) -> None:
 
 
 def tokens(lines):
-    """The vector-memory instructions, waits and barriers of a kernel, one string per basic block."""
-    blocks, cur = [], []
-    for line in lines:
+    """The vector-memory instructions, waits and barriers of a kernel in program order, and the number of loops over the
+    distinct values of a scalar operand (readfirstlane, compare, s_and_saveexec, the instruction, s_xor exec, branch)."""
+    cur, waterfalls = [], 0
+    for k, line in enumerate(lines):
         s = line.strip()
+        if s.startswith("s_cbranch_execnz") and any("s_xor_b64 exec, exec" in x for x in lines[max(0, k - 3):k]):
+            waterfalls += 1
         if re.match(r"^\.LBB\d+_\d+:", line):
-            blocks.append("".join(cur))
-            cur = []
+            cur.append(" ")
         elif s.startswith("s_barrier"):
             cur.append("|")
         elif s.startswith("s_waitcnt") and "vmcnt" in s:
@@ -60,8 +68,7 @@ def tokens(lines):
             cur.append("s")
         elif s.startswith("scratch_"):
             cur.append("X")
-    blocks.append("".join(cur))
-    return [b for b in blocks if b]
+    return [b for b in "".join(cur).split(" ") if b], waterfalls
 
 
 def audit(asm_path: str) -> int:
@@ -77,24 +84,27 @@ def audit(asm_path: str) -> int:
         el, a_kc, b_kc, epi, vary_k, bias, gather = m.group(1), *[int(x) for x in m.groups()[1:]]
         body = lines[a:b]
         end = next((k for k, line in enumerate(body) if "s_endpgm" in line), len(body))
-        blocks = tokens(body[:end])
+        blocks, waterfalls = tokens(body[:end])
         prefetch = 1 if a_kc == b_kc else 0
         request = 1 if (vary_k and gather) else 0
         stores = EPI_STORES[epi]
         wait_step, wait_first = prefetch + request, stores + prefetch + bias
         tag = f"{el} A_KC={a_kc} B_KC={b_kc} epilogue={epi} reduction_varies={vary_k} bias={bias} gather={gather}"
         found = {"step": 0, "first": 0, "body": 0, "cold": 0, "thin": 0}
+        gathers_rows = bool(gather and not vary_k)
 
         def fail(what, block):
             nonlocal problems
             problems += 1
             print(f"PROBLEM {tag}: {what}: {block[:120]}")
 
+        if waterfalls:
+            fail(f"{waterfalls} loops over the distinct values of a scalar operand", "")
         for blk in blocks:
             if "X" in blk:
                 fail("scratch access", blk)
             # waits in front of a barrier that the operand loads of a K step follow
-            for w, loads in re.findall(r"w(\d+),\|(O+)", blk):
+            for w, loads in ([] if gathers_rows else re.findall(r"w(\d+),\|(O+)", blk)):
                 n, count = int(w), len(loads)
                 if count == 8:
                     if n == wait_step:
@@ -119,16 +129,20 @@ def audit(asm_path: str) -> int:
                     fail(f"{issued} instructions between the barriers of two steps, expected {8 + wait_step}", blk)
             # the cold start: sixteen operand loads (the gathered kinds mix loads of row_index entries in), the stand-in
             # stores, the wait
-            cold = re.search(r"((?:[OLp]|w\d+,)*O)(s+)w(\d+),\|", blk)
+            cold = None if gathers_rows else re.search(r"((?:[OLp]|w\d+,)*O)(s+)w(\d+),\|", blk)
             if cold and cold.group(1).count("O") >= 16:
                 found["cold"] += 1
                 if cold.group(1).count("O") != 16 or len(cold.group(2)) != stores or int(cold.group(3)) != 8 + stores:
                     fail(f"cold start: {cold.group(1).count('O')} loads, {len(cold.group(2))} stores, wait {cold.group(3)}; "
                          f"expected 16, {stores}, {8 + stores}", blk)
-        if found["step"] == 0 or found["first"] == 0 or found["cold"] != 1:
-            fail(f"expected shapes not found ({found})", "")
-        if a_kc and found["thin"] == 0:
-            fail("no three-stage loop found", "")
+        if gathers_rows:
+            if found["body"] == 0:
+                fail(f"expected shapes not found ({found})", "")
+        else:
+            if found["step"] == 0 or found["first"] == 0 or found["cold"] != 1:
+                fail(f"expected shapes not found ({found})", "")
+            if a_kc and found["thin"] == 0:
+                fail("no three-stage loop found", "")
         print(f"ok  {tag}: steps {found['step']}, first steps {found['first']}, two-step bodies {found['body']}, "
               f"three-stage steps {found['thin']}")
     return problems
