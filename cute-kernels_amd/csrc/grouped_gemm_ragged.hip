@@ -414,13 +414,13 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     const uint32_t g_ldb = dim_k * 2u;
     const uint32_t g_row = logical_row(wave * 8u + (lane >> 3));
     const uint32_t g_chunk = (lane & 7u) ^ (g_row & 7u);
-    // n / divisor for n < 2^31: the high word of n * ceil(2^32 / divisor) is the quotient or one more
-    const uint32_t g_magic = (GATHER_ANY && args.divisor > 1u) ? (uint32_t)((0x100000000ull + args.divisor - 1u) / args.divisor) : 0u;
+    // The row an entry n of row_index names, n / divisor, or a number no row has if the entry is negative: for n < 2^31 the
+    // high word of n * floor((2^32 - 1) / divisor) is the quotient or one less (any divisor from 1 on, no branch).
+    const uint32_t g_magic = GATHER_ANY ? 0xffffffffu / args.divisor : 0u;
     auto g_source_row = [&](uint32_t n) -> uint32_t {
-        if (args.divisor == 1u) return n;
         uint32_t q = __umulhi(n, g_magic);
-        if (q * args.divisor > n) --q;
-        return q;
+        q += (n - q * args.divisor >= args.divisor) ? 1u : 0u;
+        return q | (n & 0x80000000u);
     };
     uint32_t g_bytes_nxt = 0;  // bytes of A the loads for the next tile may read: all of it, or nothing when nothing follows
     // per-lane offsets of the four loads of a K step of the tile in table half `half` (the step's k0 goes into the
@@ -432,7 +432,7 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
         for (int i = 0; i < 4; ++i) {
             // an entry that names no row of A (negative, or past the last row) reads as a row of zeros
             const uint32_t src = g_source_row(n[i]);
-            v[i] = (n[i] < 0x80000000u && src < args.a_rows) ? src * g_ldb + g_chunk * 16u : kOutOfRange;
+            v[i] = src < args.a_rows ? src * g_ldb + g_chunk * 16u : kOutOfRange;
         }
     };
     // last, partial K step: chunks past the end of K are pushed out of range, which zero-fills them
@@ -499,14 +499,10 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
     // per-lane offsets of the four loads of the K step at k0 of a group with `limit` reduction rows, from the entries n
     // (lane l holds entry l % 8): every lane forms the byte offset of its entry's row, then picks, per instruction, the
     // offset of one of the instruction's two rows from the lane that holds it, and adds its chunk.
-    // n / divisor for n < 2^31: the high word of n * floor((2^32 - 1) / divisor) is the quotient or one less
-    const uint32_t gk_magic = kGatherK ? 0xffffffffu / args.divisor : 0u;
     auto gk_offsets = [&](uint32_t k0, uint32_t limit, uint32_t n, uint32_t (&v)[4]) {
-        uint32_t q = __umulhi(n, gk_magic);
-        q += (n - q * args.divisor >= args.divisor) ? 1u : 0u;
         // an entry that names no row of B (negative, or past the last row) reads as a row of zeros, and so does a
         // reduction row past the group's end
-        q |= n & 0x80000000u;
+        uint32_t q = g_source_row(n);
         q = k0 + wave * 8u + (lane & 7u) < limit ? q : 0xffffffffu;
         const uint32_t off = q < args.a_rows ? q * (Ne * 2u) : kOutOfRange;
 #pragma unroll
@@ -534,7 +530,8 @@ __global__ __launch_bounds__(NT) void ragged_gemm_kernel(const Args args) {
                 const uint32_t n = lds_read1_quiet(lds_address(reinterpret_cast<const uint8_t*>(s_rows)) + (round & 1u) * 1024u +
                                                    (lane < 16u ? 4u * i + t.pf_c : 0u) * 4u);
                 pf_base = args.A; pf_bytes = g_full;
-                pf_voff = (lane < 16u && n < 0x80000000u && g_source_row(n) < args.a_rows) ? g_source_row(n) * g_ldb : kOutOfRange;
+                const uint32_t src = lane < 16u ? g_source_row(n) : 0xffffffffu;
+                pf_voff = src < args.a_rows ? src * g_ldb : kOutOfRange;
             } else if constexpr (A_KC) {
                 pf_base = fa_cur.base0; pf_bytes = fa_cur.extent;
                 pf_voff = lane < 16u ? (4u * i + t.pf_c) * (t.Ke * 2u) : kOutOfRange;
