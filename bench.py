@@ -38,7 +38,7 @@ WORKLOADS = {
 # (FETCH_SIZE 7.705e6 KiB, WRITE_SIZE 2.753e6 KiB per dispatch; other pairs of runs read 6.78e6 to 7.55e6 KiB fetched) scaled by what the same counters read for a 1 GiB
 # device copy (FETCH_SIZE 0.50, WRITE_SIZE 1.00 of the true bytes); profiles/grouped_gemm_mixtral_counters.txt holds
 # the runs. Measured for the mixtral workload only; a constant from those profile runs, not measured by this script.
-MEASURED_TRAFFIC_BYTES = {"mixtral": (2 * 7.814e6 + 2.753e6) * 1024}
+MEASURED_TRAFFIC_BYTES = {"mixtral": (2 * 7.509e6 + 2.753e6) * 1024}
 TRAFFIC_SOURCE = "profiles/grouped_gemm_mixtral_counters.txt (two rocprofv3 --pmc runs of this script; not measured in this run)"
 
 
