@@ -26,6 +26,10 @@
 //    that need the element-wise path) start cold: the tile before them lets its last two load slots fetch nothing and
 //    drains, and they issue their first loads themselves, followed by as many stores outside every buffer as an epilogue
 //    issues, so that the waits of the K loop are the same constants in both cases.
+//  * Two kinds of kernels read one operand through an index instead of a packed copy (GATHER): the forward product takes
+//    the rows of A as rows row_index[i] / divisor of the token matrix (a table of the tile's 256 entries in LDS, four
+//    per-lane offsets per K step), the weight gradient takes the reduction rows of B the same way (eight entries per
+//    wavefront and K step, requested two steps ahead). Both give the bits of the packed kernel on a gathered copy.
 #include "gemm_parts.h"
 
 namespace fmahip {
