@@ -62,6 +62,59 @@ class Experts(nn.Module):
             bias=self.bias,
         )
 
+    @staticmethod
+    def _routing_tensors(
+        sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor
+    ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """rows per expert (uint32), the routing order and its inverse (int32) from what the reference's callers hold:
+        the order of the (token, choice) slots sorted by expert and the inclusive offsets of the experts in it"""
+        perm = sorted_scattered_idxs.to(torch.int32).contiguous()
+        inverse = torch.empty_like(perm)
+        inverse[perm.long()] = torch.arange(perm.numel(), dtype=torch.int32, device=perm.device)
+        offsets = expert_offsets.to(torch.int32)
+        counts = torch.diff(offsets, prepend=offsets.new_zeros(1))
+        return counts.contiguous().view(torch.uint32), perm, inverse
+
+    def up_projection_triton_forward(
+        self,
+        input: torch.Tensor,
+        num_experts_per_token: int | None = None,
+        sorted_expert_idxs: torch.Tensor | None = None,
+        sorted_scattered_idxs: torch.Tensor | None = None,
+        expert_offsets: torch.Tensor | None = None,
+    ) -> torch.Tensor:
+        """The reference's entry point of this name (fma/modules/moe/__init__.py:40-62: scattered_experts with the tokens
+        as input and grouped rows as output), on the HIP kernels: row i of the result is input[sorted_scattered_idxs[i] //
+        num_experts_per_token] @ weight[expert of row i]^T, the rows gathered inside the GEMM where its limits allow."""
+        assert self.bias is None
+        expert_frequency, perm, inverse = self._routing_tensors(sorted_scattered_idxs, expert_offsets)
+        if can_gather_inside_gemm(input, self.weight, None):
+            return gathered_up_projection_experts(
+                input, self.weight, None, perm, inverse, expert_frequency, self.N_array, self.K_array,
+                num_experts_per_token, False,
+            )  # fmt: skip
+        return self.cuda_forward(gather_rows(input, perm, inverse, num_experts_per_token), expert_frequency)
+
+    def down_projection_triton_forward(
+        self,
+        input: torch.Tensor,
+        num_experts_per_token: int | None = None,
+        sorted_expert_idxs: torch.Tensor | None = None,
+        sorted_scattered_idxs: torch.Tensor | None = None,
+        expert_offsets: torch.Tensor | None = None,
+        gates: torch.Tensor | None = None,
+    ) -> torch.Tensor:
+        """The reference's entry point of this name (fma/modules/moe/__init__.py:64-87: scattered_experts with grouped rows
+        as input), on the HIP kernels: the projection of the grouped rows, returned per (token, choice) slot, or, with
+        `gates` [T, k], as the gate-weighted sum over every token's k rows."""
+        assert self.bias is None
+        expert_frequency, perm, inverse = self._routing_tensors(sorted_scattered_idxs, expert_offsets)
+        output = self.cuda_forward(input, expert_frequency)
+        if gates is None:
+            # out[slot] = output[row of slot]: the row movement of gather_rows with the two index arrays exchanged
+            return gather_rows(output, inverse, perm, 1)
+        return combine(output, gates, inverse)
+
     def extra_repr(self) -> str:
         return f"num_experts={self.num_experts}, in_features={self.in_features}, out_features={self.out_features}"
 

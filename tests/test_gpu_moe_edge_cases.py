@@ -179,3 +179,51 @@ def test_training_step_is_bit_reproducible(add_bias):
         assert torch.equal(first[name], second[name]), name
     counts = torch.bincount(moe._compute_routing_weights(x0)[2].flatten().long(), minlength=E)
     assert int(counts.max()) > 4 * max(int(counts.min()), 1), "the routing of this test is meant to be skewed"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_the_reference_s_two_projection_entry_points(dtype):
+    # Experts.up_projection_triton_forward / down_projection_triton_forward (fma/modules/moe/__init__.py:40-87), called as
+    # the reference's triton branch calls them (:247-265) with torch's own sort as routing order: the layer's result and
+    # gradients (bit for bit in bf16, where both run the same kernels; fp32 goes through the grouped copy)
+    torch.manual_seed(11)
+    E, k, H, I, T = 8, 2, 256, 384, 500
+    moe = MoE(E, k, H, I, swiglu_packed, True, False, 0.05).to(dtype).to(DEV)
+    x = torch.randn(T, H, device=DEV).to(dtype)
+    dy = torch.randn(T, H, device=DEV).to(dtype)
+    selected = torch.randint(0, E - 1, (T, k), device=DEV)  # the last expert gets no rows
+    weights = torch.softmax(torch.randn(T, k, device=DEV), dim=-1).to(dtype)
+
+    def run(through_entry_points):
+        moe.zero_grad(set_to_none=True)
+        xi, wi = x.clone().requires_grad_(), weights.clone().requires_grad_()
+        if through_entry_points:
+            sorted_expert_idxs, sorted_scattered_idxs = selected.flatten().sort(stable=True)
+            expert_offsets = torch.bincount(sorted_expert_idxs, minlength=E).cumsum(-1)
+            routing = dict(sorted_expert_idxs=sorted_expert_idxs, sorted_scattered_idxs=sorted_scattered_idxs,
+                           expert_offsets=expert_offsets)
+            h = moe.c_fc.up_projection_triton_forward(input=xi, num_experts_per_token=k, **routing)
+            y = moe.c_proj.down_projection_triton_forward(input=moe.act(h), num_experts_per_token=1, gates=wi, **routing)
+        else:
+            y = moe._compute_experts(xi, wi, selected, KernelBackend.cuda)
+        y.backward(dy)
+        return [y.detach(), xi.grad, wi.grad, moe.c_fc.weight.grad.clone(), moe.c_proj.weight.grad.clone()]
+
+    for name, a, b in zip(("y", "dx", "dgates", "dW1", "dW2"), run(True), run(False)):
+        if dtype == torch.bfloat16:
+            _assert_same(a, b, name)
+        else:
+            assert float((a - b).abs().max()) <= 1e-5 * max(1.0, float(b.abs().max())), name
+    # without gates the second entry point returns the rows per (token, choice) slot
+    sorted_expert_idxs, sorted_scattered_idxs = selected.flatten().sort(stable=True)
+    expert_offsets = torch.bincount(sorted_expert_idxs, minlength=E).cumsum(-1)
+    grouped = torch.randn(T * k, I, device=DEV).to(dtype)
+    per_slot = moe.c_proj.down_projection_triton_forward(
+        input=grouped, num_experts_per_token=1, sorted_expert_idxs=sorted_expert_idxs,
+        sorted_scattered_idxs=sorted_scattered_idxs, expert_offsets=expert_offsets,
+    )
+    counts = torch.bincount(sorted_expert_idxs, minlength=E).to(torch.int32).view(torch.uint32)
+    rows = moe.c_proj.cuda_forward(grouped, counts)
+    expect = torch.empty_like(rows)
+    expect[sorted_scattered_idxs] = rows
+    _assert_same(per_slot.detach(), expect.detach(), "rows per slot")
